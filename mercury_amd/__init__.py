@@ -1,0 +1,3 @@
+"""mercury_amd: a single-GPU inference engine for MI355X (gfx950), hand-written HIP kernels."""
+
+__version__ = "0.1.0"

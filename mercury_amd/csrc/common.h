@@ -1,0 +1,115 @@
+// Shared declarations for the gfx950 kernel library: element types, conversions, reductions
+// and the host-side error channel.  Every exported function returns 0 on success and a
+// non-zero code after recording a message that mk_last_error() returns.
+#pragma once
+
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include <stdio.h>
+
+#define MK_WAVE 64
+
+enum MkDtype { MK_F32 = 0, MK_BF16 = 1 };
+
+typedef uint16_t bf16_t;
+
+// ---------------------------------------------------------------------------------- errors
+
+void mk_set_error(const char* fmt, ...);
+
+#define MK_REQUIRE(cond, ...)      \
+  do {                             \
+    if (!(cond)) {                 \
+      mk_set_error(__VA_ARGS__);   \
+      return 1;                    \
+    }                              \
+  } while (0)
+
+#define MK_LAUNCH_CHECK(name)                                             \
+  do {                                                                    \
+    hipError_t e_ = hipGetLastError();                                    \
+    if (e_ != hipSuccess) {                                               \
+      mk_set_error("%s: launch failed: %s", name, hipGetErrorString(e_)); \
+      return 2;                                                           \
+    }                                                                     \
+  } while (0)
+
+// ------------------------------------------------------------------------------ conversions
+
+__device__ __forceinline__ float bf16_to_f32(bf16_t x) {
+  return __uint_as_float(((uint32_t)x) << 16);
+}
+
+// Round to nearest, ties to even; NaN stays NaN.
+__device__ __forceinline__ bf16_t f32_to_bf16(float f) {
+  uint32_t u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (bf16_t)(u >> 16);
+}
+
+template <typename T>
+struct Elem;
+
+template <>
+struct Elem<float> {
+  static __device__ __forceinline__ float load(const float* p) { return *p; }
+  static __device__ __forceinline__ void store(float* p, float v) { *p = v; }
+  static __device__ __forceinline__ float round(float v) { return v; }
+};
+
+template <>
+struct Elem<bf16_t> {
+  static __device__ __forceinline__ float load(const bf16_t* p) { return bf16_to_f32(*p); }
+  static __device__ __forceinline__ void store(bf16_t* p, float v) { *p = f32_to_bf16(v); }
+  static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
+};
+
+// ------------------------------------------------------------------------------- reductions
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int m = MK_WAVE / 2; m > 0; m >>= 1) v += __shfl_xor(v, m, MK_WAVE);
+  return v;
+}
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int m = MK_WAVE / 2; m > 0; m >>= 1) v = fmaxf(v, __shfl_xor(v, m, MK_WAVE));
+  return v;
+}
+
+// Sum over a block of up to 1024 threads; `scratch` holds at least 16 floats.  Every thread
+// gets the result.  The order of additions is fixed by the thread layout alone.
+__device__ __forceinline__ float block_sum(float v, float* scratch) {
+  const int lane = threadIdx.x & (MK_WAVE - 1);
+  const int wave = threadIdx.x / MK_WAVE;
+  const int waves = (blockDim.x + MK_WAVE - 1) / MK_WAVE;
+  v = wave_sum(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = 0.f;
+  for (int w = 0; w < waves; ++w) total += scratch[w];
+  return total;
+}
+
+__device__ __forceinline__ float block_max(float v, float* scratch) {
+  const int lane = threadIdx.x & (MK_WAVE - 1);
+  const int wave = threadIdx.x / MK_WAVE;
+  const int waves = (blockDim.x + MK_WAVE - 1) / MK_WAVE;
+  v = wave_max(v);
+  __syncthreads();
+  if (lane == 0) scratch[wave] = v;
+  __syncthreads();
+  float total = scratch[0];
+  for (int w = 1; w < waves; ++w) total = fmaxf(total, scratch[w]);
+  return total;
+}
+
+static inline int mk_is_pow2(int x) { return x > 0 && (x & (x - 1)) == 0; }
+static inline int mk_log2(int x) {
+  int s = 0;
+  while ((1 << s) < x) ++s;
+  return s;
+}

@@ -1,0 +1,263 @@
+// Row-wise and element-wise kernels: embedding gather, RMSNorm (with the residual sum folded
+// in), SiLU-gating, rotary position encoding fused with the write into the paged cache.
+// Arithmetic is float32 throughout; the element type only decides storage.
+#include "common.h"
+#include "mercury_kernels.h"
+
+#include <stdarg.h>
+#include <string>
+
+// ---------------------------------------------------------------------------------- errors
+
+static thread_local std::string g_last_error;
+
+void mk_set_error(const char* fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_last_error = buf;
+}
+
+extern "C" const char* mk_last_error() { return g_last_error.c_str(); }
+
+extern "C" int mk_abi_version() { return MK_ABI_VERSION; }
+
+// ------------------------------------------------------------------------------- embedding
+
+template <typename T>
+__global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                             float* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  // Ids are validated on the host; the clamp only keeps a bad id from reading outside.
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* row = table + (size_t)id * hidden;
+  float* dst = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = Elem<T>::load(row + i);
+}
+
+extern "C" int mk_embed(const int* ids, const void* table, int dtype, float* out, int tokens,
+                        int hidden, int vocab, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes T=%d H=%d V=%d", tokens,
+             hidden, vocab);
+  if (tokens == 0) return 0;
+  const int threads = hidden >= 256 ? 256 : 64;
+  if (dtype == MK_F32)
+    embed_kernel<float><<<tokens, threads, 0, stream>>>(ids, (const float*)table, out, hidden,
+                                                        vocab);
+  else if (dtype == MK_BF16)
+    embed_kernel<bf16_t><<<tokens, threads, 0, stream>>>(ids, (const bf16_t*)table, out, hidden,
+                                                         vocab);
+  else
+    MK_REQUIRE(false, "embed: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// --------------------------------------------------------------------------------- RMSNorm
+
+// One block per output row.  h is the float32 residual stream.  When `partials` is given,
+// the P partial sums of the preceding projection are first added into h (in the order
+// 0..P-1) and written back, so the residual sum and the norm are one pass.
+// out = round(round(x * rsqrt(mean(x^2) + eps)) * w): the normalised value is rounded to the
+// storage type before the weight multiplies it, as the unfused reference path does
+// (reference: mercury/model/qwen2.py:27-31).
+template <typename TO, typename TW>
+__global__ void rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ partials,
+                               int num_partials, size_t partial_stride,
+                               const TW* __restrict__ weight, float eps,
+                               const int* __restrict__ rows, TO* __restrict__ out, int hidden) {
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int in_row = rows ? rows[out_row] : out_row;
+  float* x = h + (size_t)in_row * hidden;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    float v = x[i];
+    if (num_partials > 0) {
+      const float* p = partials + (size_t)in_row * hidden + i;
+      for (int k = 0; k < num_partials; ++k) v += p[(size_t)k * partial_stride];
+      x[i] = v;
+    }
+    sq += v * v;
+  }
+  const float total = block_sum(sq, scratch);
+  const float rstd = rsqrtf(total / (float)hidden + eps);
+  TO* dst = out + (size_t)out_row * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float n = Elem<TO>::round(x[i] * rstd);
+    Elem<TO>::store(dst + i, n * Elem<TW>::load(weight + i));
+  }
+}
+
+template <typename TO>
+static int launch_rmsnorm(float* h, const float* partials, int num_partials,
+                          size_t partial_stride, const void* weight, int weight_dtype, float eps,
+                          const int* rows, TO* out, int out_rows, int hidden,
+                          hipStream_t stream) {
+  const int threads = hidden >= 1024 ? 256 : (hidden >= 256 ? 128 : 64);
+  if (weight_dtype == MK_F32)
+    rmsnorm_kernel<TO, float><<<out_rows, threads, 0, stream>>>(
+        h, partials, num_partials, partial_stride, (const float*)weight, eps, rows, out, hidden);
+  else
+    rmsnorm_kernel<TO, bf16_t><<<out_rows, threads, 0, stream>>>(
+        h, partials, num_partials, partial_stride, (const bf16_t*)weight, eps, rows, out, hidden);
+  return 0;
+}
+
+extern "C" int mk_rmsnorm(float* h, const float* partials, int num_partials,
+                          long long partial_stride, const void* weight, int weight_dtype,
+                          float eps, const int* rows, void* out, int out_dtype, int out_rows,
+                          int hidden, hipStream_t stream) {
+  MK_REQUIRE(out_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", out_rows, hidden);
+  MK_REQUIRE(num_partials >= 0 && (num_partials == 0 || partials != nullptr),
+             "rmsnorm: %d partial sums but no buffer", num_partials);
+  MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "rmsnorm: weight dtype %d",
+             weight_dtype);
+  if (out_rows == 0) return 0;
+  if (out_dtype == MK_F32)
+    launch_rmsnorm<float>(h, partials, num_partials, (size_t)partial_stride, weight,
+                          weight_dtype, eps, rows, (float*)out, out_rows, hidden, stream);
+  else if (out_dtype == MK_BF16)
+    launch_rmsnorm<bf16_t>(h, partials, num_partials, (size_t)partial_stride, weight,
+                           weight_dtype, eps, rows, (bf16_t*)out, out_rows, hidden, stream);
+  else
+    MK_REQUIRE(false, "rmsnorm: unknown out dtype %d", out_dtype);
+  MK_LAUNCH_CHECK("rmsnorm");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------ SiLU gating
+
+// gate_up is [T, 2*I]: columns [0, I) hold the gate, [I, 2I) the up projection.
+// out = round(round(silu(g)) * u) (reference: mercury/model/qwen2.py:42).
+template <typename T>
+__global__ void silu_mul_kernel(const T* __restrict__ gate_up, T* __restrict__ out,
+                                int inter, size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / inter;
+    const int i = (int)(idx - t * inter);
+    const T* row = gate_up + t * 2 * (size_t)inter;
+    const float g = Elem<T>::load(row + i);
+    const float u = Elem<T>::load(row + inter + i);
+    const float s = Elem<T>::round(g / (1.f + expf(-g)));
+    Elem<T>::store(out + idx, s * u);
+  }
+}
+
+extern "C" int mk_silu_mul(const void* gate_up, void* out, int dtype, int tokens, int inter,
+                           hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && inter > 0, "silu_mul: bad sizes T=%d I=%d", tokens, inter);
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * inter;
+  const int threads = 256;
+  size_t blocks = (total + threads - 1) / threads;
+  if (blocks > 65536) blocks = 65536;
+  if (dtype == MK_F32)
+    silu_mul_kernel<float><<<(int)blocks, threads, 0, stream>>>((const float*)gate_up,
+                                                               (float*)out, inter, total);
+  else if (dtype == MK_BF16)
+    silu_mul_kernel<bf16_t><<<(int)blocks, threads, 0, stream>>>((const bf16_t*)gate_up,
+                                                                (bf16_t*)out, inter, total);
+  else
+    MK_REQUIRE(false, "silu_mul: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("silu_mul");
+  return 0;
+}
+
+// ------------------------------------------------------- rotary encoding + paged cache write
+
+// qkv is [T, row_stride] with q heads first, then k heads, then v heads, each of width d.
+// The first `rot` dims of every q and k head are rotated in the half-split layout: dims j
+// and j + rot/2 form a pair turned by the angle of (position, j):
+//   y[j]         = x[j] * cos - x[j + rot/2] * sin
+//   y[j + rot/2] = x[j + rot/2] * cos + x[j] * sin
+// (reference: mercury/model/rope.py:6-17).  cos/sin are float32 tables [positions, rot/2].
+// q is rotated in place; rotated k and raw v go to the token's slot of the paged cache
+// [pages, n_kv, page_size, d], the page taken from the sequence's block table
+// (reference: mercury/runner.py:32-34, mercury/model/attention.py:35-45).
+template <typename T>
+__global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
+                                     const float* __restrict__ cos_table,
+                                     const float* __restrict__ sin_table,
+                                     const int* __restrict__ positions,
+                                     const int* __restrict__ token_seq,
+                                     const int* __restrict__ block_table, int table_stride,
+                                     T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                     int page_shift, int n_q, int n_kv, int d, int rot,
+                                     int write_kv) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = rot / 2;
+  const float* cs = cos_table + (size_t)pos * half;
+  const float* sn = sin_table + (size_t)pos * half;
+  T* row = qkv + (size_t)t * row_stride;
+
+  // q heads: pairwise, in place.
+  for (int idx = threadIdx.x; idx < n_q * half; idx += blockDim.x) {
+    const int head = idx / half, j = idx - head * half;
+    T* x = row + head * d;
+    const float a = Elem<T>::load(x + j), b = Elem<T>::load(x + j + half);
+    const float c = cs[j], s = sn[j];
+    Elem<T>::store(x + j, a * c - b * s);
+    Elem<T>::store(x + j + half, b * c + a * s);
+  }
+  if (!write_kv) return;
+
+  const int page_size = 1 << page_shift;
+  const int seq = token_seq[t];
+  const int page = block_table[(size_t)seq * table_stride + (pos >> page_shift)];
+  if (page < 0) return;  // the host never schedules a write into a page that was given back
+  const int off = pos & (page_size - 1);
+  const T* k_src = row + n_q * d;
+  const T* v_src = k_src + n_kv * d;
+  for (int idx = threadIdx.x; idx < n_kv * d; idx += blockDim.x) {
+    const int head = idx / d, j = idx - head * d;
+    const size_t dst = (((size_t)page * n_kv + head) * page_size + off) * d + j;
+    const T* x = k_src + head * d;
+    float y;
+    if (j < half) {
+      y = Elem<T>::load(x + j) * cs[j] - Elem<T>::load(x + j + half) * sn[j];
+    } else if (j < rot) {
+      y = Elem<T>::load(x + j) * cs[j - half] + Elem<T>::load(x + j - half) * sn[j - half];
+    } else {
+      y = Elem<T>::load(x + j);
+    }
+    Elem<T>::store(k_cache + dst, y);
+    v_cache[dst] = v_src[head * d + j];
+  }
+}
+
+extern "C" int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const float* cos_table,
+                                const float* sin_table, int table_positions,
+                                const int* positions, const int* token_seq,
+                                const int* block_table, int table_stride, void* k_cache,
+                                void* v_cache, int page_size, int n_q, int n_kv, int d, int rot,
+                                int write_kv, int tokens, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv >= 0 && d > 0, "rope: bad sizes");
+  MK_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "rope: rotary width %d not in [0, %d] / even",
+             rot, d);
+  MK_REQUIRE(mk_is_pow2(page_size), "rope: page size %d is not a power of two", page_size);
+  MK_REQUIRE(row_stride >= (n_q + (write_kv ? 2 * n_kv : 0)) * d,
+             "rope: row stride %d too small for %d+2*%d heads of %d", row_stride, n_q, n_kv, d);
+  MK_REQUIRE(rot == 0 || table_positions > 0, "rope: empty angle table");
+  if (tokens == 0) return 0;
+  const int threads = 128;
+  if (dtype == MK_F32)
+    rope_kv_write_kernel<float><<<tokens, threads, 0, stream>>>(
+        (float*)qkv, row_stride, cos_table, sin_table, positions, token_seq, block_table,
+        table_stride, (float*)k_cache, (float*)v_cache, mk_log2(page_size), n_q, n_kv, d, rot,
+        write_kv);
+  else if (dtype == MK_BF16)
+    rope_kv_write_kernel<bf16_t><<<tokens, threads, 0, stream>>>(
+        (bf16_t*)qkv, row_stride, cos_table, sin_table, positions, token_seq, block_table,
+        table_stride, (bf16_t*)k_cache, (bf16_t*)v_cache, mk_log2(page_size), n_q, n_kv, d, rot,
+        write_kv);
+  else
+    MK_REQUIRE(false, "rope: unknown dtype %d", dtype);
+  MK_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}

@@ -1,0 +1,63 @@
+// C interface of the gfx950 kernel library.  Pointers are device pointers unless a comment
+// says otherwise; `stream` is a hipStream_t.  Functions validate their arguments on the host
+// against what the kernel and its grid assume, return 0 on success and non-zero after
+// recording a message for mk_last_error().  Dtype codes: 0 = float32, 1 = bfloat16.
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+#define MK_ABI_VERSION 1
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+const char* mk_last_error();
+int mk_abi_version();
+
+// out[t, :] = table[ids[t], :] as float32 (the residual stream starts here).
+int mk_embed(const int* ids, const void* table, int dtype, float* out, int tokens, int hidden,
+             int vocab, hipStream_t stream);
+
+// RMSNorm of rows of the float32 residual stream h, optionally after adding `num_partials`
+// partial sums [p, row, hidden] (stride between partials in elements) into h.  `rows`, when
+// not null, lists the rows of h to normalise; out row i then comes from h row rows[i].
+int mk_rmsnorm(float* h, const float* partials, int num_partials, long long partial_stride,
+               const void* weight, int weight_dtype, float eps, const int* rows, void* out,
+               int out_dtype, int out_rows, int hidden, hipStream_t stream);
+
+// out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i].
+int mk_silu_mul(const void* gate_up, void* out, int dtype, int tokens, int inter,
+                hipStream_t stream);
+
+// Rotary encoding of the q and k heads of qkv [T, row_stride] (q in place) and the write of
+// rotated k and raw v into the paged cache [pages, n_kv, page_size, d].
+int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const float* cos_table,
+                     const float* sin_table, int table_positions, const int* positions,
+                     const int* token_seq, const int* block_table, int table_stride,
+                     void* k_cache, void* v_cache, int page_size, int n_q, int n_kv, int d,
+                     int rot, int write_kv, int tokens, hipStream_t stream);
+
+// y = x W^T (+ bias) with float32 FMA.  accumulate: y (float32) += instead of =.
+int mk_linear_generic(const void* x, const void* w, int dtype, const void* bias, int bias_dtype,
+                      void* out, int out_dtype, int accumulate, int M, int N, int K, int lda,
+                      int ldo, hipStream_t stream);
+
+// Causal grouped-query attention over the paged cache for any mix of prompt portions and
+// decoded tokens; window = 0 means all earlier keys.
+int mk_attention_generic(const void* q, int q_stride, void* out, int out_stride,
+                         const void* k_cache, const void* v_cache, int dtype,
+                         const int* positions, const int* token_seq, const int* block_table,
+                         int table_stride, int page_size, int n_q, int n_kv, int d, float scale,
+                         int window, int tokens, hipStream_t stream);
+
+int mk_argmax(const float* logits, int rows, int vocab, long long row_stride, int* out,
+              hipStream_t stream);
+
+int mk_sample(const float* logits, int rows, int vocab, long long row_stride,
+              const float* temperatures, const float* top_ps, const float* uniforms,
+              float* probs_scratch, int* out, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,72 @@
+"""Load the kernel libraries through ctypes and declare their C signatures.
+
+There is no fallback: when a library cannot be built or loaded, :func:`load` raises, and so
+does every op that would have called into it.
+"""
+
+from __future__ import annotations
+
+import ctypes
+from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
+
+from . import build
+
+ABI_VERSION = 1
+
+P, I, F, L = c_void_p, c_int, c_float, c_longlong
+
+# name -> argument types (every function returns int)
+_SIGNATURES = {
+    "core": {
+        "mk_embed": [P, P, I, P, I, I, I, P],
+        "mk_rmsnorm": [P, P, I, L, P, I, F, P, P, I, I, I, P],
+        "mk_silu_mul": [P, P, I, I, I, P],
+        "mk_rope_kv_write": [P, I, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
+        "mk_linear_generic": [P, P, I, P, I, P, I, I, I, I, I, I, I, P],
+        "mk_attention_generic": [P, I, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
+        "mk_argmax": [P, I, I, L, P, P],
+        "mk_sample": [P, I, I, L, P, P, P, P, P, P],
+    },
+}
+
+_loaded: dict = {}
+
+
+class KernelLibraryError(RuntimeError):
+    pass
+
+
+def load(name: str = "core") -> ctypes.CDLL:
+    """The library `name`, built first if no current build exists."""
+    lib = _loaded.get(name)
+    if lib is not None:
+        return lib
+    try:
+        path = build.build_library(name, force=False)
+    except build.BuildError as e:
+        raise KernelLibraryError(
+            f"the gfx950 kernel library '{name}' is not built and could not be built: {e}"
+        ) from e
+    try:
+        lib = ctypes.CDLL(str(path))
+    except OSError as e:
+        raise KernelLibraryError(f"cannot load {path}: {e}") from e
+    lib.mk_last_error.restype = c_char_p
+    lib.mk_last_error.argtypes = []
+    lib.mk_abi_version.restype = c_int
+    if lib.mk_abi_version() != ABI_VERSION:
+        raise KernelLibraryError(
+            f"{path} has ABI {lib.mk_abi_version()}, this package expects {ABI_VERSION}; rebuild"
+        )
+    for fn_name, argtypes in _SIGNATURES[name].items():
+        fn = getattr(lib, fn_name)
+        fn.argtypes = argtypes
+        fn.restype = c_int
+    _loaded[name] = lib
+    return lib
+
+
+def check(lib: ctypes.CDLL, code: int, what: str) -> None:
+    if code != 0:
+        message = lib.mk_last_error().decode(errors="replace")
+        raise KernelLibraryError(f"{what}: {message}")

@@ -1,0 +1,268 @@
+"""Python faces of the HIP kernels: tensors in, tensors out, shapes checked before the launch.
+
+Every function here runs a hand-written kernel on the current HIP stream of the tensors'
+device.  Nothing falls back to the CPU or to a library routine: a tensor that is not on the
+GPU, or a missing kernel library, raises.
+"""
+
+from __future__ import annotations
+
+import torch
+
+from . import lib as _lib
+
+F32, BF16 = 0, 1
+_DTYPE_CODE = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+class KernelArgumentError(ValueError):
+    pass
+
+
+def dtype_code(dtype: torch.dtype) -> int:
+    try:
+        return _DTYPE_CODE[dtype]
+    except KeyError:
+        raise KernelArgumentError(f"kernels take float32 or bfloat16 tensors, not {dtype}") from None
+
+
+def _stream() -> int:
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _dev(*tensors) -> None:
+    for t in tensors:
+        if t is None:
+            continue
+        if not t.is_cuda:
+            raise KernelArgumentError(
+                "kernel arguments must live on the GPU; there is no CPU path in this engine"
+            )
+        if not t.is_contiguous():
+            raise KernelArgumentError(f"kernel argument of shape {tuple(t.shape)} is not contiguous")
+
+
+def _ptr(t) -> int:
+    return 0 if t is None else t.data_ptr()
+
+
+def _i32(t: torch.Tensor, name: str) -> None:
+    if t.dtype != torch.int32:
+        raise KernelArgumentError(f"{name} must be int32, got {t.dtype}")
+
+
+# ------------------------------------------------------------------------------ row-wise ops
+
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t] = table[ids[t]] as float32 [T, H]."""
+    _dev(ids, table, out)
+    _i32(ids, "ids")
+    tokens, (vocab, hidden) = ids.shape[0], table.shape
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+    if out.shape != (tokens, hidden) or out.dtype != torch.float32:
+        raise KernelArgumentError("embed: out must be float32 [T, H]")
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_embed(_ptr(ids), _ptr(table), dtype_code(table.dtype), _ptr(out),
+                                 tokens, hidden, vocab, _stream()), "embed")
+    return out
+
+
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            rows: torch.Tensor | None = None, partials: torch.Tensor | None = None,
+            out: torch.Tensor | None = None) -> torch.Tensor:
+    """RMSNorm of the float32 residual stream h [T, H] into `out_dtype`.
+
+    `partials` [P, T, H] float32 are first summed into h (and h is updated); `rows` selects
+    and orders the rows to normalise.
+    """
+    _dev(h, weight, rows, partials, out)
+    if h.dtype != torch.float32 or h.dim() != 2:
+        raise KernelArgumentError("rmsnorm: h must be float32 [T, H]")
+    tokens, hidden = h.shape
+    if weight.shape != (hidden,):
+        raise KernelArgumentError(f"rmsnorm: weight {tuple(weight.shape)} does not match H={hidden}")
+    n_partials, stride = 0, 0
+    if partials is not None:
+        if partials.dtype != torch.float32 or partials.shape[1:] != h.shape:
+            raise KernelArgumentError("rmsnorm: partials must be float32 [P, T, H]")
+        n_partials, stride = partials.shape[0], tokens * hidden
+    out_rows = tokens
+    if rows is not None:
+        _i32(rows, "rows")
+        out_rows = rows.shape[0]
+    if out is None:
+        out = torch.empty((out_rows, hidden), dtype=out_dtype, device=h.device)
+    if out.shape != (out_rows, hidden) or out.dtype != out_dtype:
+        raise KernelArgumentError("rmsnorm: out has the wrong shape or dtype")
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_rmsnorm(_ptr(h), _ptr(partials), n_partials, stride, _ptr(weight),
+                                   dtype_code(weight.dtype), float(eps), _ptr(rows), _ptr(out),
+                                   dtype_code(out_dtype), out_rows, hidden, _stream()), "rmsnorm")
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up [T, 2I]."""
+    _dev(gate_up, out)
+    tokens, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelArgumentError("silu_mul: the last dimension must be even")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
+    if out.shape != (tokens, inter) or out.dtype != gate_up.dtype:
+        raise KernelArgumentError("silu_mul: out has the wrong shape or dtype")
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), tokens,
+                                    inter, _stream()), "silu_mul")
+    return out
+
+
+# --------------------------------------------------------------------------------- projection
+
+
+def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
+           out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
+           accumulate: bool = False) -> torch.Tensor:
+    """y = x W^T (+ bias) for x [M, K], W [N, K].
+
+    With `accumulate` the product is added into the float32 tensor `out` (the residual
+    stream) instead of being stored.  The result's dtype is `out_dtype` (default: x's).
+    """
+    _dev(x, w, bias, out)
+    if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
+        raise KernelArgumentError(f"linear: x {tuple(x.shape)} and W {tuple(w.shape)} do not match")
+    if x.dtype != w.dtype:
+        raise KernelArgumentError(f"linear: x is {x.dtype} but W is {w.dtype}")
+    m, k = x.shape
+    n = w.shape[0]
+    if bias is not None and bias.shape != (n,):
+        raise KernelArgumentError(f"linear: bias {tuple(bias.shape)} does not match N={n}")
+    if accumulate:
+        if out is None or out.dtype != torch.float32:
+            raise KernelArgumentError("linear: accumulation needs a float32 `out`")
+        out_dtype = torch.float32
+    if out is None:
+        out_dtype = out_dtype or x.dtype
+        out = torch.empty((m, n), dtype=out_dtype, device=x.device)
+    else:
+        out_dtype = out.dtype
+    if out.shape != (m, n):
+        raise KernelArgumentError(f"linear: out {tuple(out.shape)} is not [{m}, {n}]")
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_linear_generic(
+        _ptr(x), _ptr(w), dtype_code(x.dtype), _ptr(bias),
+        dtype_code(bias.dtype) if bias is not None else F32, _ptr(out), dtype_code(out_dtype),
+        int(accumulate), m, n, k, k, n, _stream()), "linear")
+    return out
+
+
+# ---------------------------------------------------------------------- positions and the cache
+
+
+def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
+                  positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
+                  k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, n_q: int,
+                  n_kv: int, head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
+    """Rotate q (in place) and k by their absolute positions; write k and v into the paged
+    cache [pages, n_kv, page_size, head_dim] at the slots the block table gives."""
+    _dev(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache)
+    _i32(positions, "positions")
+    _i32(token_seq, "token_seq")
+    _i32(block_table, "block_table")
+    tokens, row = qkv.shape
+    if positions.shape[0] != tokens or token_seq.shape[0] != tokens:
+        raise KernelArgumentError("rope: positions/token_seq must have one entry per token")
+    table_positions = 0
+    if rotary_dim:
+        if cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32:
+            raise KernelArgumentError("rope: float32 cos and sin tables are required")
+        if cos.shape != sin.shape or cos.shape[1] != rotary_dim // 2:
+            raise KernelArgumentError(
+                f"rope: tables {tuple(cos.shape)} do not match rotary width {rotary_dim}")
+        table_positions = cos.shape[0]
+    page_size = 1
+    if write_kv:
+        if k_cache is None or v_cache is None or k_cache.shape != v_cache.shape:
+            raise KernelArgumentError("rope: k and v caches of equal shape are required")
+        if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
+            raise KernelArgumentError("rope: cache dtype differs from the activations'")
+        if k_cache.dim() != 4 or k_cache.shape[1] != n_kv or k_cache.shape[3] != head_dim:
+            raise KernelArgumentError(
+                f"rope: cache {tuple(k_cache.shape)} is not [pages, {n_kv}, page, {head_dim}]")
+        page_size = k_cache.shape[2]
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_rope_kv_write(
+        _ptr(qkv), dtype_code(qkv.dtype), row, _ptr(cos), _ptr(sin), table_positions,
+        _ptr(positions), _ptr(token_seq), _ptr(block_table), block_table.shape[1],
+        _ptr(k_cache), _ptr(v_cache), page_size, n_q, n_kv, head_dim, rotary_dim,
+        int(write_kv), tokens, _stream()), "rope_kv_write")
+
+
+def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
+              n_q: int, n_kv: int, head_dim: int, scale: float, window: int | None = None,
+              out: torch.Tensor | None = None) -> torch.Tensor:
+    """Causal grouped-query attention of every token of the step over its sequence's cached
+    keys; q is read from rows of `q` with stride `q_stride` (the fused qkv buffer).
+    Returns [T, n_q * head_dim]."""
+    _dev(q, k_cache, v_cache, positions, token_seq, block_table, out)
+    _i32(positions, "positions")
+    _i32(token_seq, "token_seq")
+    _i32(block_table, "block_table")
+    tokens = positions.shape[0]
+    if q.numel() < (tokens - 1) * q_stride + n_q * head_dim and tokens:
+        raise KernelArgumentError("attention: q buffer too small")
+    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[1] != n_kv \
+            or k_cache.shape[3] != head_dim:
+        raise KernelArgumentError(
+            f"attention: cache {tuple(k_cache.shape)} is not [pages, {n_kv}, page, {head_dim}]")
+    if k_cache.dtype != q.dtype:
+        raise KernelArgumentError("attention: cache dtype differs from q's")
+    if out is None:
+        out = torch.empty((tokens, n_q * head_dim), dtype=q.dtype, device=q.device)
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_attention_generic(
+        _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
+        dtype_code(q.dtype), _ptr(positions), _ptr(token_seq), _ptr(block_table),
+        block_table.shape[1], k_cache.shape[2], n_q, n_kv, head_dim, float(scale),
+        int(window or 0), tokens, _stream()), "attention")
+    return out
+
+
+# ----------------------------------------------------------------------------------- sampling
+
+
+def argmax(logits: torch.Tensor) -> torch.Tensor:
+    """Lowest index of the largest value of each row of float32 logits [n, V] -> int32 [n]."""
+    _dev(logits)
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelArgumentError("argmax: logits must be float32 [n, V]")
+    rows, vocab = logits.shape
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_argmax(_ptr(logits), rows, vocab, vocab, _ptr(out), _stream()),
+               "argmax")
+    return out
+
+
+def sample(logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor,
+           uniforms: torch.Tensor) -> torch.Tensor:
+    """One token per row: argmax where temperature <= 0, else an inverse-CDF draw from the
+    temperature softmax restricted to the nucleus, using the row's uniform number."""
+    _dev(logits, temperatures, top_ps, uniforms)
+    if logits.dtype != torch.float32 or logits.dim() != 2:
+        raise KernelArgumentError("sample: logits must be float32 [n, V]")
+    rows, vocab = logits.shape
+    for name, t in (("temperatures", temperatures), ("top_ps", top_ps), ("uniforms", uniforms)):
+        if t.dtype != torch.float32 or t.shape != (rows,):
+            raise KernelArgumentError(f"sample: {name} must be float32 [{rows}]")
+    scratch = torch.empty((rows, vocab), dtype=torch.float32, device=logits.device)
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_sample(_ptr(logits), rows, vocab, vocab, _ptr(temperatures),
+                                  _ptr(top_ps), _ptr(uniforms), _ptr(scratch), _ptr(out),
+                                  _stream()), "sample")
+    return out

@@ -1,0 +1,94 @@
+"""Causal grouped-query softmax attention over a paged cache."""
+
+from __future__ import annotations
+
+import torch
+
+from ..kernels import ops
+from .base import CacheSpec, Mixer, PositionEncoding, TensorSpec
+
+
+class Attention(Mixer):
+    """q/k/v projections (optionally biased), position encoding on q and k, keys and values
+    written to the paged cache, softmax(q k^T * scale) v over the sequence's cached keys,
+    output projection (optionally biased) added into the accumulator.
+
+    Query head h reads key/value head h // (n_q / n_kv).  A query at absolute position p sees
+    keys j <= p, and with a window only j > p - window
+    (reference: mercury/model/qwen2.py:45-69, mercury/model/attention.py:9-32, :87-101).
+    Tensor names follow the checkpoint: ``q_proj``, ``k_proj``, ``v_proj``, ``o_proj``.
+    """
+
+    def __init__(self, hidden: int, n_q: int, n_kv: int, head_dim: int,
+                 position: PositionEncoding, qkv_bias: bool = True, o_bias: bool = False,
+                 scale: float | None = None, window: int | None = None):
+        if n_q % n_kv:
+            raise ValueError(f"{n_q} query heads are not a multiple of {n_kv} key/value heads")
+        self.hidden, self.n_q, self.n_kv, self.head_dim = int(hidden), int(n_q), int(n_kv), int(head_dim)
+        self.position = position
+        self.qkv_bias, self.o_bias = bool(qkv_bias), bool(o_bias)
+        self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
+        self.window = int(window) if window else None
+        self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
+
+    # ---- declarations
+
+    def cache_spec(self) -> CacheSpec:
+        return CacheSpec(self.n_kv, self.head_dim, self.window)
+
+    def param_specs(self) -> dict:
+        q, kv, h = self.n_q * self.head_dim, self.n_kv * self.head_dim, self.hidden
+        specs = {
+            "q_proj.weight": TensorSpec((q, h)),
+            "k_proj.weight": TensorSpec((kv, h)),
+            "v_proj.weight": TensorSpec((kv, h)),
+            "o_proj.weight": TensorSpec((h, q)),
+        }
+        if self.qkv_bias:
+            specs["q_proj.bias"] = TensorSpec((q,), role="vector")
+            specs["k_proj.bias"] = TensorSpec((kv,), role="vector")
+            specs["v_proj.bias"] = TensorSpec((kv,), role="vector")
+        if self.o_bias:
+            specs["o_proj.bias"] = TensorSpec((h,), role="vector")
+        return specs
+
+    def bind(self, params, dtype, device) -> None:
+        # One projection for q, k and v: rows [q heads | k heads | v heads].
+        self.w_qkv = torch.cat(
+            [params["q_proj.weight"], params["k_proj.weight"], params["v_proj.weight"]], dim=0
+        ).contiguous()
+        if self.qkv_bias:
+            biases = [params["q_proj.bias"], params["k_proj.bias"], params["v_proj.bias"]]
+            common = torch.float32 if any(b.dtype == torch.float32 for b in biases) else dtype
+            self.b_qkv = torch.cat([b.to(common) for b in biases]).contiguous()
+        self.w_o = params["o_proj.weight"]
+        self.b_o = params.get("o_proj.bias")
+
+    def prepare(self, max_positions: int, device) -> None:
+        self.position.prepare(max_positions, device)
+
+    def weight_bytes(self) -> int:
+        total = 0
+        for t in (self.w_qkv, self.b_qkv, self.w_o, self.b_o):
+            if t is not None:
+                total += t.numel() * t.element_size()
+        return total
+
+    # ---- one step
+
+    def forward(self, x, step, cache, state, accum) -> None:
+        n_q, n_kv, d = self.n_q, self.n_kv, self.head_dim
+        table = step.block_tables[cache.group]
+        if cache.writes:
+            qkv = ops.linear(x, self.w_qkv, self.b_qkv)
+        else:
+            # Reads a cache another entry fills: only the queries are projected.
+            rows = n_q * d
+            qkv = ops.linear(x, self.w_qkv[:rows], None if self.b_qkv is None else self.b_qkv[:rows])
+        pos = self.position
+        ops.rope_kv_write(qkv, pos.cos, pos.sin, step.positions, step.token_seq, table,
+                          cache.k if cache.writes else None, cache.v if cache.writes else None,
+                          n_q, n_kv if cache.writes else 0, d, pos.rotary_dim, cache.writes)
+        attended = ops.attention(qkv, qkv.shape[1], cache.k, cache.v, step.positions,
+                                 step.token_seq, table, n_q, n_kv, d, self.scale, self.window)
+        ops.linear(attended, self.w_o, self.b_o, out=accum, accumulate=True)

@@ -1,0 +1,139 @@
+"""What every part of a layer declares and does.
+
+A model is put together from parts: a *mixer* (what lets tokens see each other: attention
+here), a *feed-forward*, *norms*, a *position encoding* inside the mixer, and a *block* that
+arranges them around the residual stream.  A part is constructed from its own sizes and
+constants only; it never learns which model, layer index or checkpoint it belongs to.  The
+names under which its tensors are stored are given to it from outside (by the architecture's
+builder), as a prefix.
+
+Interfaces
+----------
+``Part.param_specs()``
+    local tensor name -> :class:`TensorSpec`.  The loader checks the checkpoint against the
+    union of all parts' specs and fills ``Part.bind``.
+``Part.bind(params, dtype, device)``
+    receives the loaded tensors (already on the device, in the dtype the spec's role
+    implies) and may repack them (concatenate q/k/v, gate/up) for its kernels.
+``Norm.forward(h, out_dtype, rows=None, partials=None) -> x``
+    h is the float32 residual stream [T, H].
+``Mixer.forward(x, step, cache, state, accum)`` / ``FeedForward.forward(x, step, accum)``
+    x is the normed input [T, H] in the compute dtype; the part **adds** its output into
+    ``accum`` (float32 [T, H]), which the block chooses (the residual stream in a pre-norm
+    block).  ``step`` is the :class:`~mercury_amd.engine.batch.StepContext` of this step
+    (per-token ids, positions and sequence index; per-sequence spans, lengths, block tables
+    and state slots).  ``cache`` is the :class:`LayerCache` the execution list assigns to this
+    call (possibly another layer's, read-only), ``state`` the per-request state tensor
+    [slots, ...] when the mixer declared a :class:`StateSpec`.
+``Mixer.cache_spec()`` / ``Mixer.state_spec()``
+    what the cache manager must provide: pages of keys and values (all of them or a window),
+    and/or a fixed-size state per request.
+"""
+
+from __future__ import annotations
+
+from dataclasses import dataclass
+
+import torch
+
+
+@dataclass(frozen=True)
+class TensorSpec:
+    """A stored tensor a part needs.
+
+    role
+        ``"matrix"``: an operand of a projection, kept in the compute dtype.
+        ``"vector"``: a bias or norm weight; kept in float32 when the checkpoint stores it in
+        32 bits, otherwise in the compute dtype.
+        ``"table"``: integers, kept as int32.
+    init
+        how the random-weights mode fills it: ``"normal"`` (mean 0), ``"one_plus_normal"``
+        (mean 1), ``"zeros"``.
+    """
+
+    shape: tuple
+    role: str = "matrix"
+    init: str = "normal"
+    optional: bool = False
+
+
+@dataclass(frozen=True)
+class CacheSpec:
+    """Per-token cache need of a mixer: keys and values of `kv_heads` heads of `head_dim`,
+    all earlier tokens (`window` None) or the last `window` of them."""
+
+    kv_heads: int
+    head_dim: int
+    window: int | None = None
+
+
+@dataclass(frozen=True)
+class StateSpec:
+    """Fixed-size per-request state of a mixer: one tensor of `shape` and `dtype` per request
+    slot, zeroed when a request takes the slot."""
+
+    shape: tuple
+    dtype: torch.dtype = torch.float32
+
+
+@dataclass
+class LayerCache:
+    """The paged keys and values one execution-list entry works on.
+
+    k, v: [pages, kv_heads, page_size, head_dim].  `group` indexes the step's block tables.
+    `writes` is false when the entry only reads a cache another entry fills.
+    """
+
+    k: torch.Tensor
+    v: torch.Tensor
+    group: int
+    page_size: int
+    writes: bool = True
+
+
+class Part:
+    """Base of all parts: declares tensors, receives them."""
+
+    def param_specs(self) -> dict:
+        return {}
+
+    def bind(self, params: dict, dtype: torch.dtype, device) -> None:
+        pass
+
+    def weight_bytes(self) -> int:
+        """Bytes of weights one step reads from this part (for roofline accounting)."""
+        return 0
+
+
+class Norm(Part):
+    def forward(self, h, out_dtype, rows=None, partials=None):
+        raise NotImplementedError
+
+
+class PositionEncoding(Part):
+    """Turns absolute positions into a transform of q and k.  `prepare` builds whatever tables
+    the transform needs for positions [0, max_positions)."""
+
+    rotary_dim = 0
+
+    def prepare(self, max_positions: int, device) -> None:
+        pass
+
+
+class Mixer(Part):
+    def cache_spec(self) -> CacheSpec | None:
+        return None
+
+    def state_spec(self) -> StateSpec | None:
+        return None
+
+    def prepare(self, max_positions: int, device) -> None:
+        pass
+
+    def forward(self, x, step, cache, state, accum) -> None:
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    def forward(self, x, step, accum) -> None:
+        raise NotImplementedError

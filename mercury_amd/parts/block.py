@@ -1,0 +1,54 @@
+"""How a layer's parts are arranged around the residual stream."""
+
+from __future__ import annotations
+
+from .base import FeedForward, Mixer, Norm, Part
+
+
+class PreNormBlock(Part):
+    """h += mixer(norm_1(h)); h += ffn(norm_2(h)), h being the float32 residual stream.
+
+    This is the reference's layer (mercury/model/qwen2.py:82-94) with its carried `residual`
+    written as the running sum: the reference adds the previous output inside the next norm,
+    here each part adds its output into h as it produces it.
+
+    `names` gives the checkpoint sub-prefix of each part, e.g. ``{"mixer": "self_attn.",
+    "ffn": "mlp.", "norm_mixer": "input_layernorm.", "norm_ffn": "post_attention_layernorm."}``.
+    """
+
+    def __init__(self, mixer: Mixer, ffn: FeedForward | None, norm_mixer: Norm,
+                 norm_ffn: Norm | None, names: dict):
+        self.mixer, self.ffn, self.norm_mixer, self.norm_ffn = mixer, ffn, norm_mixer, norm_ffn
+        self.names = dict(names)
+
+    def _children(self):
+        out = [("mixer", self.mixer), ("norm_mixer", self.norm_mixer)]
+        if self.ffn is not None:
+            out += [("ffn", self.ffn), ("norm_ffn", self.norm_ffn)]
+        return out
+
+    def param_specs(self) -> dict:
+        specs = {}
+        for key, part in self._children():
+            for name, spec in part.param_specs().items():
+                specs[self.names[key] + name] = spec
+        return specs
+
+    def bind(self, params, dtype, device) -> None:
+        for key, part in self._children():
+            prefix = self.names[key]
+            part.bind({n[len(prefix):]: t for n, t in params.items() if n.startswith(prefix)},
+                      dtype, device)
+
+    def prepare(self, max_positions: int, device) -> None:
+        self.mixer.prepare(max_positions, device)
+
+    def weight_bytes(self) -> int:
+        return sum(part.weight_bytes() for _, part in self._children())
+
+    def forward(self, h, step, cache, state, dtype) -> None:
+        x = self.norm_mixer.forward(h, dtype)
+        self.mixer.forward(x, step, cache, state, h)
+        if self.ffn is not None:
+            x = self.norm_ffn.forward(h, dtype)
+            self.ffn.forward(x, step, h)
