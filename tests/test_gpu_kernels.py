@@ -1,0 +1,450 @@
+"""Each HIP kernel alone against a plain float32 reference of the same op, at sizes other than
+the engine's own (odd row counts, widths that are no power of two, several head sizes)."""
+
+from __future__ import annotations
+
+import math
+
+import pytest
+import torch
+
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DTYPES = [torch.float32, torch.bfloat16]
+
+
+def ops():
+    from mercury_amd.kernels import ops as o
+
+    return o
+
+
+def tol(dtype):
+    # float32: a few ulps of accumulated error; bfloat16: one rounding of the output (2^-8).
+    return dict(atol=2e-6, rtol=1e-5) if dtype == torch.float32 else dict(atol=1e-2, rtol=1.6e-2)
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+def as_dtype(x, dtype):
+    """The values the kernel will see, as float32 on the host, and the device tensor."""
+    d = x.to(dtype)
+    return d.float(), d.to(DEV)
+
+
+# ------------------------------------------------------------------------------- embedding
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_embed_gathers_rows_as_float32(dtype):
+    table_h, table_d = as_dtype(rnd(1003, 168), dtype)
+    ids = torch.tensor([0, 1002, 5, 5, 77], dtype=torch.int32)
+    out = ops().embed(ids.to(DEV), table_d)
+    assert out.dtype == torch.float32
+    assert torch.equal(out.cpu(), table_h[ids.long()])
+
+
+# --------------------------------------------------------------------------------- RMSNorm
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows,cols", [(1, 896), (7, 1000), (129, 168), (3, 4100)])
+def test_rmsnorm_matches_plain(dtype, rows, cols):
+    h = rnd(rows, cols, seed=1, scale=3.0)
+    w_h, w_d = as_dtype(1 + rnd(cols, seed=2, scale=0.1), dtype)
+    want, _ = plain.rms_norm(h, w_h, 1e-5)
+    got = ops().rmsnorm(h.to(DEV), w_d, 1e-5, dtype)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype))
+
+
+def test_rmsnorm_against_the_library_routine():
+    h = rnd(5, 264, seed=3)
+    w = 1 + rnd(264, seed=4, scale=0.1)
+    want = torch.nn.functional.rms_norm(h, (264,), w, 1e-6)
+    got = ops().rmsnorm(h.to(DEV), w.to(DEV), 1e-6, torch.float32)
+    torch.testing.assert_close(got.cpu(), want, atol=2e-6, rtol=1e-5)
+
+
+def test_rmsnorm_constant_and_zero_rows():
+    eps = 1e-6
+    h = torch.zeros(2, 300)
+    h[1] = 2.5
+    got = ops().rmsnorm(h.to(DEV), torch.ones(300, device=DEV), eps, torch.float32).cpu()
+    assert torch.equal(got[0], torch.zeros(300))            # no NaN from an all-zero row
+    assert torch.allclose(got[1], torch.full((300,), 2.5 / math.sqrt(2.5**2 + eps)), atol=1e-6)
+
+
+def test_rmsnorm_adds_partial_sums_into_the_stream_first():
+    """The residual sum is part of the norm: h <- h + sum(partials), then normalise
+    (reference: the sum is the norm's second result, mercury/model/qwen2.py:27-31)."""
+    h = rnd(9, 200, seed=5)
+    parts = rnd(3, 9, 200, seed=6)
+    w = 1 + rnd(200, seed=7, scale=0.1)
+    want, total = plain.rms_norm(parts.sum(0), w, 1e-6, residual=h)
+    h_d = h.to(DEV)
+    got = ops().rmsnorm(h_d, w.to(DEV), 1e-6, torch.float32, partials=parts.to(DEV))
+    torch.testing.assert_close(h_d.cpu(), total, atol=1e-6, rtol=1e-6)
+    torch.testing.assert_close(got.cpu(), want, atol=3e-6, rtol=1e-5)
+
+
+def test_rmsnorm_selected_rows_in_caller_order():
+    h = rnd(20, 128, seed=8)
+    w = torch.ones(128)
+    rows = torch.tensor([19, 0, 7], dtype=torch.int32)
+    want, _ = plain.rms_norm(h[rows.long()], w, 1e-6)
+    got = ops().rmsnorm(h.to(DEV), w.to(DEV), 1e-6, torch.float32, rows=rows.to(DEV))
+    torch.testing.assert_close(got.cpu(), want, atol=2e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("weight_dtype", DTYPES)
+def test_rmsnorm_bfloat16_output_with_either_weight_precision(weight_dtype):
+    h = rnd(4, 896, seed=9)
+    w_h, w_d = as_dtype(1 + rnd(896, seed=10, scale=0.1), weight_dtype)
+    want, _ = plain.rms_norm(h, w_h, 1e-6)
+    got = ops().rmsnorm(h.to(DEV), w_d, 1e-6, torch.bfloat16)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(torch.bfloat16))
+
+
+# ------------------------------------------------------------------------------ projections
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("m,n,k", [(1, 1003, 168), (70, 130, 50), (129, 64, 257), (5, 1, 7)])
+def test_linear_matches_the_library_product(dtype, m, n, k):
+    x_h, x_d = as_dtype(rnd(m, k, seed=11), dtype)
+    w_h, w_d = as_dtype(rnd(n, k, seed=12, scale=0.1), dtype)
+    b_h, b_d = as_dtype(rnd(n, seed=13), dtype)
+    want = torch.nn.functional.linear(x_h.double(), w_h.double(), b_h.double()).float()
+    got = ops().linear(x_d, w_d, b_d)
+    assert got.dtype == dtype
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype))
+    # float32 result from bfloat16 operands (the logits path)
+    got32 = ops().linear(x_d, w_d, None, out_dtype=torch.float32)
+    want32 = torch.nn.functional.linear(x_h.double(), w_h.double()).float()
+    torch.testing.assert_close(got32.cpu(), want32, atol=1e-5, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_linear_accumulates_into_the_float32_stream(dtype):
+    x_h, x_d = as_dtype(rnd(33, 100, seed=14), dtype)
+    w_h, w_d = as_dtype(rnd(72, 100, seed=15, scale=0.1), dtype)
+    acc = rnd(33, 72, seed=16)
+    acc_d = acc.to(DEV)
+    ops().linear(x_d, w_d, out=acc_d, accumulate=True)
+    want = acc + (x_h.double() @ w_h.double().T).float()
+    torch.testing.assert_close(acc_d.cpu(), want, atol=1e-5, rtol=1e-5)
+
+
+def test_linear_rows_do_not_depend_on_the_batch():
+    """A row's result is bitwise the same alone and among 100 others."""
+    x = rnd(101, 300, seed=17).to(DEV)
+    w = rnd(77, 300, seed=18).to(DEV)
+    together = ops().linear(x, w)
+    alone = ops().linear(x[50:51].contiguous(), w)
+    assert torch.equal(together[50:51], alone)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_silu_mul_matches_plain(dtype):
+    gu_h, gu_d = as_dtype(rnd(13, 2 * 410, seed=19, scale=2.0), dtype)
+    want = plain.silu(gu_h[:, :410]) * gu_h[:, 410:]
+    got = ops().silu_mul(gu_d)
+    torch.testing.assert_close(got.float().cpu(), want, **tol(dtype))
+    assert torch.equal(ops().silu_mul(torch.zeros(2, 8, device=DEV)).cpu(), torch.zeros(2, 4))
+    torch.testing.assert_close(plain.silu(gu_h), torch.nn.functional.silu(gu_h))
+
+
+# ------------------------------------------------------------------- rotary + cache write
+
+
+def rotary_tables(d, theta, positions):
+    cos, sin = plain.rotary_table(d, range(positions), theta)
+    return cos[:, : d // 2].contiguous(), sin[:, : d // 2].contiguous()
+
+
+def paged(kv, pages, page_size, num_pages, dtype):
+    """Host helper: lay [S, n_kv, d] out in a cache [num_pages, n_kv, page, d]."""
+    s, n_kv, d = kv.shape
+    cache = torch.zeros(num_pages, n_kv, page_size, d, dtype=dtype)
+    for p in range(s):
+        cache[pages[p // page_size], :, p % page_size, :] = kv[p].to(dtype)
+    return cache
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(4, 2, 16, 16), (6, 1, 48, 8), (3, 3, 80, 32)])
+def test_rope_and_cache_write(dtype, n_q, n_kv, d, page):
+    theta, max_pos = 10000.0, 128
+    cos, sin = rotary_tables(d, theta, max_pos)
+    # two sequences: tokens at positions 30..39 of sequence 0, position 70 of sequence 1
+    positions = list(range(30, 40)) + [70]
+    token_seq = [0] * 10 + [1]
+    table = torch.full((2, max_pos // page), -1, dtype=torch.int32)
+    table[0, : 40 // page + 1] = torch.arange(3, 3 + 40 // page + 1, dtype=torch.int32)
+    table[1, : 70 // page + 1] = torch.arange(20, 20 + 70 // page + 1, dtype=torch.int32)
+    tokens = len(positions)
+    qkv_h, qkv_d = as_dtype(rnd(tokens, (n_q + 2 * n_kv) * d, seed=20), dtype)
+    k_cache = torch.zeros(40, n_kv, page, d, dtype=dtype, device=DEV)
+    v_cache = torch.zeros_like(k_cache)
+    ops().rope_kv_write(qkv_d, cos.to(DEV), sin.to(DEV),
+                        torch.tensor(positions, dtype=torch.int32, device=DEV),
+                        torch.tensor(token_seq, dtype=torch.int32, device=DEV), table.to(DEV),
+                        k_cache, v_cache, n_q, n_kv, d, d)
+    q = qkv_h[:, : n_q * d].view(tokens, n_q, d)
+    k = qkv_h[:, n_q * d: (n_q + n_kv) * d].view(tokens, n_kv, d)
+    v = qkv_h[:, (n_q + n_kv) * d:].view(tokens, n_kv, d)
+    full_cos, full_sin = plain.rotary_table(d, positions, theta)
+    q_want, k_want = plain.apply_rotary(q, k, full_cos, full_sin)
+    torch.testing.assert_close(qkv_d[:, : n_q * d].float().cpu().view(tokens, n_q, d), q_want, **tol(dtype))
+    touched = torch.zeros(40, page, dtype=torch.bool)
+    for t, (p, s) in enumerate(zip(positions, token_seq)):
+        pg, off = int(table[s, p // page]), p % page
+        assert plain.slot_mapping(table[s].tolist(), p, p + 1, page) == [pg * page + off]
+        torch.testing.assert_close(k_cache[pg, :, off].float().cpu(), k_want[t], **tol(dtype))
+        assert torch.equal(v_cache[pg, :, off].float().cpu(), v[t])
+        touched[pg, off] = True
+    untouched = ~touched[:, None, :, None].expand(40, n_kv, page, d)
+    assert torch.count_nonzero(k_cache.cpu()[untouched]) == 0
+    assert torch.count_nonzero(v_cache.cpu()[untouched]) == 0
+
+
+def test_rotary_pairing_sign_and_identity_at_zero():
+    """rotate_half([1,2,3,4]) = [-3,-4,1,2] (reference: tests/test_attention.py:177-179):
+    with cos = 0 and sin = 1 the kernel must return exactly that; position 0 is the identity."""
+    assert torch.equal(plain.rotate_half(torch.tensor([[1.0, 2.0, 3.0, 4.0]])),
+                       torch.tensor([[-3.0, -4.0, 1.0, 2.0]]))
+    cos = torch.tensor([[1.0, 1.0], [0.0, 0.0]], device=DEV)
+    sin = torch.tensor([[0.0, 0.0], [1.0, 1.0]], device=DEV)
+    qkv = torch.tensor([[1.0, 2.0, 3.0, 4.0], [1.0, 2.0, 3.0, 4.0]], device=DEV)
+    ops().rope_kv_write(qkv, cos, sin, torch.tensor([0, 1], dtype=torch.int32, device=DEV),
+                        torch.zeros(2, dtype=torch.int32, device=DEV),
+                        torch.zeros(1, 1, dtype=torch.int32, device=DEV), None, None, 1, 0, 4, 4,
+                        write_kv=False)
+    assert torch.equal(qkv.cpu(), torch.tensor([[1.0, 2.0, 3.0, 4.0], [-3.0, -4.0, 1.0, 2.0]]))
+
+
+def test_rotary_scores_depend_on_distance_only():
+    """<rot(q, m), rot(k, n)> is the same for (3, 3) and (9, 9), and for (5, 2) and (105, 102)
+    (reference: tests/test_attention.py:182-197)."""
+    d = 32
+    cos, sin = rotary_tables(d, 10000.0, 128)
+    base_h = rnd(1, 2 * d, seed=21)
+
+    def rotated(pos_q, pos_k):
+        out = []
+        for pos in (pos_q, pos_k):
+            buf = base_h.clone().to(DEV)  # two heads: q and "k" both as q heads
+            ops().rope_kv_write(buf, cos.to(DEV), sin.to(DEV),
+                                torch.tensor([pos], dtype=torch.int32, device=DEV),
+                                torch.zeros(1, dtype=torch.int32, device=DEV),
+                                torch.zeros(1, 1, dtype=torch.int32, device=DEV), None, None, 2, 0,
+                                d, d, write_kv=False)
+            out.append(buf.cpu())
+        return float((out[0][0, :d] * out[1][0, d:]).sum())
+
+    assert abs(rotated(3, 3) - rotated(9, 9)) < 1e-5
+    assert abs(rotated(5, 2) - rotated(105, 102)) < 1e-4
+    assert abs(rotated(5, 2) - rotated(2, 5)) > 1e-3   # the sign of the distance matters
+
+
+# --------------------------------------------------------------------------------- attention
+
+
+def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens, q_lens, scale,
+                  window=None, poison=None):
+    """q_h: list per sequence of [q_len, n_q, d] (the last q_len positions of the sequence);
+    k_h/v_h: list per sequence of [seq_len, n_kv, d]."""
+    n_q, d = q_h[0].shape[1:]
+    n_kv = k_h[0].shape[1]
+    k_cache = torch.zeros(num_pages, n_kv, page, d, dtype=dtype)
+    v_cache = torch.zeros_like(k_cache)
+    if poison is not None:
+        k_cache[:] = poison
+        v_cache[:] = poison
+    width = max(len(p) for p in pages_per_seq)
+    table = torch.full((len(q_h), width), -1, dtype=torch.int32)
+    positions, token_seq = [], []
+    for s, pages in enumerate(pages_per_seq):
+        table[s, : len(pages)] = torch.tensor(pages, dtype=torch.int32)
+        for p in range(seq_lens[s]):
+            k_cache[pages[p // page], :, p % page] = k_h[s][p].to(dtype)
+            v_cache[pages[p // page], :, p % page] = v_h[s][p].to(dtype)
+        positions += list(range(seq_lens[s] - q_lens[s], seq_lens[s]))
+        token_seq += [s] * q_lens[s]
+    q_flat = torch.cat([q.reshape(q.shape[0], n_q * d) for q in q_h]).to(dtype).to(DEV)
+    out = ops().attention(q_flat, n_q * d, k_cache.to(DEV), v_cache.to(DEV),
+                          torch.tensor(positions, dtype=torch.int32, device=DEV),
+                          torch.tensor(token_seq, dtype=torch.int32, device=DEV), table.to(DEV),
+                          n_q, n_kv, d, scale, window)
+    return out.float().cpu().view(-1, n_q, d)
+
+
+def rounded(x, dtype):
+    return x.to(dtype).float()
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("n_q,n_kv,d,page", [(4, 2, 8, 16), (6, 1, 48, 8), (2, 2, 128, 16),
+                                             (14, 2, 64, 16), (3, 1, 80, 4)])
+def test_attention_whole_prompt_matches_plain(dtype, n_q, n_kv, d, page):
+    """(reference: tests/test_attention.py:67-81; scattered pages as in :135-153)"""
+    s = 40 if d < 100 else 70
+    q, k, v = (rounded(rnd(s, h, d, seed=30 + i), dtype) for i, h in enumerate((n_q, n_kv, n_kv)))
+    pages = [11, 3, 7, 30, 2, 19, 25, 1, 9, 14, 22, 5, 28, 8, 17, 6, 4, 12][: -(-s // page)]
+    got = run_attention([q], [k], [v], dtype, [pages], page, 32, [s], [s], d ** -0.5, poison=1e4)
+    want = plain.causal_attention(q, k, v, d ** -0.5)
+    torch.testing.assert_close(got, want, **tol(dtype))
+    if dtype == torch.float32:
+        lib = torch.nn.functional.scaled_dot_product_attention(
+            q.transpose(0, 1)[None], k.repeat_interleave(n_q // n_kv, 1).transpose(0, 1)[None],
+            v.repeat_interleave(n_q // n_kv, 1).transpose(0, 1)[None], is_causal=True)[0].transpose(0, 1)
+        torch.testing.assert_close(got, lib, atol=2e-6, rtol=1e-5)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_suffix_over_a_cached_prefix_and_decode_rows(dtype):
+    """A 16-token portion at positions 32..47, beside two single decoded tokens of sequences
+    of 33 and 17 tokens, in one batch (reference: tests/test_attention.py:84-132 tests the two
+    cases separately)."""
+    n_q, n_kv, d, page = 4, 2, 8, 16
+    lens, q_lens = [48, 33, 17], [16, 1, 1]
+    qs, ks, vs = [], [], []
+    for i, (s, ql) in enumerate(zip(lens, q_lens)):
+        ks.append(rounded(rnd(s, n_kv, d, seed=40 + i), dtype))
+        vs.append(rounded(rnd(s, n_kv, d, seed=50 + i), dtype))
+        qs.append(rounded(rnd(s, n_q, d, seed=60 + i), dtype))
+    got = run_attention([q[-ql:] for q, ql in zip(qs, q_lens)], ks, vs, dtype,
+                        [[2, 5, 9], [12, 1, 30], [7, 20]], page, 32, lens, q_lens, d ** -0.5,
+                        poison=1e4)
+    want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5)[-ql:]
+                      for q, k, v, ql in zip(qs, ks, vs, q_lens)])
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("target", [0, 15, 16, 255, 256, 499, 500])
+def test_attention_finds_one_far_key(dtype, target):
+    """One key among 501 is made to win the softmax outright (its score stands 40 above the
+    rest); the output must be that key's value row.  Random weights alone would average over
+    hundreds of keys and hide a key that is skipped or read from the wrong slot: the first
+    key, the last, and both sides of page edges are each tried."""
+    n_q, n_kv, d, page, s = 2, 1, 32, 16, 501
+    k = rounded(rnd(s, n_kv, d, seed=70, scale=0.1), dtype)
+    v = rounded(rnd(s, n_kv, d, seed=71), dtype)
+    q = rounded(rnd(1, n_q, d, seed=72, scale=0.1), dtype)
+    direction = torch.zeros(d)
+    direction[3] = 16.0
+    k[target, 0] = direction
+    q[0, :] = direction * (40.0 * math.sqrt(d) / 256.0)
+    q = rounded(q, dtype)
+    pages = list(range(40, 40 + -(-s // page)))
+    got = run_attention([q], [k], [v], dtype, [pages], page, 80, [s], [1], d ** -0.5, poison=1e4)
+    torch.testing.assert_close(got[0, 0], v[target, 0], atol=1e-3, rtol=1e-3)
+    torch.testing.assert_close(got, plain.causal_attention(q, k, v, d ** -0.5, s - 1), **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+def test_attention_special_cases_reduce_to_means(dtype):
+    """One visible key -> its value; equal scores -> the mean of the visible values."""
+    n_q, n_kv, d, page = 2, 1, 16, 8
+    v = rounded(rnd(20, n_kv, d, seed=73), dtype)
+    k = torch.zeros(20, n_kv, d)
+    q = rounded(rnd(20, n_q, d, seed=74), dtype)
+    got = run_attention([q], [k], [v], dtype, [[4, 2, 6]], page, 8, [20], [20], d ** -0.5)
+    for p in (0, 1, 7, 8, 19):
+        want = v[: p + 1, 0].mean(0)
+        torch.testing.assert_close(got[p, 0], want, **tol(dtype))
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 64])
+def test_attention_window_edge(dtype, window):
+    """With a window w the query at p sees keys p-w+1..p; pages wholly before the window are
+    absent from the table (-1), as the cache manager leaves them."""
+    n_q, n_kv, d, page, s = 4, 2, 16, 8, 45
+    q, k, v = (rounded(rnd(s, h, d, seed=80 + i), dtype) for i, h in enumerate((n_q, n_kv, n_kv)))
+    q_len = 6
+    pages = list(range(10, 10 + -(-s // page)))
+    first_needed = max(0, (s - q_len) - window + 1)
+    gone = first_needed // page
+    table_pages = [-1] * gone + pages[gone:]
+    # the helper writes through the table, so fill the cache with the full list and only
+    # hide the pages afterwards
+    n_qh = q[-q_len:]
+    k_cache = paged(k, pages, page, 32, dtype)
+    v_cache = paged(v, pages, page, 32, dtype)
+    for g in range(gone):
+        k_cache[pages[g]] = 1e4
+        v_cache[pages[g]] = 1e4
+    table = torch.tensor([table_pages], dtype=torch.int32)
+    out = ops().attention(n_qh.reshape(q_len, n_q * d).to(dtype).to(DEV), n_q * d,
+                          k_cache.to(DEV), v_cache.to(DEV),
+                          torch.arange(s - q_len, s, dtype=torch.int32, device=DEV),
+                          torch.zeros(q_len, dtype=torch.int32, device=DEV), table.to(DEV),
+                          n_q, n_kv, d, d ** -0.5, window)
+    want = plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-q_len:]
+    torch.testing.assert_close(out.float().cpu().view(q_len, n_q, d), want, **tol(dtype))
+
+
+def test_attention_gqa_equals_mha_with_repeated_heads():
+    n_q, n_kv, d, page, s = 6, 2, 16, 16, 37
+    q, k, v = (rnd(s, h, d, seed=90 + i) for i, h in enumerate((n_q, n_kv, n_kv)))
+    grouped = run_attention([q], [k], [v], torch.float32, [[1, 2, 3]], page, 8, [s], [s], 0.25)
+    repeated = run_attention([q], [k.repeat_interleave(3, 1)], [v.repeat_interleave(3, 1)],
+                             torch.float32, [[1, 2, 3]], page, 8, [s], [s], 0.25)
+    assert torch.equal(grouped, repeated)
+
+
+# ----------------------------------------------------------------------------------- sampling
+
+
+def test_argmax_takes_the_lowest_index_among_equals():
+    logits = rnd(5, 1003, seed=100)
+    logits[2, 77] = logits[2, 900] = 50.0
+    logits[4, 1002] = 60.0
+    got = ops().argmax(logits.to(DEV)).cpu()
+    assert got.tolist() == logits.argmax(-1).tolist()
+    assert got[2] == 77 and got[4] == 1002
+
+
+def test_sampling_rules():
+    """(reference: mercury/sampling.py:17-35)  Greedy rows take the argmax whatever top_p says;
+    sampled rows follow the inverse CDF of the plain distribution for their own uniform."""
+    vocab = 1003
+    logits = rnd(6, vocab, seed=101, scale=2.0)
+    temps = torch.tensor([0.0, 0.8, 0.8, 1.5, 1e-7, 0.8])
+    top_ps = torch.tensor([0.5, 1.0, 0.9, 0.3, 1.0, 0.9])
+    us = torch.tensor([0.3, 0.999, 0.5, 0.01, 0.7, 0.0])
+    got = ops().sample(logits.to(DEV), temps.to(DEV), top_ps.to(DEV), us.to(DEV)).cpu().tolist()
+    assert got[0] == int(logits[0].argmax())
+    assert got[4] == int(logits[4].argmax())       # temperature -> 0 is the argmax
+    for r in (1, 2, 3, 5):
+        probs = plain.sampling_distribution(logits[r], float(temps[r]), float(top_ps[r]))
+        want = plain.inverse_cdf_draw(probs, float(us[r]))
+        assert probs[got[r]] > 0, "drew a token outside the nucleus"
+        if got[r] != want:  # only a rounding of the cumulative sum may move the draw
+            cum = probs.double().cumsum(-1)
+            lo, hi = sorted((got[r], want))
+            assert abs(float(cum[hi - 1] - float(us[r]))) < 1e-5 or float(cum[hi] - cum[lo]) < 1e-5
+
+
+def test_sampling_frequencies_follow_the_distribution():
+    vocab = 50
+    logits = rnd(1, vocab, seed=102, scale=1.5).repeat(4000, 1)
+    g = torch.Generator().manual_seed(5)
+    us = torch.rand(4000, generator=g)
+    temps, top_ps = torch.full((4000,), 0.7), torch.full((4000,), 0.8)
+    got = ops().sample(logits.to(DEV), temps.to(DEV), top_ps.to(DEV), us.to(DEV)).cpu()
+    probs = plain.sampling_distribution(logits[0], 0.7, 0.8)
+    freq = torch.bincount(got.long(), minlength=vocab).float() / 4000
+    assert torch.all(freq[probs == 0] == 0)
+    assert (freq - probs).abs().max() < 0.03
+    # the crossing token stays: the kept mass reaches top_p
+    full = torch.softmax(logits[0] / 0.7, -1)
+    assert full[probs > 0].sum() >= 0.8
