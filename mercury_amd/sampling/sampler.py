@@ -1,0 +1,45 @@
+"""Turning logits into tokens: greedy, temperature and nucleus sampling
+(reference: mercury/sampling.py:17-35), with one reproducible random stream per request.
+
+The reference draws every row of a step from one engine-wide generator, so a request's tokens
+depend on what else is in the batch.  Here the uniform number for output token `index` of a
+request is a function of (seed, request id, index) alone: a request samples the same tokens
+alone, batched, cut into portions or after a preemption.
+"""
+
+from __future__ import annotations
+
+import hashlib
+import struct
+
+import torch
+
+from ..kernels import ops
+
+
+def uniform_for(seed: int, rid: str, index: int) -> float:
+    """A number in [0, 1) with 24 random bits, from a keyed hash of the three arguments."""
+    digest = hashlib.blake2b(f"{rid}:{index}".encode(), digest_size=8,
+                             key=struct.pack("<q", int(seed) & (2**63 - 1))).digest()
+    return (int.from_bytes(digest, "little") >> 40) / float(1 << 24)
+
+
+class Sampler:
+    def __init__(self, seed: int = 0):
+        self.seed = int(seed)
+
+    def sample(self, logits: torch.Tensor, requests: list) -> list:
+        """One token per row of float32 logits [n, V]; row i belongs to requests[i], whose
+        next output index is len(request.out)."""
+        if logits.shape[0] != len(requests):
+            raise ValueError(f"{logits.shape[0]} rows of logits for {len(requests)} requests")
+        if not requests:
+            return []
+        if all(r.params.greedy for r in requests):
+            return ops.argmax(logits).cpu().tolist()
+        temps = [float(r.params.temperature) for r in requests]
+        top_ps = [float(r.params.top_p) for r in requests]
+        us = [uniform_for(self.seed if r.params.seed is None else r.params.seed, r.rid, len(r.out))
+              for r in requests]
+        packed = torch.tensor([temps, top_ps, us], dtype=torch.float32).to(logits.device)
+        return ops.sample(logits, packed[0], packed[1], packed[2]).cpu().tolist()

@@ -1,0 +1,159 @@
+"""Generation through the Python entry point and the command line, against the plain
+implementation; the same tokens alone, batched, cut into portions, after a warm prefix cache
+and after forced preemption (reference: tests/test_runner.py:84-155)."""
+
+from __future__ import annotations
+
+import json
+import subprocess
+import sys
+
+import pytest
+import torch
+
+from tests import helpers
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+
+PROMPT = [(i * 13 + 7) % 500 for i in range(80)]
+OTHER = [(i * 29 + 3) % 500 for i in range(56)]
+
+
+def engine(name="A", dtype="float32", **kw):
+    from mercury_amd import Engine, EngineConfig
+
+    kw.setdefault("num_blocks", 64)
+    kw.setdefault("max_model_len", 512)
+    return Engine(EngineConfig(model=str(helpers.model_folder(name)), dtype=dtype, **kw))
+
+
+def generate(eng, prompts, max_tokens=12, **params):
+    from mercury_amd import SamplingParams
+
+    out = eng.generate(prompts, SamplingParams(ignore_eos=True, **params), max_tokens)
+    assert eng.leaked_blocks() == 0
+    return out
+
+
+def plausible(folder, prompt, tokens, fraction=0.02):
+    """Every generated token is the plain model's argmax at its place, or within the
+    bfloat16 bound of it (2% of the largest logit)."""
+    w, cfg = helpers.plain_model(folder)
+    logits = plain.forward_logits(w, cfg, prompt + tokens)[len(prompt) - 1:-1]
+    chosen = logits[torch.arange(len(tokens)), torch.tensor(tokens)]
+    return bool((logits.max(-1).values - chosen <= 2 * fraction * logits.abs().max()).all())
+
+
+@pytest.mark.parametrize("name", ["A", "B", "C"])
+def test_greedy_generation_equals_the_plain_implementation(name):
+    folder = helpers.model_folder(name)
+    w, cfg = helpers.plain_model(folder)
+    vocab = cfg["vocab_size"]
+    prompts = [helpers.random_tokens(vocab, n, seed=n) for n in (5, 17, 33, 1)]
+    want = [plain.greedy_generate(w, cfg, p, 8) for p in prompts]
+    assert generate(engine(name), prompts, 8) == want
+    got = generate(engine(name, "bfloat16"), prompts, 8)
+    assert all(plausible(folder, p, g) for p, g in zip(prompts, got))
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_the_same_tokens_however_the_work_is_cut(dtype):
+    alone = {k: generate(engine(dtype=dtype), [p])[0] for k, p in (("a", PROMPT), ("b", OTHER))}
+    together = generate(engine(dtype=dtype), [PROMPT, OTHER])
+    assert together == [alone["a"], alone["b"]]
+    portions = generate(engine(dtype=dtype, prefill_budget=24), [PROMPT, OTHER])
+    assert portions == together
+    crowd = [[(i * 31 + j) % 500 for j in range(48)] for i in range(6)] + [PROMPT]
+    assert generate(engine(dtype=dtype, max_running=8), crowd)[-1] == alone["a"]
+    small_pages = generate(engine(dtype=dtype, block_size=8, num_blocks=128), [PROMPT, OTHER])
+    assert small_pages == together
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_warm_prefix_cache_and_rope_positions_after_it(dtype):
+    eng = engine(dtype=dtype)
+    cold = generate(eng, [PROMPT])[0]
+    assert eng.manager.main_pool.stats["hit_tokens"] == 0
+    assert generate(eng, [PROMPT])[0] == cold
+    assert eng.manager.main_pool.stats["hit_tokens"] == 64
+    longer = PROMPT + OTHER
+    assert generate(eng, [longer])[0] == generate(engine(dtype=dtype), [longer])[0]
+    assert eng.manager.main_pool.stats["hit_tokens"] > 64
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_forced_preemption_does_not_change_the_output(dtype):
+    expected = generate(engine(dtype=dtype), [PROMPT], 24)[0]
+    tight = engine(dtype=dtype, num_blocks=11, max_running=4, max_model_len=176,
+                   debug_invariants=True)
+    crowd = [PROMPT] + [[(i * 37 + j) % 500 for j in range(80)] for i in range(3)]
+    got = generate(tight, crowd, 24)
+    assert tight.sched.stats["preemptions"] > 0
+    assert got[0] == expected
+
+
+def test_every_policy_produces_the_same_tokens():
+    prompts = [PROMPT, OTHER, PROMPT + [5] * 16]
+    base = generate(engine(policy="fcfs"), prompts)
+    for policy in ("lpm", "lpm_aging"):
+        assert generate(engine(policy=policy), prompts) == base
+
+
+def test_temperature_sampling_is_per_request_reproducible():
+    """(BASELINE configuration B: temperature 0.8 under a seeded generator.)  A request draws
+    the same tokens alone, in a batch and cut into portions of 16."""
+    folder = helpers.model_folder("B")
+    vocab = 1000
+    shared = helpers.random_tokens(vocab, 24, seed=99)
+    prompts = [helpers.random_tokens(vocab, 1, seed=1), helpers.random_tokens(vocab, 9, seed=2),
+               shared + helpers.random_tokens(vocab, 16, seed=3),
+               shared + helpers.random_tokens(vocab, 40, seed=4)]
+
+    def run(which, **kw):
+        from mercury_amd import SamplingParams
+
+        eng = engine("B", block_size=8, num_blocks=64, seed=5, **kw)
+        outs = {}
+        for i in which:
+            eng.submit(f"req{i}", prompts[i], 6, lambda e, i=i: outs.setdefault(i, []).append(e),
+                       params=SamplingParams(temperature=0.8, ignore_eos=True))
+        eng._drain_commands()
+        while eng.sched.has_work():
+            eng.step()
+        return {i: [e.token for e in ev if e.kind == "token"] for i, ev in outs.items()}
+
+    batched = run(range(4), prefill_budget=16)
+    for i in range(4):
+        assert run([i])[i] == batched[i]
+    assert len({tuple(v) for v in batched.values()}) == 4
+    other_seed = engine("B", block_size=8, num_blocks=64, seed=6)
+    from mercury_amd import SamplingParams
+    assert other_seed.generate([prompts[3]], SamplingParams(temperature=0.8), 6) != [batched[3]] \
+        or True  # a different seed may coincide on a peaked distribution; the run must succeed
+
+
+def test_command_line_generates_and_writes_random_weights(tmp_path):
+    config = tmp_path / "config.json"
+    config.write_text(json.dumps(helpers.TINY_A))
+    out = subprocess.run([sys.executable, "-m", "mercury_amd", "random-weights", "--config",
+                          str(config), "--out", str(tmp_path / "m"), "--seed", "3", "--std", "0.05"],
+                         capture_output=True, text=True, cwd=helpers.ROOT)
+    assert out.returncode == 0, out.stderr
+    prompt = [(i * 7) % 500 for i in range(20)]
+    run = subprocess.run([sys.executable, "-m", "mercury_amd", "generate", "--model",
+                          str(tmp_path / "m"), "--prompt-ids", ",".join(map(str, prompt)),
+                          "--prompt-ids", "1 2 3", "--max-tokens", "5", "--dtype", "float32",
+                          "--num-blocks", "32", "--max-model-len", "256", "--ignore-eos"],
+                         capture_output=True, text=True, cwd=helpers.ROOT)
+    assert run.returncode == 0, run.stderr
+    lines = [json.loads(line) for line in run.stdout.strip().splitlines()]
+    w, cfg = helpers.plain_model(tmp_path / "m")
+    assert lines[0] == {"prompt_index": 0, "tokens": plain.greedy_generate(w, cfg, prompt, 5)}
+    assert lines[1]["tokens"] == plain.greedy_generate(w, cfg, [1, 2, 3], 5)
+
+
+def test_smoke_entry_point():
+    import __graft_entry__
+
+    __graft_entry__.smoke()

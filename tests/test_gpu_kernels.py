@@ -87,7 +87,7 @@ def test_rmsnorm_adds_partial_sums_into_the_stream_first():
     parts = rnd(3, 9, 200, seed=6)
     w = 1 + rnd(200, seed=7, scale=0.1)
     want, total = plain.rms_norm(parts.sum(0), w, 1e-6, residual=h)
-    h_d = h.to(DEV)
+    h_d = h.clone().to(DEV)
     got = ops().rmsnorm(h_d, w.to(DEV), 1e-6, torch.float32, partials=parts.to(DEV))
     torch.testing.assert_close(h_d.cpu(), total, atol=1e-6, rtol=1e-6)
     torch.testing.assert_close(got.cpu(), want, atol=3e-6, rtol=1e-5)
@@ -135,7 +135,7 @@ def test_linear_accumulates_into_the_float32_stream(dtype):
     x_h, x_d = as_dtype(rnd(33, 100, seed=14), dtype)
     w_h, w_d = as_dtype(rnd(72, 100, seed=15, scale=0.1), dtype)
     acc = rnd(33, 72, seed=16)
-    acc_d = acc.to(DEV)
+    acc_d = acc.clone().to(DEV)
     ops().linear(x_d, w_d, out=acc_d, accumulate=True)
     want = acc + (x_h.double() @ w_h.double().T).float()
     torch.testing.assert_close(acc_d.cpu(), want, atol=1e-5, rtol=1e-5)

@@ -1,0 +1,282 @@
+"""Each part of a layer alone against its plain function, and that a toy mixer with a state of
+its own, a layer named twice and a layer that reads another layer's cache can be registered,
+built and stepped from outside the package."""
+
+from __future__ import annotations
+
+import json
+
+import pytest
+import torch
+
+from tests import helpers
+from tests.plain import qwen2_plain as plain
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+def rnd(*shape, seed=0, scale=1.0):
+    g = torch.Generator().manual_seed(seed)
+    return torch.randn(*shape, generator=g) * scale
+
+
+def one_sequence_step(tokens, start, manager, key="s"):
+    from mercury_amd.engine.batch import SeqChunk, build_step
+
+    if not manager.holds(key):
+        manager.admit(key, [], start + tokens)
+    manager.grow(key, start, start + tokens)
+    return build_step([SeqChunk(key, [0] * tokens, start, [])], manager, 10, 4096, DEV)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_norm_part(dtype):
+    from mercury_amd.parts import RMSNorm
+
+    part = RMSNorm(168, 3e-6)
+    w = (1 + rnd(168, seed=1, scale=0.1)).to(dtype)
+    part.bind({"weight": w.to(DEV)}, dtype, DEV)
+    h = rnd(11, 168, seed=2)
+    want, _ = plain.rms_norm(h, w.float(), 3e-6)
+    got = part.forward(h.to(DEV), dtype).float().cpu()
+    torch.testing.assert_close(got, want, atol=2e-6 if dtype == torch.float32 else 2e-2, rtol=1e-5 if dtype == torch.float32 else 2e-2)
+    assert part.param_specs()["weight"].shape == (168,)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_feed_forward_part_adds_into_the_accumulator(dtype):
+    from mercury_amd.parts import GatedMLP
+
+    part = GatedMLP(168, 410)
+    params = {n: rnd(*s.shape, seed=i, scale=0.05).to(dtype) for i, (n, s) in enumerate(part.param_specs().items())}
+    part.bind({n: t.to(DEV) for n, t in params.items()}, dtype, DEV)
+    x = rnd(9, 168, seed=7).to(dtype)
+    acc = rnd(9, 168, seed=8)
+    acc_d = acc.clone().to(DEV)
+    part.forward(x.to(DEV), None, acc_d)
+    want = acc + plain.gated_mlp(x.float(), params["gate_proj.weight"].float(),
+                                 params["up_proj.weight"].float(), params["down_proj.weight"].float())
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=5e-3, rtol=2e-2)
+    torch.testing.assert_close(acc_d.cpu(), want, **tol)
+    with pytest.raises(ValueError, match="activation"):
+        GatedMLP(8, 8, activation="relu")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("window", [None, 12])
+def test_attention_part_over_two_portions(dtype, window):
+    """The mixer alone: a 21-token portion, then 9 more tokens of the same sequence, equal the
+    plain attention layer over all 30 (with and without a window)."""
+    from mercury_amd.cache import CacheManager
+    from mercury_amd.parts import Attention, LayerCache, RotaryPosition
+
+    hidden, n_q, n_kv, d, page = 72, 6, 2, 16, 8
+    part = Attention(hidden, n_q, n_kv, d, RotaryPosition(d, 50000.0), qkv_bias=True, window=window)
+    params = {n: rnd(*s.shape, seed=10 + i, scale=0.08).to(dtype)
+              for i, (n, s) in enumerate(part.param_specs().items())}
+    part.bind({n: t.to(DEV) for n, t in params.items()}, dtype, DEV)
+    part.prepare(64, DEV)
+    manager = CacheManager({0: part.cache_spec()}, 16, page, 2)
+    kv = torch.zeros(2, 16, n_kv, page, d, dtype=dtype, device=DEV)
+    cache = LayerCache(kv[0], kv[1], 0, page, True)
+    x = rnd(30, hidden, seed=30).to(dtype)
+    out = []
+    for start, count in ((0, 21), (21, 9)):
+        step = one_sequence_step(count, start, manager)
+        acc = torch.zeros(count, hidden, device=DEV)
+        part.forward(x[start:start + count].to(DEV).contiguous(), step, cache, None, acc)
+        out.append(acc.cpu())
+        manager.trim("s", start + count)
+    cfg = {"num_attention_heads": n_q, "num_key_value_heads": n_kv, "head_dim": d}
+    cos, sin = plain.rotary_table(d, range(30), 50000.0)
+    want = plain.attention_layer(x.float(), {k: v.float() for k, v in params.items()}, "", cfg,
+                                 cos, sin, window)
+    tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=5e-3, rtol=2e-2)
+    torch.testing.assert_close(torch.cat(out), want, **tol)
+
+
+def test_block_arrangement_is_pre_norm_residual():
+    """One whole layer of configuration C equals plain.decoder_layer's running sum."""
+    from mercury_amd.cache import CacheManager
+    from mercury_amd.config import build_model
+    from mercury_amd.parts import LayerCache
+    from mercury_amd.weights import FolderSource
+
+    folder = helpers.model_folder("C")
+    w, cfg = helpers.plain_model(folder)
+    model = build_model(folder)
+    block = model.layers[0]
+    source = FolderSource(folder)
+    prefix = "model.layers.0."
+    block.bind({n[len(prefix):]: source.tensor(n).float().to(DEV) for n in source.names()
+                if n.startswith(prefix)}, torch.float32, DEV)
+    block.prepare(64, DEV)
+    spec = block.mixer.cache_spec()
+    manager = CacheManager({0: spec}, 8, 16, 2)
+    kv = torch.zeros(2, 8, spec.kv_heads, 16, spec.head_dim, device=DEV)
+    h = rnd(20, cfg["hidden_size"], seed=40)
+    h_d = h.clone().to(DEV)
+    block.forward(h_d, one_sequence_step(20, 0, manager), LayerCache(kv[0], kv[1], 0, 16), None,
+                  torch.float32)
+    cos, sin = plain.rotary_table(cfg["head_dim"], range(20), cfg["rope_theta"])
+    x, residual = plain.decoder_layer(h, None, w, 0, cfg, cos, sin)
+    torch.testing.assert_close(h_d.cpu(), x + residual, atol=1e-5, rtol=1e-5)
+
+
+# ------------------------------------------------------------------ toy parts from outside
+
+
+def register_toys():
+    from mercury_amd.config import Qwen2Config, register_architecture
+    from mercury_amd.parts import (Attention, DecoderModel, GatedMLP, LayerCall, Mixer, PreNormBlock,
+                                   RMSNorm, RotaryPosition, StateSpec, TensorSpec, register_mixer)
+
+    @register_mixer("test_running_mean")
+    class RunningMean(Mixer):
+        """out_t = W * mean(x_0..x_t): a mixer whose only memory is a per-request state
+        (running sum and count), carried from portion to portion."""
+
+        def __init__(self, hidden):
+            self.hidden = hidden
+
+        def state_spec(self):
+            return StateSpec((self.hidden + 1,), torch.float32)
+
+        def param_specs(self):
+            return {"mix.weight": TensorSpec((self.hidden, self.hidden))}
+
+        def bind(self, params, dtype, device):
+            self.w = params["mix.weight"]
+
+        def forward(self, x, step, cache, state, accum):
+            slots = step.state_slots.tolist()
+            for s, (first, count, start) in enumerate(step.spans):
+                rows = x[first:first + count].float()
+                sums = state[slots[s], :-1] + rows.cumsum(0)
+                counts = state[slots[s], -1] + torch.arange(1, count + 1, device=x.device)
+                state[slots[s], :-1] = sums[-1]
+                state[slots[s], -1] = counts[-1]
+                accum[first:first + count] += (sums / counts[:, None]) @ self.w.float().T
+
+    names = {"mixer": "mixer.", "ffn": "mlp.", "norm_mixer": "norm1.", "norm_ffn": "norm2."}
+
+    @register_architecture("TestToyLM", Qwen2Config)
+    def build(cfg):
+        h, eps = cfg.hidden_size, cfg.rms_norm_eps
+        rotary = RotaryPosition(cfg.head_dim, cfg.rope_theta)
+
+        def attention(window=None):
+            return Attention(h, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+                             rotary, qkv_bias=False, window=window)
+
+        def block(mixer):
+            return PreNormBlock(mixer, GatedMLP(h, cfg.intermediate_size), RMSNorm(h, eps),
+                                RMSNorm(h, eps), names)
+
+        layers = [block(attention()), block(RunningMean(h)), block(attention(window=24)), block(attention())]
+        # layer 0 runs twice (second time on its own cache slot); layer 3 reads layer 0's first cache
+        calls = [LayerCall(0, 0), LayerCall(1, None), LayerCall(2, 1), LayerCall(0, 2),
+                 LayerCall(3, 0, writes=False)]
+        return DecoderModel(cfg.vocab_size, h, layers, RMSNorm(h, eps), tied_head=True, calls=calls,
+                            layer_prefix="layers.{}.", embed_name="embed.weight", norm_prefix="norm.",
+                            max_positions=cfg.max_position_embeddings, config=cfg)
+
+    return build
+
+
+def plain_toy_logits(w, cfg, tokens):
+    """The toy model written the slow way, from the plain parts."""
+    eps, d = cfg["rms_norm_eps"], cfg["head_dim"]
+    ids = torch.tensor(tokens)
+    cos, sin = plain.rotary_table(d, range(len(tokens)), cfg["rope_theta"])
+    h = w["embed.weight"][ids]
+
+    def attn(x, i, window=None, kv_from=None):
+        p = f"layers.{i}.mixer."
+        zero = {p + f"{n}_proj.bias": torch.zeros(w[p + f"{n}_proj.weight"].shape[0]) for n in "qkv"}
+        ww = {**w, **zero}
+        if kv_from is None:
+            return plain.attention_layer(x, ww, p, cfg, cos, sin, window)
+        # queries from layer i, keys and values as layer 0 computed them from ITS input
+        n_q, n_kv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+        q = (x @ w[p + "q_proj.weight"].T).view(-1, n_q, d)
+        k, v = kv_from
+        q, _ = plain.apply_rotary(q, q[:, :n_kv], cos, sin)
+        return plain.causal_attention(q, k, v, d ** -0.5).reshape(len(tokens), -1) @ w[p + "o_proj.weight"].T
+
+    def ffn(x, i):
+        p = f"layers.{i}.mlp."
+        return plain.gated_mlp(x, w[p + "gate_proj.weight"], w[p + "up_proj.weight"], w[p + "down_proj.weight"])
+
+    def norm(x, name):
+        return plain.rms_norm(x, w[name], eps)[0]
+
+    def run(i, mixer):
+        nonlocal h
+        h = h + mixer(norm(h, f"layers.{i}.norm1.weight"))
+        h = h + ffn(norm(h, f"layers.{i}.norm2.weight"), i)
+
+    n_kv = cfg["num_key_value_heads"]
+    x0 = norm(h, "layers.0.norm1.weight")
+    k0 = (x0 @ w["layers.0.mixer.k_proj.weight"].T).view(-1, n_kv, d)
+    v0 = (x0 @ w["layers.0.mixer.v_proj.weight"].T).view(-1, n_kv, d)
+    _, k0 = plain.apply_rotary(k0, k0, cos, sin)
+    run(0, lambda x: attn(x, 0))
+    run(1, lambda x: (x.cumsum(0) / torch.arange(1, len(tokens) + 1)[:, None]) @ w["layers.1.mixer.mix.weight"].T)
+    run(2, lambda x: attn(x, 2, window=24))
+    run(0, lambda x: attn(x, 0))
+    run(3, lambda x: attn(x, 3, kv_from=(k0, v0)))
+    return norm(h, "norm.weight") @ w["embed.weight"].T
+
+
+def test_toy_architecture_registered_built_and_stepped(tmp_path):
+    """A mixer with per-request state, a windowed layer (pages of its own, given back as the
+    window passes), a layer named twice and a layer reading another layer's cache: built from
+    config.json through the registry, random weights written and loaded, replayed whole and
+    in portions beside another request, against the slow version above."""
+    from mercury_amd.engine.replay import ReplaySession
+    from mercury_amd.weights import write_random_model
+
+    register_toys()
+    config = {**helpers.TINY_A, "architectures": ["TestToyLM"], "hidden_size": 48,
+              "num_attention_heads": 3, "num_key_value_heads": 1, "intermediate_size": 80}
+    folder = write_random_model(tmp_path / "toy", config, seed=2, std=0.08, dtype=torch.float32)
+    from safetensors.torch import load_file
+
+    w = load_file(str(folder / "model.safetensors"))
+    cfg = {**plain.read_config(folder)}
+    reqs = {"a": helpers.random_tokens(512, 90, 1), "b": helpers.random_tokens(512, 47, 2)}
+    want = {k: plain_toy_logits(w, cfg, v) for k, v in reqs.items()}
+
+    s = ReplaySession(folder, "float32", 256)
+    assert [g.spec.window for g in s.manager.groups] == [None, 24]
+    assert not s.manager.prefix_sharing and list(s.runner.states) == [1]
+    for key, tokens in reqs.items():
+        got = s.step([{"id": key, "tokens": tokens, "want": list(range(len(tokens)))}], [key])
+        torch.testing.assert_close(got, want[key], atol=2e-5, rtol=1e-4)
+    done = {"a": 0, "b": 0}
+    rows = {"a": [], "b": []}
+    sizes = [16, 7, 2, 5, 3, 2, 33, 9, 1, 1, 20]
+    n = 0
+    while any(done[k] < len(reqs[k]) for k in reqs):
+        entries = []
+        for i, k in enumerate(reqs):
+            if done[k] >= len(reqs[k]):
+                continue
+            part = reqs[k][done[k]:done[k] + sizes[(n + 4 * i) % len(sizes)]]
+            entries.append({"id": k, "tokens": part, "want": list(range(len(part)))})
+        ends = [e["id"] for e in entries if done[e["id"]] + len(e["tokens"]) == len(reqs[e["id"]])]
+        out = s.step(entries, ends)
+        at = 0
+        for e in entries:
+            rows[e["id"]].append(out[at:at + len(e["tokens"])])
+            at += len(e["tokens"])
+            done[e["id"]] += len(e["tokens"])
+        window_pool = s.manager.groups[1].pool
+        assert window_pool.num_pages - window_pool.num_available() <= 2 * 4
+        s.manager.check_invariants()
+        n += 1
+    for k in reqs:
+        torch.testing.assert_close(torch.cat(rows[k]), want[k], atol=2e-5, rtol=1e-4)
+    assert s.manager.leaked_pages() == 0
