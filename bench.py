@@ -1,0 +1,231 @@
+"""Decode and prefill throughput of the engine on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--batch 8] [--layers L]
+
+A "step" is one decode step of the whole engine (schedule, run the batch through the model from
+the cache, sample), at the layer sizes of Qwen2.5-0.5B with random weights, synthetic uniform
+random token ids, a batch of 8 and a context that reaches 4,096 tokens at the last timed step.
+One JSON line is printed: `value` is decoded tokens per second; `prefill` times one 2,048-token
+prompt as one step; `roofline` divides the bytes a decode step has to read (every weight it
+uses once, and the cache of the live requests) by its time and by the HBM peak; `points`
+holds decode throughput at batch 1 and 64.
+"""
+
+from __future__ import annotations
+
+import argparse
+import json
+import statistics
+import sys
+import time
+from pathlib import Path
+
+ROOT = Path(__file__).resolve().parent
+if str(ROOT) not in sys.path:
+    sys.path.insert(0, str(ROOT))
+
+# Qwen2.5-0.5B layer sizes (the model this benchmark names).
+QWEN25_05B = {
+    "architectures": ["Qwen2ForCausalLM"], "model_type": "qwen2",
+    "hidden_size": 896, "intermediate_size": 4864, "num_hidden_layers": 24,
+    "num_attention_heads": 14, "num_key_value_heads": 2, "head_dim": 64,
+    "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
+    "tie_word_embeddings": True, "max_position_embeddings": 32768,
+}
+CONTEXT = 4096
+PREFILL_TOKENS = 2048
+BLOCK_SIZE = 16
+PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
+PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
+
+
+def parse_args(argv=None):
+    p = argparse.ArgumentParser()
+    p.add_argument("--gpus", type=int, default=1)
+    p.add_argument("--steps", type=int, default=64)
+    p.add_argument("--warmup", type=int, default=8)
+    p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
+    p.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
+    p.add_argument("--context", type=int, default=CONTEXT)
+    p.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 runs")
+    p.add_argument("--seed", type=int, default=0)
+    return p.parse_args(argv)
+
+
+def prefill_flops(cfg: dict, tokens: int) -> float:
+    """Multiply-adds times two of one whole-prompt step: the projections of every layer for
+    every token, causal attention (scores and weighted sum), and the head for one row."""
+    h, i = cfg["hidden_size"], cfg["intermediate_size"]
+    n_q, n_kv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    linear = 2.0 * (h * (n_q + 2 * n_kv) * d + n_q * d * h + 3 * h * i)
+    attention = 4.0 * n_q * d * tokens * (tokens + 1) / 2
+    layers = cfg["num_hidden_layers"]
+    return layers * (linear * tokens + attention) + 2.0 * h * cfg["vocab_size"]
+
+
+class Bench:
+    def __init__(self, cfg: dict, dtype: str, max_batch: int, context: int, seed: int):
+        import torch
+
+        from mercury_amd.cache import CacheManager, PageHasher
+        from mercury_amd.config import EngineConfig, build_model
+        from mercury_amd.engine.engine import Engine
+        from mercury_amd.engine.executor import GpuExecutor
+        from mercury_amd.engine.runner import ModelRunner
+        from mercury_amd.sampling import Sampler
+        from mercury_amd.weights import DictSource, load_weights, random_state
+
+        self.torch = torch
+        self.cfg = cfg
+        device = torch.device("cuda:0")
+        t0 = time.time()
+        model = build_model(cfg)
+        torch_dtype = torch.bfloat16 if dtype == "bfloat16" else torch.float32
+        state = random_state(model, seed, std=0.02, dtype=torch_dtype)
+        load_weights(model, DictSource(state), torch_dtype, device)
+        del state
+        pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + PREFILL_TOKENS // BLOCK_SIZE + 8
+        self.engine_cfg = EngineConfig(
+            model="random", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
+            max_running=max_batch + 1, prefill_budget=8192, max_model_len=context + 128, seed=seed)
+        manager = CacheManager(model.cache_slots, pages, BLOCK_SIZE, max_batch + 1, False)
+        runner = ModelRunner(model, manager, torch_dtype, device, context + 128)
+        self.engine = Engine(self.engine_cfg, executor=GpuExecutor(runner, Sampler(seed)),
+                             manager=manager, eos_token_ids=())
+        self.model, self.runner, self.manager = model, runner, manager
+        self.rng = torch.Generator().manual_seed(seed)
+        self.counter = 0
+        print(f"[bench] model ready in {time.time() - t0:.1f} s: "
+              f"{model.decode_weight_bytes() / 1e9:.3f} GB of weights a step reads, "
+              f"{pages} pages", file=sys.stderr, flush=True)
+
+    def tokens(self, count: int) -> list:
+        return self.torch.randint(0, self.cfg["vocab_size"], (count,), generator=self.rng).tolist()
+
+    def sync(self):
+        self.torch.cuda.synchronize()
+
+    def decode(self, batch: int, context: int, steps: int, warmup: int) -> dict:
+        """Time `steps` decode steps of `batch` requests whose context reaches `context` at
+        the last timed step."""
+        from mercury_amd import SamplingParams
+
+        prompt_len = context - steps - warmup
+        rids = []
+        for _ in range(batch):
+            rid = f"bench-{self.counter}"
+            self.counter += 1
+            self.engine.submit(rid, self.tokens(prompt_len), steps + warmup + batch + 8, lambda e: None,
+                               params=SamplingParams(ignore_eos=True))
+            rids.append(rid)
+        self.engine._drain_commands()
+        t0 = time.time()
+        while any(r.remaining > 1 for r in self.engine.sched.running) or self.engine.sched.waiting:
+            self.engine.step()          # prompts, in portions under the token budget
+        self.sync()
+        fill_s = time.time() - t0
+        assert len(self.engine.sched.running) == batch
+        for _ in range(warmup):
+            self.engine.step()
+        self.sync()
+        start = time.perf_counter()
+        for _ in range(steps):
+            record = self.engine.step()
+            assert record.num_decode == batch and record.num_prefill == 0
+        self.sync()
+        elapsed = time.perf_counter() - start
+        kv_tokens = sum(r.num_computed for r in self.engine.sched.running)
+        kv_bytes = kv_tokens * self.runner.kv_bytes_per_token()
+        for rid in rids:
+            self.engine.abort(rid)
+        self.engine._drain_commands()
+        assert self.engine.leaked_blocks() == 0
+        ms = 1e3 * elapsed / steps
+        return {"tok_s": batch * steps / elapsed, "ms": ms, "fill_s": fill_s,
+                "bytes": self.model.decode_weight_bytes() + kv_bytes}
+
+    def prefill(self, tokens: int, repeats: int = 5) -> dict:
+        from mercury_amd import SamplingParams
+
+        times = []
+        for _ in range(repeats + 1):
+            rid = f"bench-{self.counter}"
+            self.counter += 1
+            self.engine.submit(rid, self.tokens(tokens), 1, lambda e: None,
+                               params=SamplingParams(ignore_eos=True))
+            self.sync()
+            start = time.perf_counter()
+            record = self.engine.step()
+            self.sync()
+            times.append(time.perf_counter() - start)
+            assert record.prefill_tokens == tokens and not self.engine.sched.has_work()
+        seconds = statistics.median(times[1:])
+        return {"tok_s": tokens / seconds, "ms": 1e3 * seconds}
+
+
+def main(argv=None) -> int:
+    args = parse_args(argv)
+    if args.gpus != 1:
+        print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine "
+              "has no multi-GPU path)")
+        return 2
+    cfg = dict(QWEN25_05B)
+    full_layers = cfg["num_hidden_layers"]
+    if args.layers:
+        cfg["num_hidden_layers"] = args.layers
+    max_batch = args.batch if args.no_points else max(args.batch, 64)
+    bench = Bench(cfg, args.dtype, max_batch, args.context, args.seed)
+
+    main_run = bench.decode(args.batch, args.context, args.steps, args.warmup)
+    print(f"[bench] decode b{args.batch}: {main_run['ms']:.3f} ms/step "
+          f"(cache filled in {main_run['fill_s']:.1f} s)", file=sys.stderr, flush=True)
+    pre = bench.prefill(PREFILL_TOKENS)
+    print(f"[bench] prefill {PREFILL_TOKENS}: {pre['ms']:.2f} ms", file=sys.stderr, flush=True)
+    points = {}
+    if not args.no_points:
+        for b in (1, 64):
+            steps = max(8, args.steps // 2)
+            run = bench.decode(b, args.context, steps, min(args.warmup, 4))
+            points[f"decode_b{b}"] = round(run["tok_s"], 1)
+            print(f"[bench] decode b{b}: {run['ms']:.3f} ms/step", file=sys.stderr, flush=True)
+
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    achieved = main_run["bytes"] / (main_run["ms"] * 1e-3) / 1e9
+    line = {
+        "metric": "decode tok/s at batch 8, context 4096 (Qwen2.5-0.5B shapes)",
+        "value": round(main_run["tok_s"], 1),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(main_run["ms"], 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": short,
+        "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
+        "config": {
+            "model": "Qwen2.5-0.5B shapes", "layers": cfg["num_hidden_layers"],
+            "layers_full": full_layers, "hidden": cfg["hidden_size"],
+            "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
+            "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"],
+            "vocab": cfg["vocab_size"], "tied_embeddings": cfg["tie_word_embeddings"],
+            "global_batch": args.batch, "seq_len": args.context,
+            "prompt_len": args.context - args.steps - args.warmup, "block_size": BLOCK_SIZE,
+            "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
+        },
+        "prefill": {"value": round(pre["tok_s"], 1), "tokens": PREFILL_TOKENS,
+                    "ms": round(pre["ms"], 3),
+                    "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / (pre["ms"] * 1e-3)
+                                  / PEAK_FLOPS[short], 5)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 5)},
+        "points": points,
+    }
+    print(json.dumps(line), flush=True)
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -3,9 +3,10 @@
 // This kernel serves the true 32-bit path and every head size the matrix-core kernels do not
 // cover.  It makes no distinction between a prompt portion and a decoded token: a query at
 // absolute position p of its sequence reads the keys [first, p] of that sequence from the
-// cache, first being 0 or p - window + 1.  Keys are walked in ascending chunks of 64 from
-// `first`, so the order of every sum depends on the query's own position only, not on how
-// the sequence was cut into steps or on what else is in the batch.
+// cache, first being 0 or p - window + 1.  Keys lie as [page, kv head, slot, dim], values
+// transposed within the page as [page, kv head, dim, slot].  Keys are walked in ascending
+// chunks of 64 from `first`, so the order of every sum depends on the query's own position
+// only, not on how the sequence was cut into steps or on what else is in the batch.
 //
 // Scores, softmax and the weighted sum are float32 (reference formulas:
 // mercury/model/attention.py:9-32 and :87-101, scale = head_dim^-0.5 passed by the caller).
@@ -63,13 +64,15 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     for (int jj = 0; jj < count; ++jj) {
       const int key = j0 + jj;
       const int page = table[key >> page_shift];
-      const T* vrow =
-          v_cache + (((size_t)page * n_kv + kvh) * page_size + (key & page_mask)) * d;
+      // values are stored transposed within a page: [page, kv head, dim, slot]
+      const T* vcol =
+          v_cache + ((size_t)page * n_kv + kvh) * page_size * d + (key & page_mask);
       const float pj = probs[jj];
 #pragma unroll
       for (int c = 0; c < AG_MAX_D / MK_WAVE; ++c) {
         const int dim = lane + c * MK_WAVE;
-        if (dim < d) acc[c] = fmaf(pj, Elem<T>::load(vrow + dim), acc[c]);
+        if (dim < d)
+          acc[c] = fmaf(pj, Elem<T>::load(vcol + (size_t)dim * page_size), acc[c]);
       }
     }
     m = m_new;

@@ -176,8 +176,9 @@ extern "C" int mk_silu_mul(const void* gate_up, void* out, int dtype, int tokens
 //   y[j]         = x[j] * cos - x[j + rot/2] * sin
 //   y[j + rot/2] = x[j + rot/2] * cos + x[j] * sin
 // (reference: mercury/model/rope.py:6-17).  cos/sin are float32 tables [positions, rot/2].
-// q is rotated in place; rotated k and raw v go to the token's slot of the paged cache
-// [pages, n_kv, page_size, d], the page taken from the sequence's block table
+// q is rotated in place; rotated k and raw v go to the token's slot of the paged cache, keys
+// as [pages, n_kv, page_size, d] and values transposed within the page as
+// [pages, n_kv, d, page_size], the page taken from the sequence's block table
 // (reference: mercury/runner.py:32-34, mercury/model/attention.py:35-45).
 template <typename T>
 __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
@@ -227,7 +228,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
       y = Elem<T>::load(x + j);
     }
     Elem<T>::store(k_cache + dst, y);
-    v_cache[dst] = v_src[head * d + j];
+    v_cache[(((size_t)page * n_kv + head) * d + j) * page_size + off] = v_src[head * d + j];
   }
 }
 

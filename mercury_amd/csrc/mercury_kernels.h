@@ -31,7 +31,8 @@ int mk_silu_mul(const void* gate_up, void* out, int dtype, int tokens, int inter
                 hipStream_t stream);
 
 // Rotary encoding of the q and k heads of qkv [T, row_stride] (q in place) and the write of
-// rotated k and raw v into the paged cache [pages, n_kv, page_size, d].
+// rotated k into the paged key cache [pages, n_kv, page_size, d] and of raw v into the value
+// cache, which is transposed within a page: [pages, n_kv, d, page_size].
 int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const float* cos_table,
                      const float* sin_table, int table_positions, const int* positions,
                      const int* token_seq, const int* block_table, int table_stride,

@@ -34,20 +34,22 @@ class ModelRunner:
         self.page_size = manager.page_size
         model.prepare(self.max_model_len, device)
 
-        # Paged keys and values: one [2, pages, kv_heads, page_size, head_dim] tensor per slot.
+        # Paged keys [pages, kv_heads, page, head_dim] and values [pages, kv_heads, head_dim,
+        # page] per cache slot.
         self.kv = {}
         for slot, spec in model.cache_slots.items():
             group = manager.group_of_slot[slot]
             pages = manager.groups[group].pool.num_pages
-            self.kv[slot] = torch.zeros(
-                (2, pages, spec.kv_heads, self.page_size, spec.head_dim), dtype=dtype, device=device)
+            self.kv[slot] = (
+                torch.zeros((pages, spec.kv_heads, self.page_size, spec.head_dim), dtype=dtype, device=device),
+                torch.zeros((pages, spec.kv_heads, spec.head_dim, self.page_size), dtype=dtype, device=device))
         self.caches = {}
         for n, call in enumerate(model.calls):
             if call.cache is None:
                 continue
-            kv = self.kv[call.cache]
-            self.caches[n] = LayerCache(kv[0], kv[1], manager.group_of_slot[call.cache],
-                                        self.page_size, call.writes)
+            k, v = self.kv[call.cache]
+            self.caches[n] = LayerCache(k, v, manager.group_of_slot[call.cache], self.page_size,
+                                        call.writes)
         # Per-request state of fixed size, one tensor per layer that declares it.
         self.states = {}
         for i, layer in enumerate(model.layers):
@@ -58,10 +60,10 @@ class ModelRunner:
 
     @property
     def kv_bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for t in self.kv.values())
+        return sum(t.numel() * t.element_size() for kv in self.kv.values() for t in kv)
 
     def kv_bytes_per_token(self) -> int:
-        return sum(2 * t.shape[2] * t.shape[4] * t.element_size() for t in self.kv.values())
+        return sum(2 * k.shape[1] * k.shape[3] * k.element_size() for k, _ in self.kv.values())
 
     def build(self, chunks: list) -> StepContext:
         return build_step(chunks, self.manager, self.model.vocab_size, self.max_model_len,

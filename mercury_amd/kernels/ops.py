@@ -162,12 +162,27 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
 # ---------------------------------------------------------------------- positions and the cache
 
 
+def _check_caches(what, k_cache, v_cache, n_kv, head_dim, dtype) -> int:
+    """Keys [pages, n_kv, page, d]; values transposed in the page [pages, n_kv, d, page]."""
+    if k_cache is None or v_cache is None or k_cache.dim() != 4 or v_cache.dim() != 4:
+        raise KernelArgumentError(f"{what}: 4-dimensional key and value caches are required")
+    pages, heads, page_size, d = k_cache.shape
+    if heads != n_kv or d != head_dim or tuple(v_cache.shape) != (pages, n_kv, head_dim, page_size):
+        raise KernelArgumentError(
+            f"{what}: caches {tuple(k_cache.shape)} / {tuple(v_cache.shape)} are not "
+            f"[pages, {n_kv}, page, {head_dim}] / [pages, {n_kv}, {head_dim}, page]")
+    if k_cache.dtype != dtype or v_cache.dtype != dtype:
+        raise KernelArgumentError(f"{what}: cache dtype differs from the activations'")
+    return page_size
+
+
 def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
                   positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                   k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, n_q: int,
                   n_kv: int, head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
-    """Rotate q (in place) and k by their absolute positions; write k and v into the paged
-    cache [pages, n_kv, page_size, head_dim] at the slots the block table gives."""
+    """Rotate q (in place) and k by their absolute positions; write k into the paged key
+    cache [pages, n_kv, page_size, head_dim] and v into the value cache
+    [pages, n_kv, head_dim, page_size] at the slots the block table gives."""
     _dev(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache)
     _i32(positions, "positions")
     _i32(token_seq, "token_seq")
@@ -185,14 +200,7 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor
         table_positions = cos.shape[0]
     page_size = 1
     if write_kv:
-        if k_cache is None or v_cache is None or k_cache.shape != v_cache.shape:
-            raise KernelArgumentError("rope: k and v caches of equal shape are required")
-        if k_cache.dtype != qkv.dtype or v_cache.dtype != qkv.dtype:
-            raise KernelArgumentError("rope: cache dtype differs from the activations'")
-        if k_cache.dim() != 4 or k_cache.shape[1] != n_kv or k_cache.shape[3] != head_dim:
-            raise KernelArgumentError(
-                f"rope: cache {tuple(k_cache.shape)} is not [pages, {n_kv}, page, {head_dim}]")
-        page_size = k_cache.shape[2]
+        page_size = _check_caches("rope", k_cache, v_cache, n_kv, head_dim, qkv.dtype)
     lib = _lib.load("core")
     _lib.check(lib, lib.mk_rope_kv_write(
         _ptr(qkv), dtype_code(qkv.dtype), row, _ptr(cos), _ptr(sin), table_positions,
@@ -215,19 +223,14 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     tokens = positions.shape[0]
     if q.numel() < (tokens - 1) * q_stride + n_q * head_dim and tokens:
         raise KernelArgumentError("attention: q buffer too small")
-    if k_cache.dim() != 4 or k_cache.shape != v_cache.shape or k_cache.shape[1] != n_kv \
-            or k_cache.shape[3] != head_dim:
-        raise KernelArgumentError(
-            f"attention: cache {tuple(k_cache.shape)} is not [pages, {n_kv}, page, {head_dim}]")
-    if k_cache.dtype != q.dtype:
-        raise KernelArgumentError("attention: cache dtype differs from q's")
+    page_size = _check_caches("attention", k_cache, v_cache, n_kv, head_dim, q.dtype)
     if out is None:
         out = torch.empty((tokens, n_q * head_dim), dtype=q.dtype, device=q.device)
     lib = _lib.load("core")
     _lib.check(lib, lib.mk_attention_generic(
         _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
         dtype_code(q.dtype), _ptr(positions), _ptr(token_seq), _ptr(block_table),
-        block_table.shape[1], k_cache.shape[2], n_q, n_kv, head_dim, float(scale),
+        block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
         int(window or 0), tokens, _stream()), "attention")
     return out
 

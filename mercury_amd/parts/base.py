@@ -80,7 +80,9 @@ class StateSpec:
 class LayerCache:
     """The paged keys and values one execution-list entry works on.
 
-    k, v: [pages, kv_heads, page_size, head_dim].  `group` indexes the step's block tables.
+    k: [pages, kv_heads, page_size, head_dim]; v: [pages, kv_heads, head_dim, page_size]
+    (values lie transposed within a page, which is how the matrix-core attention kernels
+    read them).  `group` indexes the step's block tables.
     `writes` is false when the entry only reads a cache another entry fills.
     """
 

@@ -168,13 +168,14 @@ def rotary_tables(d, theta, positions):
     return cos[:, : d // 2].contiguous(), sin[:, : d // 2].contiguous()
 
 
-def paged(kv, pages, page_size, num_pages, dtype):
-    """Host helper: lay [S, n_kv, d] out in a cache [num_pages, n_kv, page, d]."""
+def paged(kv, pages, page_size, num_pages, dtype, transposed=False):
+    """Host helper: lay [S, n_kv, d] out in a key cache [num_pages, n_kv, page, d] or, with
+    `transposed`, a value cache [num_pages, n_kv, d, page]."""
     s, n_kv, d = kv.shape
     cache = torch.zeros(num_pages, n_kv, page_size, d, dtype=dtype)
     for p in range(s):
         cache[pages[p // page_size], :, p % page_size, :] = kv[p].to(dtype)
-    return cache
+    return cache.transpose(2, 3).contiguous() if transposed else cache
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
@@ -191,7 +192,7 @@ def test_rope_and_cache_write(dtype, n_q, n_kv, d, page):
     tokens = len(positions)
     qkv_h, qkv_d = as_dtype(rnd(tokens, (n_q + 2 * n_kv) * d, seed=20), dtype)
     k_cache = torch.zeros(40, n_kv, page, d, dtype=dtype, device=DEV)
-    v_cache = torch.zeros_like(k_cache)
+    v_cache = torch.zeros(40, n_kv, d, page, dtype=dtype, device=DEV)
     ops().rope_kv_write(qkv_d, cos.to(DEV), sin.to(DEV),
                         torch.tensor(positions, dtype=torch.int32, device=DEV),
                         torch.tensor(token_seq, dtype=torch.int32, device=DEV), table.to(DEV),
@@ -207,11 +208,11 @@ def test_rope_and_cache_write(dtype, n_q, n_kv, d, page):
         pg, off = int(table[s, p // page]), p % page
         assert plain.slot_mapping(table[s].tolist(), p, p + 1, page) == [pg * page + off]
         torch.testing.assert_close(k_cache[pg, :, off].float().cpu(), k_want[t], **tol(dtype))
-        assert torch.equal(v_cache[pg, :, off].float().cpu(), v[t])
+        assert torch.equal(v_cache[pg, :, :, off].float().cpu(), v[t])
         touched[pg, off] = True
     untouched = ~touched[:, None, :, None].expand(40, n_kv, page, d)
     assert torch.count_nonzero(k_cache.cpu()[untouched]) == 0
-    assert torch.count_nonzero(v_cache.cpu()[untouched]) == 0
+    assert torch.count_nonzero(v_cache.cpu().transpose(2, 3)[untouched]) == 0
 
 
 def test_rotary_pairing_sign_and_identity_at_zero():
@@ -278,6 +279,7 @@ def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens
         positions += list(range(seq_lens[s] - q_lens[s], seq_lens[s]))
         token_seq += [s] * q_lens[s]
     q_flat = torch.cat([q.reshape(q.shape[0], n_q * d) for q in q_h]).to(dtype).to(DEV)
+    v_cache = v_cache.transpose(2, 3).contiguous()      # values lie transposed within a page
     out = ops().attention(q_flat, n_q * d, k_cache.to(DEV), v_cache.to(DEV),
                           torch.tensor(positions, dtype=torch.int32, device=DEV),
                           torch.tensor(token_seq, dtype=torch.int32, device=DEV), table.to(DEV),
@@ -378,7 +380,7 @@ def test_attention_window_edge(dtype, window):
     # hide the pages afterwards
     n_qh = q[-q_len:]
     k_cache = paged(k, pages, page, 32, dtype)
-    v_cache = paged(v, pages, page, 32, dtype)
+    v_cache = paged(v, pages, page, 32, dtype, transposed=True)
     for g in range(gone):
         k_cache[pages[g]] = 1e4
         v_cache[pages[g]] = 1e4

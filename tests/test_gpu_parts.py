@@ -78,8 +78,8 @@ def test_attention_part_over_two_portions(dtype, window):
     part.bind({n: t.to(DEV) for n, t in params.items()}, dtype, DEV)
     part.prepare(64, DEV)
     manager = CacheManager({0: part.cache_spec()}, 16, page, 2)
-    kv = torch.zeros(2, 16, n_kv, page, d, dtype=dtype, device=DEV)
-    cache = LayerCache(kv[0], kv[1], 0, page, True)
+    cache = LayerCache(torch.zeros(16, n_kv, page, d, dtype=dtype, device=DEV),
+                       torch.zeros(16, n_kv, d, page, dtype=dtype, device=DEV), 0, page, True)
     x = rnd(30, hidden, seed=30).to(dtype)
     out = []
     for start, count in ((0, 21), (21, 9)):
@@ -114,10 +114,11 @@ def test_block_arrangement_is_pre_norm_residual():
     block.prepare(64, DEV)
     spec = block.mixer.cache_spec()
     manager = CacheManager({0: spec}, 8, 16, 2)
-    kv = torch.zeros(2, 8, spec.kv_heads, 16, spec.head_dim, device=DEV)
+    k_pages = torch.zeros(8, spec.kv_heads, 16, spec.head_dim, device=DEV)
+    v_pages = torch.zeros(8, spec.kv_heads, spec.head_dim, 16, device=DEV)
     h = rnd(20, cfg["hidden_size"], seed=40)
     h_d = h.clone().to(DEV)
-    block.forward(h_d, one_sequence_step(20, 0, manager), LayerCache(kv[0], kv[1], 0, 16), None,
+    block.forward(h_d, one_sequence_step(20, 0, manager), LayerCache(k_pages, v_pages, 0, 16), None,
                   torch.float32)
     cos, sin = plain.rotary_table(cfg["head_dim"], range(20), cfg["rope_theta"])
     x, residual = plain.decoder_layer(h, None, w, 0, cfg, cos, sin)
