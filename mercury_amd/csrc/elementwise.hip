@@ -4,26 +4,6 @@
 #include "common.h"
 #include "mercury_kernels.h"
 
-#include <stdarg.h>
-#include <string>
-
-// ---------------------------------------------------------------------------------- errors
-
-static thread_local std::string g_last_error;
-
-void mk_set_error(const char* fmt, ...) {
-  char buf[1024];
-  va_list ap;
-  va_start(ap, fmt);
-  vsnprintf(buf, sizeof(buf), fmt, ap);
-  va_end(ap);
-  g_last_error = buf;
-}
-
-extern "C" const char* mk_last_error() { return g_last_error.c_str(); }
-
-extern "C" int mk_abi_version() { return MK_ABI_VERSION; }
-
 // ------------------------------------------------------------------------------- embedding
 
 template <typename T>
@@ -260,5 +240,143 @@ extern "C" int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const floa
   else
     MK_REQUIRE(false, "rope: unknown dtype %d", dtype);
   MK_LAUNCH_CHECK("rope_kv_write");
+  return 0;
+}
+
+// ------------------------------------------ consumers of split-K partial sums (decode path)
+
+// SiLU gating of a projection that arrives as `num_partials` float32 slices [p, T, 2I].
+template <typename T>
+__global__ void silu_mul_partials_kernel(const float* __restrict__ partials, int num_partials,
+                                         size_t partial_stride, T* __restrict__ out, int inter,
+                                         size_t total) {
+  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
+       idx += (size_t)gridDim.x * blockDim.x) {
+    const size_t t = idx / inter;
+    const int i = (int)(idx - t * inter);
+    const float* row = partials + t * 2 * (size_t)inter;
+    float g = 0.f, u = 0.f;
+    for (int p = 0; p < num_partials; ++p) {
+      g += row[p * partial_stride + i];
+      u += row[p * partial_stride + inter + i];
+    }
+    // The reference rounds both projections to the storage type before gating.
+    g = Elem<T>::round(g);
+    u = Elem<T>::round(u);
+    const float s = Elem<T>::round(g / (1.f + expf(-g)));
+    Elem<T>::store(out + idx, s * u);
+  }
+}
+
+extern "C" int mk_silu_mul_partials(const float* partials, int num_partials,
+                                    long long partial_stride, void* out, int out_dtype,
+                                    int tokens, int inter, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && inter > 0 && num_partials >= 1, "silu_mul: bad sizes");
+  if (tokens == 0) return 0;
+  const size_t total = (size_t)tokens * inter;
+  size_t blocks = (total + 255) / 256;
+  if (blocks > 65536) blocks = 65536;
+  if (out_dtype == MK_BF16)
+    silu_mul_partials_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>(
+        partials, num_partials, (size_t)partial_stride, (bf16_t*)out, inter, total);
+  else if (out_dtype == MK_F32)
+    silu_mul_partials_kernel<float><<<(int)blocks, 256, 0, stream>>>(
+        partials, num_partials, (size_t)partial_stride, (float*)out, inter, total);
+  else
+    MK_REQUIRE(false, "silu_mul: unknown dtype %d", out_dtype);
+  MK_LAUNCH_CHECK("silu_mul_partials");
+  return 0;
+}
+
+// The q/k/v projection arrives as float32 slices [p, T, (n_q + 2 n_kv) d]; this adds them up,
+// adds the bias, rotates q and k, writes q [T, n_q d] and the cache.  Sums and rotation are
+// float32; q, k and v are rounded to the storage type first, as a stored projection would be.
+template <typename T, typename TB>
+__global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_partials,
+                                  size_t partial_stride, const TB* __restrict__ bias,
+                                  T* __restrict__ q_out, const float* __restrict__ cos_table,
+                                  const float* __restrict__ sin_table,
+                                  const int* __restrict__ positions,
+                                  const int* __restrict__ token_seq,
+                                  const int* __restrict__ block_table, int table_stride,
+                                  T* __restrict__ k_cache, T* __restrict__ v_cache,
+                                  int page_shift, int n_q, int n_kv, int d, int rot,
+                                  int write_kv) {
+  const int t = blockIdx.x;
+  const int pos = positions[t];
+  const int half = rot / 2;
+  const float* cs = cos_table + (size_t)pos * half;
+  const float* sn = sin_table + (size_t)pos * half;
+  const int width = (n_q + 2 * n_kv) * d;
+  const float* row = partials + (size_t)t * width;
+  auto value = [&](int col) {
+    float v = 0.f;
+    for (int p = 0; p < num_partials; ++p) v += row[p * partial_stride + col];
+    if (bias) v += Elem<TB>::load(bias + col);
+    return Elem<T>::round(v);
+  };
+
+  for (int idx = threadIdx.x; idx < n_q * d; idx += blockDim.x) {
+    const int head = idx / d, j = idx - head * d;
+    float y;
+    if (j < half)
+      y = value(idx) * cs[j] - value(idx + half) * sn[j];
+    else if (j < rot)
+      y = value(idx) * cs[j - half] + value(idx - half) * sn[j - half];
+    else
+      y = value(idx);
+    Elem<T>::store(q_out + (size_t)t * n_q * d + idx, y);
+  }
+  if (!write_kv) return;
+
+  const int page_size = 1 << page_shift;
+  const int page = block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)];
+  if (page < 0) return;
+  const int off = pos & (page_size - 1);
+  const int k0 = n_q * d, v0 = (n_q + n_kv) * d;
+  for (int idx = threadIdx.x; idx < n_kv * d; idx += blockDim.x) {
+    const int head = idx / d, j = idx - head * d;
+    float y;
+    if (j < half)
+      y = value(k0 + idx) * cs[j] - value(k0 + idx + half) * sn[j];
+    else if (j < rot)
+      y = value(k0 + idx) * cs[j - half] + value(k0 + idx - half) * sn[j - half];
+    else
+      y = value(k0 + idx);
+    Elem<T>::store(k_cache + (((size_t)page * n_kv + head) * page_size + off) * d + j, y);
+    Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * d + j) * page_size + off,
+                   value(v0 + idx));
+  }
+}
+
+extern "C" int mk_qkv_finish(const float* partials, int num_partials, long long partial_stride,
+                             const void* bias, int bias_dtype, void* q_out, int dtype,
+                             const float* cos_table, const float* sin_table, int table_positions,
+                             const int* positions, const int* token_seq, const int* block_table,
+                             int table_stride, void* k_cache, void* v_cache, int page_size,
+                             int n_q, int n_kv, int d, int rot, int write_kv, int tokens,
+                             hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv >= 0 && d > 0 && num_partials >= 1,
+             "qkv_finish: bad sizes");
+  MK_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "qkv_finish: rotary width %d", rot);
+  MK_REQUIRE(mk_is_pow2(page_size), "qkv_finish: page size %d is not a power of two", page_size);
+  MK_REQUIRE(rot == 0 || table_positions > 0, "qkv_finish: empty angle table");
+  MK_REQUIRE(dtype == MK_BF16 || dtype == MK_F32, "qkv_finish: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  const int shift = mk_log2(page_size);
+#define QKV_LAUNCH(T, TB)                                                                      \
+  qkv_finish_kernel<T, TB><<<tokens, 256, 0, stream>>>(                                        \
+      partials, num_partials, (size_t)partial_stride, (const TB*)bias, (T*)q_out, cos_table,   \
+      sin_table, positions, token_seq, block_table, table_stride, (T*)k_cache, (T*)v_cache,    \
+      shift, n_q, n_kv, d, rot, write_kv)
+  if (dtype == MK_BF16) {
+    if (bias && bias_dtype == MK_BF16) QKV_LAUNCH(bf16_t, bf16_t);
+    else QKV_LAUNCH(bf16_t, float);
+  } else {
+    if (bias && bias_dtype == MK_BF16) QKV_LAUNCH(float, bf16_t);
+    else QKV_LAUNCH(float, float);
+  }
+#undef QKV_LAUNCH
+  MK_LAUNCH_CHECK("qkv_finish");
   return 0;
 }

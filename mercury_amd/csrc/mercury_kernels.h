@@ -52,6 +52,49 @@ int mk_attention_generic(const void* q, int q_stride, void* out, int out_stride,
                          int table_stride, int page_size, int n_q, int n_kv, int d, float scale,
                          int window, int tokens, hipStream_t stream);
 
+// The same two for a projection that arrives as float32 partial sums [p, T, width] of a
+// K-split product: the slices are added in order (with the bias) before the op proper.
+int mk_silu_mul_partials(const float* partials, int num_partials, long long partial_stride,
+                         void* out, int out_dtype, int tokens, int inter, hipStream_t stream);
+int mk_qkv_finish(const float* partials, int num_partials, long long partial_stride,
+                  const void* bias, int bias_dtype, void* q_out, int dtype,
+                  const float* cos_table, const float* sin_table, int table_positions,
+                  const int* positions, const int* token_seq, const int* block_table,
+                  int table_stride, void* k_cache, void* v_cache, int page_size, int n_q,
+                  int n_kv, int d, int rot, int write_kv, int tokens, hipStream_t stream);
+
+// ---- library "mfma": bfloat16 kernels on the matrix cores
+
+// y = x W^T for 1 <= M <= 64 rows of x, K split into `slices` (ask mk_linear_skinny_slices
+// for a good count): out is float32 [slices, M, N], to be summed over the slices.
+int mk_linear_skinny_slices(int M, int N, int K);
+int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int K, int slices,
+                     hipStream_t stream);
+
+// y = x W^T (+ bias) for any M, tiled through LDS; output bfloat16 or float32, or float32
+// accumulated into `out`.
+int mk_linear_tiled(const void* x, const void* w, const void* bias, int bias_dtype, void* out,
+                    int out_dtype, int accumulate, int M, int N, int K, int ldo,
+                    hipStream_t stream);
+
+// Whether mk_attention_mfma takes this head size and page size.
+int mk_attention_mfma_supported(int head_dim, int page_size);
+
+// The same attention on the matrix cores.  The caller cuts the step into tiles of 16 rows
+// (row f of a sequence = token f / G, head kvh * G + f % G): tile_seq / tile_row0 name each
+// tile's sequence and first row.  cu_q [S+1] are the prefix sums of the sequences' token
+// counts, kv_len [S] their lengths once this step's tokens are written.  With num_splits > 1
+// the keys are split and part_o [tiles, n_kv, splits, 16, d] / part_ml [.., 16, 2] hold the
+// partial results.
+int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
+                      const void* k_cache, const void* v_cache, const int* tile_seq,
+                      const int* tile_row0, int num_tiles, const int* cu_q, const int* kv_len,
+                      const int* block_table, int table_stride, int page_size, int n_q, int n_kv,
+                      int d, float scale, int window, int num_splits, float* part_o,
+                      float* part_ml, hipStream_t stream);
+
+// ---- library "core" again
+
 int mk_argmax(const float* logits, int rows, int vocab, long long row_stride, int* out,
               hipStream_t stream);
 

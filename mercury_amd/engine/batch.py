@@ -53,10 +53,50 @@ class StepContext:
         self.max_q_len = self.max_kv_len = 0
         self.all_decode = False
         self.fresh_slots: list = []
+        self._tiles: dict = {}
+
+    def tiles(self, group: int):
+        """(tile_seq, tile_row0, count) for attention tiles of 16 rows, a row being a
+        (token, head within a group of `group` query heads) pair: sequence s with n tokens
+        this step has ceil(n * group / 16) tiles."""
+        cached = self._tiles.get(group)
+        if cached is None:
+            seqs, rows = [], []
+            for s, (_first, count, _start) in enumerate(self.spans):
+                n = -(-count * group // 16)
+                seqs.extend([s] * n)
+                rows.extend(range(0, 16 * n, 16))
+            device = self.token_ids.device
+            both = torch.tensor([seqs, rows], dtype=torch.int32).to(device, non_blocking=True)
+            cached = (both[0], both[1], len(seqs))
+            self._tiles[group] = cached
+        return cached
 
 
 class BatchError(ValueError):
     pass
+
+
+def context_from_spans(spans: list, device, token_ids=None) -> StepContext:
+    """A step context without a cache manager: `spans` lists (token count, start position)
+    per sequence.  Block tables are left to the caller."""
+    step = StepContext()
+    counts = [c for c, _ in spans]
+    starts = [s for _, s in spans]
+    cu = np.zeros(len(spans) + 1, dtype=np.int64)
+    np.cumsum(counts, out=cu[1:])
+    token_seq = np.repeat(np.arange(len(spans)), counts)
+    positions = np.arange(int(cu[-1])) - cu[token_seq] + np.asarray(starts)[token_seq]
+    as_dev = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=device)
+    step.num_tokens, step.num_seqs = int(cu[-1]), len(spans)
+    step.token_ids = as_dev(token_ids if token_ids is not None else np.zeros(int(cu[-1])))
+    step.positions, step.token_seq, step.cu_q = as_dev(positions), as_dev(token_seq), as_dev(cu)
+    step.kv_len = as_dev(np.asarray(starts) + np.asarray(counts))
+    step.state_slots = as_dev(np.arange(len(spans)))
+    step.spans = [(int(cu[s]), counts[s], starts[s]) for s in range(len(spans))]
+    step.max_q_len, step.max_kv_len = max(counts), max(s + c for c, s in spans)
+    step.all_decode = step.max_q_len == 1
+    return step
 
 
 def build_step(chunks: list, manager, vocab_size: int, max_positions: int, device,

@@ -27,10 +27,16 @@ CSRC = PACKAGE_DIR / "csrc"
 
 LIBRARIES = {
     "core": [
+        "host_support.hip",
         "elementwise.hip",
         "gemm_generic.hip",
         "attention_generic.hip",
         "sampling.hip",
+    ],
+    "mfma": [
+        "host_support.hip",
+        "attention_mfma.hip",
+        "gemm_mfma.hip",
     ],
 }
 

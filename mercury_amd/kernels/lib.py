@@ -24,8 +24,17 @@ _SIGNATURES = {
         "mk_rope_kv_write": [P, I, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_linear_generic": [P, P, I, P, I, P, I, I, I, I, I, I, I, P],
         "mk_attention_generic": [P, I, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
+        "mk_silu_mul_partials": [P, I, L, P, I, I, I, P],
+        "mk_qkv_finish": [P, I, L, P, I, P, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_argmax": [P, I, I, L, P, P],
         "mk_sample": [P, I, I, L, P, P, P, P, P, P],
+    },
+    "mfma": {
+        "mk_linear_skinny_slices": [I, I, I],
+        "mk_linear_skinny": [P, P, P, I, I, I, I, P],
+        "mk_linear_tiled": [P, P, P, I, P, I, I, I, I, I, I, P],
+        "mk_attention_mfma_supported": [I, I],
+        "mk_attention_mfma": [P, I, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P, P, P],
     },
 }
 

@@ -103,9 +103,23 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
     return out
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up [T, 2I]."""
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None,
+             out_dtype: torch.dtype | None = None) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up [T, 2I], or for
+    float32 partial sums [P, T, 2I] of it (summed first; the result is `out_dtype`)."""
     _dev(gate_up, out)
+    if gate_up.dim() == 3:
+        if gate_up.dtype != torch.float32 or out_dtype is None:
+            raise KernelArgumentError("silu_mul: partial sums are float32 and need an out_dtype")
+        slices, tokens, two_i = gate_up.shape
+        inter = two_i // 2
+        if out is None:
+            out = torch.empty((tokens, inter), dtype=out_dtype, device=gate_up.device)
+        lib = _lib.load("core")
+        _lib.check(lib, lib.mk_silu_mul_partials(_ptr(gate_up), slices, tokens * two_i, _ptr(out),
+                                                 dtype_code(out_dtype), tokens, inter, _stream()),
+                   "silu_mul")
+        return out
     tokens, two_i = gate_up.shape
     if two_i % 2:
         raise KernelArgumentError("silu_mul: the last dimension must be even")
@@ -123,13 +137,42 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Te
 # --------------------------------------------------------------------------------- projection
 
 
+SKINNY_MAX_ROWS = 64
+
+
+def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
+    """Whether x W^T is best computed as K-split float32 partial sums (`linear_partials`):
+    few rows of bfloat16 x, where the weights are the traffic and the chip needs the split to
+    have enough wavefronts in flight."""
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and 0 < x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0)
+
+
+def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
+    """Float32 partial sums [P, M, N] of x W^T over P slices of K; the consumer (rmsnorm,
+    rope_kv_write, silu_mul: their `partials` forms) adds them up in slice order."""
+    _dev(x, w)
+    if not wants_partials(x, w) or x.shape[1] != w.shape[1]:
+        raise KernelArgumentError(f"linear_partials: x {tuple(x.shape)} / W {tuple(w.shape)} not eligible")
+    m, k = x.shape
+    n = w.shape[0]
+    lib = _lib.load("mfma")
+    slices = lib.mk_linear_skinny_slices(m, n, k)
+    out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+    _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream()),
+               "linear_partials")
+    return out
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
            out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
-           accumulate: bool = False) -> torch.Tensor:
+           accumulate: bool = False, kernel: str = "auto") -> torch.Tensor:
     """y = x W^T (+ bias) for x [M, K], W [N, K].
 
     With `accumulate` the product is added into the float32 tensor `out` (the residual
     stream) instead of being stored.  The result's dtype is `out_dtype` (default: x's).
+    kernel: "auto" takes the matrix-core kernels for bfloat16 with K % 8 == 0 and the float32
+    multiply-add kernel otherwise; "generic" and "mfma" force one.
     """
     _dev(x, w, bias, out)
     if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
@@ -151,6 +194,22 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
         out_dtype = out.dtype
     if out.shape != (m, n):
         raise KernelArgumentError(f"linear: out {tuple(out.shape)} is not [{m}, {n}]")
+    if m == 0:
+        return out
+    if kernel == "auto":
+        kernel = "mfma" if x.dtype == torch.bfloat16 and k % 8 == 0 else "generic"
+    if kernel == "mfma":
+        if x.dtype != torch.bfloat16 or k % 8:
+            raise KernelArgumentError("linear: the matrix-core kernels take bfloat16 with K % 8 == 0")
+        lib = _lib.load("mfma")
+        if m <= SKINNY_MAX_ROWS and out_dtype == torch.float32 and bias is None and not accumulate:
+            _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, 1, _stream()),
+                       "linear")
+            return out
+        _lib.check(lib, lib.mk_linear_tiled(
+            _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
+            _ptr(out), dtype_code(out_dtype), int(accumulate), m, n, k, n, _stream()), "linear")
+        return out
     lib = _lib.load("core")
     _lib.check(lib, lib.mk_linear_generic(
         _ptr(x), _ptr(w), dtype_code(x.dtype), _ptr(bias),
@@ -179,11 +238,21 @@ def _check_caches(what, k_cache, v_cache, n_kv, head_dim, dtype) -> int:
 def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
                   positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                   k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, n_q: int,
-                  n_kv: int, head_dim: int, rotary_dim: int, write_kv: bool = True) -> None:
-    """Rotate q (in place) and k by their absolute positions; write k into the paged key
-    cache [pages, n_kv, page_size, head_dim] and v into the value cache
-    [pages, n_kv, head_dim, page_size] at the slots the block table gives."""
-    _dev(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache)
+                  n_kv: int, head_dim: int, rotary_dim: int, write_kv: bool = True,
+                  bias: torch.Tensor | None = None, out_dtype: torch.dtype | None = None):
+    """Rotate q and k by their absolute positions; write k into the paged key cache
+    [pages, n_kv, page_size, head_dim] and v into the value cache
+    [pages, n_kv, head_dim, page_size] at the slots the block table gives.
+
+    qkv [T, (n_q + 2 n_kv) d] in the compute dtype is rotated in place (q part) and returned.
+    qkv as float32 partial sums [P, T, width] is summed (plus `bias`) first, and the rotated q
+    comes back as a new [T, n_q d] tensor of `out_dtype`."""
+    _dev(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache, bias)
+    if qkv.dim() == 3:
+        return _qkv_finish(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache,
+                           n_q, n_kv, head_dim, rotary_dim, write_kv, bias, out_dtype)
+    if bias is not None:
+        raise KernelArgumentError("rope: a bias is only added to partial sums")
     _i32(positions, "positions")
     _i32(token_seq, "token_seq")
     _i32(block_table, "block_table")
@@ -207,32 +276,98 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor
         _ptr(positions), _ptr(token_seq), _ptr(block_table), block_table.shape[1],
         _ptr(k_cache), _ptr(v_cache), page_size, n_q, n_kv, head_dim, rotary_dim,
         int(write_kv), tokens, _stream()), "rope_kv_write")
+    return qkv
 
 
-def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
-              positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
-              n_q: int, n_kv: int, head_dim: int, scale: float, window: int | None = None,
-              out: torch.Tensor | None = None) -> torch.Tensor:
-    """Causal grouped-query attention of every token of the step over its sequence's cached
-    keys; q is read from rows of `q` with stride `q_stride` (the fused qkv buffer).
-    Returns [T, n_q * head_dim]."""
-    _dev(q, k_cache, v_cache, positions, token_seq, block_table, out)
+def _qkv_finish(parts, cos, sin, positions, token_seq, block_table, k_cache, v_cache, n_q, n_kv,
+                head_dim, rotary_dim, write_kv, bias, out_dtype):
     _i32(positions, "positions")
     _i32(token_seq, "token_seq")
     _i32(block_table, "block_table")
-    tokens = positions.shape[0]
+    slices, tokens, width = parts.shape
+    if parts.dtype != torch.float32 or out_dtype is None:
+        raise KernelArgumentError("rope: partial sums are float32 and need an out_dtype")
+    if width != (n_q + (2 * n_kv if write_kv else 0)) * head_dim:
+        raise KernelArgumentError(f"rope: partial sums of width {width} do not match the heads")
+    if bias is not None and bias.shape != (width,):
+        raise KernelArgumentError("rope: bias does not match the projection width")
+    table_positions = 0
+    if rotary_dim:
+        if cos is None or sin is None or cos.dtype != torch.float32 or cos.shape != sin.shape \
+                or cos.shape[1] != rotary_dim // 2:
+            raise KernelArgumentError("rope: float32 cos and sin tables of the rotary width are required")
+        table_positions = cos.shape[0]
+    page_size = _check_caches("rope", k_cache, v_cache, n_kv, head_dim, out_dtype) if write_kv else 1
+    q = torch.empty((tokens, n_q * head_dim), dtype=out_dtype, device=parts.device)
+    lib = _lib.load("core")
+    _lib.check(lib, lib.mk_qkv_finish(
+        _ptr(parts), slices, tokens * width, _ptr(bias),
+        dtype_code(bias.dtype) if bias is not None else F32, _ptr(q), dtype_code(out_dtype),
+        _ptr(cos), _ptr(sin), table_positions, _ptr(positions), _ptr(token_seq),
+        _ptr(block_table), block_table.shape[1], _ptr(k_cache), _ptr(v_cache), page_size, n_q,
+        n_kv if write_kv else 0, head_dim, rotary_dim, int(write_kv), tokens, _stream()),
+        "qkv_finish")
+    return q
+
+
+def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+              step, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int, scale: float,
+              window: int | None = None, out: torch.Tensor | None = None,
+              kernel: str = "auto") -> torch.Tensor:
+    """Causal grouped-query attention of every token of the step over its sequence's cached
+    keys; q is read from rows of `q` with stride `q_stride` (the fused qkv buffer).
+    `step` describes the batch (positions, token_seq, cu_q, kv_len, spans, tiles());
+    `block_table` is the step's table of the cache group.  Returns [T, n_q * head_dim].
+
+    kernel: "auto" takes the matrix-core kernel for bfloat16 where it covers the head and page
+    size and the float32-arithmetic kernel otherwise; "generic" and "mfma" force one.
+    """
+    _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out)
+    _i32(block_table, "block_table")
+    tokens = step.num_tokens
     if q.numel() < (tokens - 1) * q_stride + n_q * head_dim and tokens:
         raise KernelArgumentError("attention: q buffer too small")
+    if block_table.dim() != 2 or block_table.shape[0] != step.num_seqs:
+        raise KernelArgumentError("attention: the block table needs one row per sequence")
     page_size = _check_caches("attention", k_cache, v_cache, n_kv, head_dim, q.dtype)
     if out is None:
         out = torch.empty((tokens, n_q * head_dim), dtype=q.dtype, device=q.device)
-    lib = _lib.load("core")
-    _lib.check(lib, lib.mk_attention_generic(
+    use_mfma = kernel == "mfma"
+    if kernel == "auto" and q.dtype == torch.bfloat16:
+        use_mfma = bool(_lib.load("mfma").mk_attention_mfma_supported(head_dim, page_size))
+    if not use_mfma:
+        lib = _lib.load("core")
+        _lib.check(lib, lib.mk_attention_generic(
+            _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
+            dtype_code(q.dtype), _ptr(step.positions), _ptr(step.token_seq), _ptr(block_table),
+            block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
+            int(window or 0), tokens, _stream()), "attention")
+        return out
+    if q.dtype != torch.bfloat16:
+        raise KernelArgumentError("attention: the matrix-core kernel takes bfloat16 only")
+    lib = _lib.load("mfma")
+    group = n_q // n_kv
+    tile_seq, tile_row0, num_tiles = step.tiles(group)
+    # Split the keys when the tiles alone would leave most of the chip idle: aim at about a
+    # thousand wavefronts, each with at least one block of 32 keys.
+    span = step.max_kv_len if not window else min(step.max_kv_len, window + step.max_q_len)
+    blocks = max(1, -(-span // 32))
+    waves = max(1, num_tiles * n_kv)
+    splits = max(1, min(blocks // ATTENTION_MIN_BLOCKS_PER_SPLIT or 1, -(-ATTENTION_TARGET_WAVES // waves)))
+    part_o = part_ml = None
+    if splits > 1:
+        part_o = torch.empty((num_tiles, n_kv, splits, 16, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((num_tiles, n_kv, splits, 16, 2), dtype=torch.float32, device=q.device)
+    _lib.check(lib, lib.mk_attention_mfma(
         _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
-        dtype_code(q.dtype), _ptr(positions), _ptr(token_seq), _ptr(block_table),
-        block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
-        int(window or 0), tokens, _stream()), "attention")
+        _ptr(tile_seq), _ptr(tile_row0), num_tiles, _ptr(step.cu_q), _ptr(step.kv_len),
+        _ptr(block_table), block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
+        int(window or 0), splits, _ptr(part_o), _ptr(part_ml), _stream()), "attention")
     return out
+
+
+ATTENTION_TARGET_WAVES = 1024
+ATTENTION_MIN_BLOCKS_PER_SPLIT = 2
 
 
 # ----------------------------------------------------------------------------------- sampling

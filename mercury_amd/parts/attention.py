@@ -76,19 +76,28 @@ class Attention(Mixer):
 
     # ---- one step
 
-    def forward(self, x, step, cache, state, accum) -> None:
+    def forward(self, x, step, cache, state, accum):
         n_q, n_kv, d = self.n_q, self.n_kv, self.head_dim
         table = step.block_tables[cache.group]
-        if cache.writes:
-            qkv = ops.linear(x, self.w_qkv, self.b_qkv)
-        else:
-            # Reads a cache another entry fills: only the queries are projected.
-            rows = n_q * d
-            qkv = ops.linear(x, self.w_qkv[:rows], None if self.b_qkv is None else self.b_qkv[:rows])
         pos = self.position
-        ops.rope_kv_write(qkv, pos.cos, pos.sin, step.positions, step.token_seq, table,
-                          cache.k if cache.writes else None, cache.v if cache.writes else None,
-                          n_q, n_kv if cache.writes else 0, d, pos.rotary_dim, cache.writes)
-        attended = ops.attention(qkv, qkv.shape[1], cache.k, cache.v, step.positions,
-                                 step.token_seq, table, n_q, n_kv, d, self.scale, self.window)
+        w, b = self.w_qkv, self.b_qkv
+        if not cache.writes:
+            # Reads a cache another entry fills: only the queries are projected.
+            w, b = w[:n_q * d], None if b is None else b[:n_q * d]
+        k_cache, v_cache = (cache.k, cache.v) if cache.writes else (None, None)
+        heads_kv = n_kv if cache.writes else 0
+        if ops.wants_partials(x, w):
+            # Few rows: K-split partial sums, added up by the rotary kernel.
+            q = ops.rope_kv_write(ops.linear_partials(x, w), pos.cos, pos.sin, step.positions,
+                                  step.token_seq, table, k_cache, v_cache, n_q, heads_kv, d,
+                                  pos.rotary_dim, cache.writes, bias=b, out_dtype=x.dtype)
+        else:
+            q = ops.rope_kv_write(ops.linear(x, w, b), pos.cos, pos.sin, step.positions,
+                                  step.token_seq, table, k_cache, v_cache, n_q, heads_kv, d,
+                                  pos.rotary_dim, cache.writes)
+        attended = ops.attention(q, q.shape[1], cache.k, cache.v, step, table, n_q, n_kv, d,
+                                 self.scale, self.window)
+        if self.b_o is None and ops.wants_partials(attended, self.w_o):
+            return ops.linear_partials(attended, self.w_o)    # the next norm adds them into accum
         ops.linear(attended, self.w_o, self.b_o, out=accum, accumulate=True)
+        return None

@@ -46,9 +46,13 @@ class PreNormBlock(Part):
     def weight_bytes(self) -> int:
         return sum(part.weight_bytes() for _, part in self._children())
 
-    def forward(self, h, step, cache, state, dtype) -> None:
-        x = self.norm_mixer.forward(h, dtype)
-        self.mixer.forward(x, step, cache, state, h)
+    def forward(self, h, step, cache, state, dtype, pending=None):
+        """Runs the layer on the stream h.  `pending` are partial sums [P, T, H] that still
+        have to be added into h (the previous projection's, when it left them to its
+        consumer); the return value is the same for whoever reads h next."""
+        x = self.norm_mixer.forward(h, dtype, partials=pending)
+        pending = self.mixer.forward(x, step, cache, state, h)
         if self.ffn is not None:
-            x = self.norm_ffn.forward(h, dtype)
-            self.ffn.forward(x, step, h)
+            x = self.norm_ffn.forward(h, dtype, partials=pending)
+            pending = self.ffn.forward(x, step, h)
+        return pending

@@ -40,7 +40,12 @@ class GatedMLP(FeedForward):
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.w_gate_up, self.w_down))
 
-    def forward(self, x, step, accum) -> None:
-        gate_up = ops.linear(x, self.w_gate_up)
-        act = ops.silu_mul(gate_up)
+    def forward(self, x, step, accum):
+        if ops.wants_partials(x, self.w_gate_up):
+            act = ops.silu_mul(ops.linear_partials(x, self.w_gate_up), out_dtype=x.dtype)
+        else:
+            act = ops.silu_mul(ops.linear(x, self.w_gate_up))
+        if ops.wants_partials(act, self.w_down):
+            return ops.linear_partials(act, self.w_down)      # the next norm adds them into accum
         ops.linear(act, self.w_down, out=accum, accumulate=True)
+        return None

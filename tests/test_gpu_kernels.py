@@ -141,6 +141,84 @@ def test_linear_accumulates_into_the_float32_stream(dtype):
     torch.testing.assert_close(acc_d.cpu(), want, atol=1e-5, rtol=1e-5)
 
 
+@pytest.mark.parametrize("m,n,k", [(1, 1003, 168), (8, 896, 4864), (17, 1152, 896), (64, 130, 264),
+                                   (33, 9728, 896), (5, 7, 8)])
+def test_skinny_projection_partial_sums(m, n, k):
+    """Few rows on the matrix cores: float32 slices over K whose sum is the product."""
+    x_h, x_d = as_dtype(rnd(m, k, seed=21), torch.bfloat16)
+    w_h, w_d = as_dtype(rnd(n, k, seed=22, scale=0.1), torch.bfloat16)
+    assert ops().wants_partials(x_d, w_d)
+    parts = ops().linear_partials(x_d, w_d)
+    assert parts.dtype == torch.float32 and parts.shape[1:] == (m, n)
+    want = (x_h.double() @ w_h.double().T).float()
+    torch.testing.assert_close(parts.sum(0).cpu(), want, atol=2e-4, rtol=1e-4)
+    whole = ops().linear(x_d, w_d, out_dtype=torch.float32, kernel="mfma")   # one slice: the logits path
+    torch.testing.assert_close(whole.cpu(), want, atol=2e-4, rtol=1e-4)
+    assert not ops().wants_partials(torch.zeros(65, k, dtype=torch.bfloat16, device=DEV), w_d)
+    assert not ops().wants_partials(x_d.float(), w_d.float())
+
+
+@pytest.mark.parametrize("m,n,k", [(70, 130, 56), (129, 1152, 896), (300, 64, 264), (2048, 896, 4864),
+                                   (65, 1003, 168)])
+def test_tiled_projection(m, n, k):
+    """Many rows on the matrix cores through LDS: bfloat16 with bias, float32, accumulate."""
+    x_h, x_d = as_dtype(rnd(m, k, seed=23), torch.bfloat16)
+    w_h, w_d = as_dtype(rnd(n, k, seed=24, scale=0.1), torch.bfloat16)
+    b_h, b_d = as_dtype(rnd(n, seed=25), torch.bfloat16)
+    want = (x_h.double() @ w_h.double().T).float()
+    got = ops().linear(x_d, w_d, b_d, kernel="mfma")
+    torch.testing.assert_close(got.float().cpu(), want + b_h, **tol(torch.bfloat16))
+    got = ops().linear(x_d, w_d, b_d.float(), kernel="mfma")            # a float32 bias
+    torch.testing.assert_close(got.float().cpu(), want + b_h, **tol(torch.bfloat16))
+    got32 = ops().linear(x_d, w_d, out_dtype=torch.float32, kernel="mfma")
+    torch.testing.assert_close(got32.cpu(), want, atol=5e-4, rtol=1e-4)
+    acc = rnd(m, n, seed=26)
+    acc_d = acc.clone().to(DEV)
+    ops().linear(x_d, w_d, out=acc_d, accumulate=True, kernel="mfma")
+    torch.testing.assert_close(acc_d.cpu(), acc + want, atol=5e-4, rtol=1e-4)
+
+
+def test_matrix_core_projection_refuses_what_it_cannot_do():
+    from mercury_amd.kernels.ops import KernelArgumentError
+
+    x = torch.zeros(4, 50, dtype=torch.bfloat16, device=DEV)      # K % 8 != 0
+    w = torch.zeros(6, 50, dtype=torch.bfloat16, device=DEV)
+    with pytest.raises(KernelArgumentError):
+        ops().linear(x, w, kernel="mfma")
+    assert ops().linear(x, w).shape == (4, 6)                       # "auto" takes the other kernel
+
+
+def test_consumers_of_partial_sums():
+    """SiLU gating and rotary + cache write over K-split slices equal the stored-projection
+    forms applied to the rounded sum."""
+    parts = rnd(3, 9, 2 * 200, seed=27)
+    whole = parts.sum(0).to(torch.bfloat16)
+    want = ops().silu_mul(whole.to(DEV))
+    got = ops().silu_mul(parts.to(DEV), out_dtype=torch.bfloat16)
+    assert torch.equal(got.cpu(), want.cpu())
+
+    n_q, n_kv, d, page = 6, 2, 32, 16
+    width = (n_q + 2 * n_kv) * d
+    parts = rnd(4, 5, width, seed=28)
+    bias = rnd(width, seed=29).to(torch.bfloat16)
+    cos, sin = rotary_tables(d, 10000.0, 64)
+    positions = torch.tensor([3, 4, 40, 41, 0], dtype=torch.int32, device=DEV)
+    token_seq = torch.tensor([0, 0, 1, 1, 2], dtype=torch.int32, device=DEV)
+    table = torch.tensor([[1, -1, -1], [2, 3, 4], [5, -1, -1]], dtype=torch.int32, device=DEV)
+    caches = [[torch.zeros(8, n_kv, page, d, dtype=torch.bfloat16, device=DEV),
+               torch.zeros(8, n_kv, d, page, dtype=torch.bfloat16, device=DEV)] for _ in range(2)]
+    stored = (parts.sum(0) + bias.float()).to(torch.bfloat16).to(DEV)
+    q_want = ops().rope_kv_write(stored, cos.to(DEV), sin.to(DEV), positions, token_seq, table,
+                                 caches[0][0], caches[0][1], n_q, n_kv, d, d)[:, : n_q * d]
+    q_got = ops().rope_kv_write(parts.to(DEV), cos.to(DEV), sin.to(DEV), positions, token_seq, table,
+                                caches[1][0], caches[1][1], n_q, n_kv, d, d, bias=bias.to(DEV),
+                                out_dtype=torch.bfloat16)
+    assert torch.equal(q_got.cpu(), q_want.cpu())
+    assert torch.equal(caches[0][0].cpu(), caches[1][0].cpu())
+    assert torch.equal(caches[0][1].cpu(), caches[1][1].cpu())
+    assert caches[0][0].abs().sum() > 0
+
+
 def test_linear_rows_do_not_depend_on_the_batch():
     """A row's result is bitwise the same alone and among 100 others."""
     x = rnd(101, 300, seed=17).to(DEV)
@@ -258,9 +336,12 @@ def test_rotary_scores_depend_on_distance_only():
 
 
 def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens, q_lens, scale,
-                  window=None, poison=None):
+                  window=None, poison=None, kernel="auto", hide_before=None):
     """q_h: list per sequence of [q_len, n_q, d] (the last q_len positions of the sequence);
-    k_h/v_h: list per sequence of [seq_len, n_kv, d]."""
+    k_h/v_h: list per sequence of [seq_len, n_kv, d].  `hide_before`: per sequence, the number
+    of leading pages to drop from the table (-1) and to poison, as after a window passed."""
+    from mercury_amd.engine.batch import context_from_spans
+
     n_q, d = q_h[0].shape[1:]
     n_kv = k_h[0].shape[1]
     k_cache = torch.zeros(num_pages, n_kv, page, d, dtype=dtype)
@@ -270,36 +351,50 @@ def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens
         v_cache[:] = poison
     width = max(len(p) for p in pages_per_seq)
     table = torch.full((len(q_h), width), -1, dtype=torch.int32)
-    positions, token_seq = [], []
     for s, pages in enumerate(pages_per_seq):
         table[s, : len(pages)] = torch.tensor(pages, dtype=torch.int32)
         for p in range(seq_lens[s]):
             k_cache[pages[p // page], :, p % page] = k_h[s][p].to(dtype)
             v_cache[pages[p // page], :, p % page] = v_h[s][p].to(dtype)
-        positions += list(range(seq_lens[s] - q_lens[s], seq_lens[s]))
-        token_seq += [s] * q_lens[s]
+        for g in range(hide_before[s] if hide_before else 0):
+            k_cache[pages[g]] = 1e4
+            v_cache[pages[g]] = 1e4
+            table[s, g] = -1
+    step = context_from_spans([(ql, sl - ql) for ql, sl in zip(q_lens, seq_lens)], DEV)
     q_flat = torch.cat([q.reshape(q.shape[0], n_q * d) for q in q_h]).to(dtype).to(DEV)
     v_cache = v_cache.transpose(2, 3).contiguous()      # values lie transposed within a page
-    out = ops().attention(q_flat, n_q * d, k_cache.to(DEV), v_cache.to(DEV),
-                          torch.tensor(positions, dtype=torch.int32, device=DEV),
-                          torch.tensor(token_seq, dtype=torch.int32, device=DEV), table.to(DEV),
-                          n_q, n_kv, d, scale, window)
+    out = ops().attention(q_flat, n_q * d, k_cache.to(DEV), v_cache.to(DEV), step, table.to(DEV),
+                          n_q, n_kv, d, scale, window, kernel=kernel)
     return out.float().cpu().view(-1, n_q, d)
+
+
+# (dtype, kernel) pairs: the float32-arithmetic kernel in both dtypes, the matrix-core kernel
+# in bfloat16 where the head size allows it.
+def kernels_for(d, page):
+    pairs = [(torch.float32, "generic"), (torch.bfloat16, "generic")]
+    if d % 32 == 0 and page >= 16:
+        pairs.append((torch.bfloat16, "mfma"))
+    return pairs
 
 
 def rounded(x, dtype):
     return x.to(dtype).float()
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("n_q,n_kv,d,page", [(4, 2, 8, 16), (6, 1, 48, 8), (2, 2, 128, 16),
-                                             (14, 2, 64, 16), (3, 1, 80, 4)])
-def test_attention_whole_prompt_matches_plain(dtype, n_q, n_kv, d, page):
+ATTENTION_SHAPES = [(4, 2, 8, 16), (6, 1, 48, 8), (2, 2, 128, 16), (14, 2, 64, 16), (3, 1, 80, 4),
+                    (5, 5, 32, 32), (12, 4, 96, 16), (8, 1, 256, 64), (28, 4, 128, 16)]
+ATTENTION_CASES = [(n_q, n_kv, d, page, dtype, kernel) for n_q, n_kv, d, page in ATTENTION_SHAPES
+                   for dtype, kernel in kernels_for(d, page)]
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page,dtype,kernel", ATTENTION_CASES)
+def test_attention_whole_prompt_matches_plain(n_q, n_kv, d, page, dtype, kernel):
     """(reference: tests/test_attention.py:67-81; scattered pages as in :135-153)"""
     s = 40 if d < 100 else 70
     q, k, v = (rounded(rnd(s, h, d, seed=30 + i), dtype) for i, h in enumerate((n_q, n_kv, n_kv)))
     pages = [11, 3, 7, 30, 2, 19, 25, 1, 9, 14, 22, 5, 28, 8, 17, 6, 4, 12][: -(-s // page)]
-    got = run_attention([q], [k], [v], dtype, [pages], page, 32, [s], [s], d ** -0.5, poison=1e4)
+    got = run_attention([q], [k], [v], dtype, [pages], page, 32, [s], [s], d ** -0.5, poison=1e4,
+                        kernel=kernel)
     want = plain.causal_attention(q, k, v, d ** -0.5)
     torch.testing.assert_close(got, want, **tol(dtype))
     if dtype == torch.float32:
@@ -309,12 +404,13 @@ def test_attention_whole_prompt_matches_plain(dtype, n_q, n_kv, d, page):
         torch.testing.assert_close(got, lib, atol=2e-6, rtol=1e-5)
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_attention_suffix_over_a_cached_prefix_and_decode_rows(dtype):
+@pytest.mark.parametrize("d,dtype,kernel", [(8, torch.float32, "generic"), (8, torch.bfloat16, "generic"),
+                                            (64, torch.bfloat16, "mfma"), (32, torch.bfloat16, "mfma")])
+def test_attention_suffix_over_a_cached_prefix_and_decode_rows(d, dtype, kernel):
     """A 16-token portion at positions 32..47, beside two single decoded tokens of sequences
     of 33 and 17 tokens, in one batch (reference: tests/test_attention.py:84-132 tests the two
     cases separately)."""
-    n_q, n_kv, d, page = 4, 2, 8, 16
+    n_q, n_kv, page = 4, 2, 16
     lens, q_lens = [48, 33, 17], [16, 1, 1]
     qs, ks, vs = [], [], []
     for i, (s, ql) in enumerate(zip(lens, q_lens)):
@@ -323,15 +419,16 @@ def test_attention_suffix_over_a_cached_prefix_and_decode_rows(dtype):
         qs.append(rounded(rnd(s, n_q, d, seed=60 + i), dtype))
     got = run_attention([q[-ql:] for q, ql in zip(qs, q_lens)], ks, vs, dtype,
                         [[2, 5, 9], [12, 1, 30], [7, 20]], page, 32, lens, q_lens, d ** -0.5,
-                        poison=1e4)
+                        poison=1e4, kernel=kernel)
     want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5)[-ql:]
                       for q, k, v, ql in zip(qs, ks, vs, q_lens)])
     torch.testing.assert_close(got, want, **tol(dtype))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("target", [0, 15, 16, 255, 256, 499, 500])
-def test_attention_finds_one_far_key(dtype, target):
+@pytest.mark.parametrize("dtype,kernel", [(torch.float32, "generic"), (torch.bfloat16, "generic"),
+                                          (torch.bfloat16, "mfma")])
+@pytest.mark.parametrize("target", [0, 15, 16, 31, 32, 255, 256, 499, 500])
+def test_attention_finds_one_far_key(dtype, kernel, target):
     """One key among 501 is made to win the softmax outright (its score stands 40 above the
     rest); the output must be that key's value row.  Random weights alone would average over
     hundreds of keys and hide a key that is skipped or read from the wrong slot: the first
@@ -346,52 +443,61 @@ def test_attention_finds_one_far_key(dtype, target):
     q[0, :] = direction * (40.0 * math.sqrt(d) / 256.0)
     q = rounded(q, dtype)
     pages = list(range(40, 40 + -(-s // page)))
-    got = run_attention([q], [k], [v], dtype, [pages], page, 80, [s], [1], d ** -0.5, poison=1e4)
+    got = run_attention([q], [k], [v], dtype, [pages], page, 80, [s], [1], d ** -0.5, poison=1e4,
+                        kernel=kernel)
     torch.testing.assert_close(got[0, 0], v[target, 0], atol=1e-3, rtol=1e-3)
     torch.testing.assert_close(got, plain.causal_attention(q, k, v, d ** -0.5, s - 1), **tol(dtype))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-def test_attention_special_cases_reduce_to_means(dtype):
+@pytest.mark.parametrize("d,page,dtype,kernel", [(16, 8, torch.float32, "generic"),
+                                                 (16, 8, torch.bfloat16, "generic"),
+                                                 (32, 16, torch.bfloat16, "mfma")])
+def test_attention_special_cases_reduce_to_means(d, page, dtype, kernel):
     """One visible key -> its value; equal scores -> the mean of the visible values."""
-    n_q, n_kv, d, page = 2, 1, 16, 8
+    n_q, n_kv = 2, 1
     v = rounded(rnd(20, n_kv, d, seed=73), dtype)
     k = torch.zeros(20, n_kv, d)
     q = rounded(rnd(20, n_q, d, seed=74), dtype)
-    got = run_attention([q], [k], [v], dtype, [[4, 2, 6]], page, 8, [20], [20], d ** -0.5)
+    got = run_attention([q], [k], [v], dtype, [[4, 2, 6]], page, 8, [20], [20], d ** -0.5,
+                        kernel=kernel)
     for p in (0, 1, 7, 8, 19):
         want = v[: p + 1, 0].mean(0)
         torch.testing.assert_close(got[p, 0], want, **tol(dtype))
 
 
-@pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("window", [1, 5, 16, 17, 64])
-def test_attention_window_edge(dtype, window):
+@pytest.mark.parametrize("d,page,dtype,kernel", [(16, 8, torch.float32, "generic"),
+                                                 (16, 8, torch.bfloat16, "generic"),
+                                                 (64, 16, torch.bfloat16, "mfma")])
+@pytest.mark.parametrize("window", [1, 5, 16, 17, 33, 64])
+def test_attention_window_edge(d, page, dtype, kernel, window):
     """With a window w the query at p sees keys p-w+1..p; pages wholly before the window are
-    absent from the table (-1), as the cache manager leaves them."""
-    n_q, n_kv, d, page, s = 4, 2, 16, 8, 45
+    absent from the table (-1) and hold garbage, as the cache manager leaves them."""
+    n_q, n_kv, s, q_len = 4, 2, 77, 6
     q, k, v = (rounded(rnd(s, h, d, seed=80 + i), dtype) for i, h in enumerate((n_q, n_kv, n_kv)))
-    q_len = 6
     pages = list(range(10, 10 + -(-s // page)))
-    first_needed = max(0, (s - q_len) - window + 1)
-    gone = first_needed // page
-    table_pages = [-1] * gone + pages[gone:]
-    # the helper writes through the table, so fill the cache with the full list and only
-    # hide the pages afterwards
-    n_qh = q[-q_len:]
-    k_cache = paged(k, pages, page, 32, dtype)
-    v_cache = paged(v, pages, page, 32, dtype, transposed=True)
-    for g in range(gone):
-        k_cache[pages[g]] = 1e4
-        v_cache[pages[g]] = 1e4
-    table = torch.tensor([table_pages], dtype=torch.int32)
-    out = ops().attention(n_qh.reshape(q_len, n_q * d).to(dtype).to(DEV), n_q * d,
-                          k_cache.to(DEV), v_cache.to(DEV),
-                          torch.arange(s - q_len, s, dtype=torch.int32, device=DEV),
-                          torch.zeros(q_len, dtype=torch.int32, device=DEV), table.to(DEV),
-                          n_q, n_kv, d, d ** -0.5, window)
+    gone = max(0, (s - q_len) - window + 1) // page
+    got = run_attention([q[-q_len:]], [k], [v], dtype, [pages], page, 32, [s], [q_len], d ** -0.5,
+                        window=window, kernel=kernel, hide_before=[gone])
     want = plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-q_len:]
-    torch.testing.assert_close(out.float().cpu().view(q_len, n_q, d), want, **tol(dtype))
+    torch.testing.assert_close(got, want, **tol(dtype))
+
+
+@pytest.mark.parametrize("batch,context", [(1, 4096), (3, 1500), (64, 300)])
+def test_attention_decode_with_split_keys(batch, context):
+    """Decoded tokens over long contexts: the matrix-core kernel splits the keys over many
+    wavefronts and merges the partial results; the float32 kernel does not."""
+    n_q, n_kv, d, page = 14, 2, 64, 16
+    lens = [context - 37 * i for i in range(batch)] if batch < 10 else [context - i for i in range(batch)]
+    per = -(-context // page)
+    qs = [rounded(rnd(1, n_q, d, seed=200 + i), torch.bfloat16) for i in range(batch)]
+    ks = [rounded(rnd(n, n_kv, d, seed=300 + i), torch.bfloat16) for i, n in enumerate(lens)]
+    vs = [rounded(rnd(n, n_kv, d, seed=400 + i), torch.bfloat16) for i, n in enumerate(lens)]
+    pages = [list(range(i * per, (i + 1) * per)) for i in range(batch)]
+    got = run_attention(qs, ks, vs, torch.bfloat16, pages, page, batch * per, lens, [1] * batch,
+                        d ** -0.5, kernel="mfma")
+    want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, n - 1)
+                      for q, k, v, n in zip(qs, ks, vs, lens)])
+    torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
 def test_attention_gqa_equals_mha_with_repeated_heads():

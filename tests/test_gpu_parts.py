@@ -21,6 +21,13 @@ def rnd(*shape, seed=0, scale=1.0):
     return torch.randn(*shape, generator=g) * scale
 
 
+def settle(acc, pending):
+    """A part may hand back partial sums it has not added into the accumulator."""
+    if pending is not None:
+        acc += pending.sum(0)
+    return acc
+
+
 def one_sequence_step(tokens, start, manager, key="s"):
     from mercury_amd.engine.batch import SeqChunk, build_step
 
@@ -54,7 +61,7 @@ def test_feed_forward_part_adds_into_the_accumulator(dtype):
     x = rnd(9, 168, seed=7).to(dtype)
     acc = rnd(9, 168, seed=8)
     acc_d = acc.clone().to(DEV)
-    part.forward(x.to(DEV), None, acc_d)
+    settle(acc_d, part.forward(x.to(DEV), None, acc_d))
     want = acc + plain.gated_mlp(x.float(), params["gate_proj.weight"].float(),
                                  params["up_proj.weight"].float(), params["down_proj.weight"].float())
     tol = dict(atol=1e-5, rtol=1e-5) if dtype == torch.float32 else dict(atol=5e-3, rtol=2e-2)
@@ -85,7 +92,7 @@ def test_attention_part_over_two_portions(dtype, window):
     for start, count in ((0, 21), (21, 9)):
         step = one_sequence_step(count, start, manager)
         acc = torch.zeros(count, hidden, device=DEV)
-        part.forward(x[start:start + count].to(DEV).contiguous(), step, cache, None, acc)
+        settle(acc, part.forward(x[start:start + count].to(DEV).contiguous(), step, cache, None, acc))
         out.append(acc.cpu())
         manager.trim("s", start + count)
     cfg = {"num_attention_heads": n_q, "num_key_value_heads": n_kv, "head_dim": d}
@@ -118,8 +125,8 @@ def test_block_arrangement_is_pre_norm_residual():
     v_pages = torch.zeros(8, spec.kv_heads, spec.head_dim, 16, device=DEV)
     h = rnd(20, cfg["hidden_size"], seed=40)
     h_d = h.clone().to(DEV)
-    block.forward(h_d, one_sequence_step(20, 0, manager), LayerCache(k_pages, v_pages, 0, 16), None,
-                  torch.float32)
+    settle(h_d, block.forward(h_d, one_sequence_step(20, 0, manager),
+                              LayerCache(k_pages, v_pages, 0, 16), None, torch.float32))
     cos, sin = plain.rotary_table(cfg["head_dim"], range(20), cfg["rope_theta"])
     x, residual = plain.decoder_layer(h, None, w, 0, cfg, cos, sin)
     torch.testing.assert_close(h_d.cpu(), x + residual, atol=1e-5, rtol=1e-5)
