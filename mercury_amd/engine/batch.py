@@ -99,10 +99,27 @@ def context_from_spans(spans: list, device, token_ids=None) -> StepContext:
     return step
 
 
-def build_step(chunks: list, manager, vocab_size: int, max_positions: int, device,
-               pinned: bool = True) -> StepContext:
-    """Flatten `chunks` into one packed int32 buffer, copy it to the device once, and slice
-    the context's tensors out of it."""
+class PackedStep:
+    """A step flattened into one int32 host buffer (pinned when a GPU will read it), with the
+    offsets of its parts: token ids, positions, token -> sequence, prefix sums of the
+    sequences' token counts, lengths, state slots, wanted rows, one block table per group."""
+
+    def __init__(self, host, sizes, num_tokens, num_seqs, num_rows, widths, spans, max_q_len,
+                 max_kv_len, fresh_slots):
+        self.host, self.sizes = host, sizes
+        self.num_tokens, self.num_seqs, self.num_rows = num_tokens, num_seqs, num_rows
+        self.widths, self.spans = widths, spans
+        self.max_q_len, self.max_kv_len, self.fresh_slots = max_q_len, max_kv_len, fresh_slots
+
+    def layout(self):
+        """What must be equal for two steps to share device buffers (and a captured graph)."""
+        return (self.num_tokens, self.num_seqs, self.num_rows, tuple(self.widths))
+
+
+def pack_step(chunks: list, manager, vocab_size: int, max_positions: int, pinned: bool = True,
+              table_width: int | None = None) -> PackedStep:
+    """Flatten `chunks` into one packed int32 host buffer.  `table_width` fixes the number of
+    columns of every block table (default: as many as the longest sequence needs)."""
     if not chunks:
         raise BatchError("a step needs at least one sequence")
     num_seqs = len(chunks)
@@ -132,9 +149,12 @@ def build_step(chunks: list, manager, vocab_size: int, max_positions: int, devic
             rows.append(int(cu[s]) + w)
     slots = [manager.requests[c.key].state_slot for c in chunks]
 
+    needed = max(-(-int(kv) // ps) for kv in kv_len)
+    width = needed if table_width is None else table_width
+    if width < needed:
+        raise BatchError(f"block tables of width {width} cannot hold {needed} pages")
     tables = []
     for g in range(n_groups):
-        width = max(-(-int(kv) // ps) for kv in kv_len)
         t = np.full((num_seqs, width), -1, dtype=np.int64)
         for s, c in enumerate(chunks):
             pages = manager.table(c.key, g)
@@ -148,22 +168,36 @@ def build_step(chunks: list, manager, vocab_size: int, max_positions: int, devic
     parts = [ids, positions, token_seq, cu, kv_len, np.asarray(slots, dtype=np.int64),
              np.asarray(rows, dtype=np.int64)] + [t.reshape(-1) for t in tables]
     sizes = [p.size for p in parts]
-    packed = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=pinned and torch.device(device).type == "cuda")
-    np.concatenate(parts, out=packed.numpy().view(np.int32).reshape(-1), casting="unsafe")
-    on_device = packed.to(device, non_blocking=True)
+    host = torch.empty(sum(sizes), dtype=torch.int32, pin_memory=pinned)
+    np.concatenate(parts, out=host.numpy().reshape(-1), casting="unsafe")
+    spans = [(int(cu[s]), counts[s], int(starts[s])) for s in range(num_seqs)]
+    fresh = [slots[s] for s in range(num_seqs) if starts[s] == 0]
+    return PackedStep(host, sizes, total, num_seqs, len(rows), [width] * n_groups, spans,
+                      max(counts), int(kv_len.max()), fresh)
+
+
+def context_from_packed(packed: PackedStep, on_device: torch.Tensor) -> StepContext:
+    """Slice a step context out of the device copy of a packed step."""
     views, offset = [], 0
-    for size in sizes:
+    for size in packed.sizes:
         views.append(on_device[offset:offset + size])
         offset += size
-
     step = StepContext()
-    step.num_tokens, step.num_seqs, step.num_logit_rows = total, num_seqs, len(rows)
+    step.num_tokens, step.num_seqs, step.num_logit_rows = packed.num_tokens, packed.num_seqs, packed.num_rows
     (step.token_ids, step.positions, step.token_seq, step.cu_q, step.kv_len, step.state_slots,
      step.logit_rows) = views[:7]
-    step.block_tables = [views[7 + g].view(num_seqs, tables[g].shape[1]) for g in range(n_groups)]
-    step.spans = [(int(cu[s]), counts[s], int(starts[s])) for s in range(num_seqs)]
-    step.max_q_len, step.max_kv_len = max(counts), int(kv_len.max())
+    step.block_tables = [views[7 + g].view(packed.num_seqs, w) for g, w in enumerate(packed.widths)]
+    step.spans = packed.spans
+    step.max_q_len, step.max_kv_len = packed.max_q_len, packed.max_kv_len
     step.all_decode = step.max_q_len == 1
-    step.fresh_slots = [slots[s] for s in range(num_seqs) if starts[s] == 0]
-    step._packed_host = packed  # keeps the pinned buffer alive until the copy has run
+    step.fresh_slots = packed.fresh_slots
+    step._packed_host = packed.host  # keeps the pinned buffer alive until the copy has run
     return step
+
+
+def build_step(chunks: list, manager, vocab_size: int, max_positions: int, device,
+               pinned: bool = True) -> StepContext:
+    """Pack `chunks`, copy the buffer to the device once, and slice the context out of it."""
+    packed = pack_step(chunks, manager, vocab_size, max_positions,
+                       pinned and torch.device(device).type == "cuda")
+    return context_from_packed(packed, packed.host.to(device, non_blocking=True))

@@ -105,7 +105,8 @@ class Engine:
             cfg.validate_against(model.max_positions or cfg.max_model_len)
         manager = CacheManager(model.cache_slots, cfg.num_blocks, cfg.block_size, cfg.max_running,
                                has_state)
-        runner = ModelRunner(model, manager, cfg.torch_dtype, device, cfg.max_model_len)
+        runner = ModelRunner(model, manager, cfg.torch_dtype, device, cfg.max_model_len,
+                             use_graphs=cfg.use_graphs)
         return GpuExecutor(runner, Sampler(cfg.seed)), manager, model.eos_token_ids
 
     # ---------------------------------------------------------------- lifecycle

@@ -39,15 +39,13 @@ class GpuExecutor:
         for w in plan.work:
             tokens = w.request.tokens[w.start:w.start + w.count]
             chunks.append(SeqChunk(w.request.rid, tokens, w.start, [w.count - 1] if w.emits else []))
-        ctx = self.runner.build(chunks)
-        prepared = time.perf_counter()
-        logits = self.runner.run(ctx)
+        logits = self.runner.step(chunks)
         emitting = [w.request for w in plan.work if w.emits]
         sampled = iter(self.sampler.sample(logits, emitting))
         result = ExecResult(tokens=[next(sampled) if w.emits else None for w in plan.work])
         torch.cuda.synchronize()
-        result.prepare_seconds = prepared - started
-        result.forward_seconds = time.perf_counter() - prepared
+        result.prepare_seconds = self.runner.last_prepare_seconds
+        result.forward_seconds = time.perf_counter() - started - result.prepare_seconds
         return result
 
     def snapshot(self) -> dict:

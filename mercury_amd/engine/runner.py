@@ -13,7 +13,41 @@ from __future__ import annotations
 import torch
 
 from ..parts.base import LayerCache
-from .batch import SeqChunk, StepContext, build_step
+from .batch import SeqChunk, StepContext, build_step, context_from_packed, pack_step
+
+
+class DecodeGraph:
+    """One captured HIP graph of a decode-only step (one token per sequence) for a fixed
+    number of sequences and a fixed bound on their length.
+
+    The step's index tensors live in one static device buffer that every replay refills with a
+    single copy; block tables have the full width of the longest sequence the engine allows,
+    and the number of key splits of the attention kernel is the one chosen for the length
+    bound, so any shorter step replays the same launches.
+    """
+
+    def __init__(self, runner, packed, kv_bound: int):
+        self.layout = packed.layout()
+        self.static = torch.empty(packed.host.shape, dtype=torch.int32, device=runner.device)
+        self.static.copy_(packed.host, non_blocking=True)
+        self.ctx = context_from_packed(packed, self.static)
+        self.ctx.max_kv_len = kv_bound
+        self.ctx.fresh_slots = []
+        # Once outside the capture: loads libraries, fills the context's tile tables.
+        side = torch.cuda.Stream(device=runner.device)
+        side.wait_stream(torch.cuda.current_stream(runner.device))
+        with torch.cuda.stream(side):
+            runner.model.forward(self.ctx, runner.caches, runner.states)
+        torch.cuda.current_stream(runner.device).wait_stream(side)
+        torch.cuda.synchronize(runner.device)
+        self.graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(self.graph):
+            self.logits = runner.model.forward(self.ctx, runner.caches, runner.states)
+
+    def replay(self, packed) -> torch.Tensor:
+        self.static.copy_(packed.host, non_blocking=True)
+        self.graph.replay()
+        return self.logits
 
 
 def require_gpu(device: torch.device) -> None:
@@ -25,9 +59,15 @@ def require_gpu(device: torch.device) -> None:
 
 
 class ModelRunner:
-    def __init__(self, model, manager, dtype: torch.dtype, device, max_model_len: int):
+    def __init__(self, model, manager, dtype: torch.dtype, device, max_model_len: int,
+                 use_graphs: bool = True, max_graph_batch: int = 256):
         device = torch.device(device)
         require_gpu(device)
+        self.graphs: dict = {}
+        self.use_graphs = bool(use_graphs) and all(
+            getattr(layer.mixer, "graph_safe", False) for layer in model.layers)
+        self.max_graph_batch = int(max_graph_batch)
+        self.last_prepare_seconds = 0.0
         self.model, self.manager = model, manager
         self.dtype, self.device = dtype, device
         self.max_model_len = int(max_model_len)
@@ -72,9 +112,40 @@ class ModelRunner:
     @torch.inference_mode()
     def step(self, chunks: list) -> torch.Tensor:
         """Run the chunks' tokens as one batch.  Returns float32 logits [wanted, V] in the
-        order of the chunks and of each chunk's `want`."""
+        order of the chunks and of each chunk's `want`.  The tensor may be overwritten by the
+        next step."""
+        import time
+
+        started = time.perf_counter()
+        if self._graphable(chunks):
+            return self.step_graphed(chunks, started)
         ctx = self.build(chunks)
+        self.last_prepare_seconds = time.perf_counter() - started
         return self.run(ctx)
+
+    def _graphable(self, chunks: list) -> bool:
+        return (self.use_graphs and len(chunks) <= self.max_graph_batch
+                and all(len(c.tokens) == 1 and c.want == [0] and c.start > 0 for c in chunks))
+
+    @torch.inference_mode()
+    def step_graphed(self, chunks: list, started: float | None = None) -> torch.Tensor:
+        """A decode-only step through a captured graph (captured on first use for this number
+        of sequences and length bound)."""
+        width = -(-self.max_model_len // self.page_size)
+        packed = pack_step(chunks, self.manager, self.model.vocab_size, self.max_model_len,
+                           pinned=True, table_width=width)
+        bound = 256
+        while bound < packed.max_kv_len:
+            bound *= 2
+        key = (len(chunks), bound)
+        graph = self.graphs.get(key)
+        if graph is None:
+            graph = self.graphs[key] = DecodeGraph(self, packed, bound)
+        if started is not None:
+            import time
+
+            self.last_prepare_seconds = time.perf_counter() - started
+        return graph.replay(packed)
 
     @torch.inference_mode()
     def run(self, ctx: StepContext) -> torch.Tensor:

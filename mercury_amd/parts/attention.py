@@ -19,6 +19,8 @@ class Attention(Mixer):
     Tensor names follow the checkpoint: ``q_proj``, ``k_proj``, ``v_proj``, ``o_proj``.
     """
 
+    graph_safe = True   # forward launches kernels only: a decode step may be captured in a graph
+
     def __init__(self, hidden: int, n_q: int, n_kv: int, head_dim: int,
                  position: PositionEncoding, qkv_bias: bool = True, o_bias: bool = False,
                  scale: float | None = None, window: int | None = None):

@@ -123,6 +123,11 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
+    # True when forward() only launches kernels on the current stream (no host reads of device
+    # data, no host-side branching on them), so a decode step through it can be captured in a
+    # HIP graph and replayed.
+    graph_safe = False
+
     def cache_spec(self) -> CacheSpec | None:
         return None
 

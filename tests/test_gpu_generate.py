@@ -157,3 +157,18 @@ def test_smoke_entry_point():
     import __graft_entry__
 
     __graft_entry__.smoke()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_captured_decode_graphs_replay_like_eager_steps(dtype):
+    """Decode steps run through captured HIP graphs.  Replays of one graph, with other work
+    (prompts, other batch sizes, synchronisations) between them, give the tokens of an engine
+    that never captures."""
+    prompts = [PROMPT, OTHER, PROMPT[:33], OTHER[:7]]
+    eager = generate(engine(dtype=dtype, use_graphs=False), prompts, 40)
+    graphed_engine = engine(dtype=dtype, use_graphs=True)
+    assert generate(graphed_engine, prompts, 40) == eager
+    assert len(graphed_engine.runner.runner.graphs) >= 1
+    # the same graphs again, after unrelated work in between
+    assert generate(graphed_engine, prompts[:2], 20) == [e[:20] for e in eager[:2]]
+    assert generate(graphed_engine, prompts, 40) == eager
