@@ -105,31 +105,43 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p
 
   for (int b = b0; b < b1; ++b) {
     const int key0 = b << 5;
-    float s[8];
-    size_t vbase[2];
+    // Addresses first, then every load of the block (keys and values) before any use, so
+    // that one trip to memory covers them all.
     bool live[2];
+    const bf16_t* krow[2];
+    const bf16_t* vrow[2];
 #pragma unroll
     for (int h = 0; h < 2; ++h) {
       const int kh = key0 + h * 16;
       live[h] = kh <= kmax && kh + 15 >= kmin;  // the same for the whole wavefront
-      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
-      vbase[h] = 0;
-      if (live[h]) {
-        const int page = table[kh >> p.page_shift];
-        const int off = kh & (ps - 1);
-        const size_t head_base = (size_t)page * p.n_kv + kvh;
-        vbase[h] = head_base * ps * D + off;
-        const bf16_t* krow = p.k_cache + (head_base * ps + off + r) * D + g4 * 8;
+      const int page = live[h] ? table[kh >> p.page_shift] : 0;
+      const int off = kh & (ps - 1);
+      const size_t head_base = (size_t)page * p.n_kv + kvh;
+      krow[h] = p.k_cache + (head_base * ps + off + r) * D + g4 * 8;
+      vrow[h] = p.v_cache + head_base * ps * D + off + (size_t)r * ps + g4 * 4;
+    }
+    Frag kf[2][D / 32], vf[D / 16];
 #pragma unroll
-        for (int c = 0; c < D / 32; ++c) {
-          Frag kf;
-          kf.u = *(const uint4*)(krow + c * 32);
-          sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf.v, qf[c].v, sc, 0, 0, 0);
-        }
-      }
+    for (int h = 0; h < 2; ++h)
+#pragma unroll
+      for (int c = 0; c < D / 32; ++c)
+        kf[h][c].u = live[h] ? *(const uint4*)(krow[h] + c * 32) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt)
+#pragma unroll
+      for (int h = 0; h < 2; ++h)
+        vf[dt].u2[h] = live[h] ? *(const uint2*)(vrow[h] + (size_t)dt * 16 * ps) : make_uint2(0, 0);
+
+    float s[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int c = 0; c < D / 32; ++c)
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[h][c].v, qf[c].v, sc, 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        const int key = kh + g4 * 4 + i;
+        const int key = key0 + h * 16 + g4 * 4 + i;
         const bool ok = live[h] && row_ok && key <= pos && key >= lo;
         s[h * 4 + i] = ok ? sc[i] * p.scale : -INFINITY;
       }
@@ -156,14 +168,7 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p
 #pragma unroll
     for (int dt = 0; dt < D / 16; ++dt) {
       acc[dt] *= corr;
-      Frag vf;
-#pragma unroll
-      for (int h = 0; h < 2; ++h) {
-        vf.u2[h] = make_uint2(0, 0);
-        if (live[h])
-          vf.u2[h] = *(const uint2*)(p.v_cache + vbase[h] + (size_t)(dt * 16 + r) * ps + g4 * 4);
-      }
-      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf.v, pf.v, acc[dt], 0, 0, 0);
+      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, acc[dt], 0, 0, 0);
     }
   }
 
@@ -197,31 +202,58 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p
   }
 }
 
-// Merge the key splits of every (tile, kv head, row): the maximum of the running maxima,
-// then the sums and partial results rescaled to it, in split order.
+// Merge the key splits of one (tile, kv head, row) per workgroup: the maximum of the running
+// maxima, then the sums and the partial results rescaled to it.  Thread (g, dim) adds the
+// splits g, g + 4, ... of its dim, four loads in flight at a time; the four groups are then
+// added in order, so the result does not depend on timing.
 template <int D>
 __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
-  const int tile = blockIdx.x, kvh = blockIdx.y;
+  __shared__ float weight[1024];
+  __shared__ float group_sum[4][D];
+  __shared__ float scratch[16];
+  const int tile = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z;
   const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
   const int G = p.group;
-  const size_t base = ((size_t)tile * p.n_kv + kvh) * p.num_splits;
-  for (int idx = threadIdx.x; idx < 16 * D; idx += blockDim.x) {
-    const int r = idx / D, dim = idx - r * D;
-    const int flat = row0 + r;
-    if (flat >= q_len * G) continue;
-    float mx = -INFINITY;
-    for (int s = 0; s < p.num_splits; ++s) mx = fmaxf(mx, p.part_ml[((base + s) * 16 + r) * 2]);
-    float total = 0.f, o = 0.f;
-    for (int s = 0; s < p.num_splits; ++s) {
-      const size_t slot = (base + s) * 16 + r;
-      const float ms = p.part_ml[slot * 2];
-      if (ms == -INFINITY) continue;
-      const float w = __expf(ms - mx);
-      total += p.part_ml[slot * 2 + 1] * w;
-      o += p.part_o[slot * D + dim] * w;
+  const int flat = row0 + r;
+  if (flat >= q_len * G) return;
+  const int S = p.num_splits;
+  const size_t base = ((size_t)tile * p.n_kv + kvh) * S;
+
+  float mx = -INFINITY;
+  for (int s = threadIdx.x; s < S; s += blockDim.x)
+    mx = fmaxf(mx, p.part_ml[((base + s) * 16 + r) * 2]);
+  mx = block_max(mx, scratch);
+  float part = 0.f;
+  for (int s = threadIdx.x; s < S; s += blockDim.x) {
+    const size_t slot = (base + s) * 16 + r;
+    const float ms = p.part_ml[slot * 2];
+    const float w = ms == -INFINITY ? 0.f : __expf(ms - mx);
+    weight[s] = w;
+    part += p.part_ml[slot * 2 + 1] * w;
+  }
+  const float total = block_sum(part, scratch);  // also orders the writes of weight[]
+
+  const int g = threadIdx.x >> 6;
+  for (int dim = threadIdx.x & 63; dim < D; dim += 64) {
+    const float* src = p.part_o + ((base * 16) + r) * D + dim;
+    const size_t stride = (size_t)16 * D;
+    float o = 0.f;
+    int s = g;
+    for (; s + 12 < S; s += 16) {
+      const float a = src[(size_t)s * stride] * weight[s];
+      const float b = src[(size_t)(s + 4) * stride] * weight[s + 4];
+      const float c = src[(size_t)(s + 8) * stride] * weight[s + 8];
+      const float d = src[(size_t)(s + 12) * stride] * weight[s + 12];
+      o += (a + b) + (c + d);
     }
-    const int tok = flat / G, head = kvh * G + flat % G;
+    for (; s < S; s += 4) o += src[(size_t)s * stride] * weight[s];
+    group_sum[g][dim] = o;
+  }
+  __syncthreads();
+  const int tok = flat / G, head = kvh * G + flat % G;
+  for (int dim = threadIdx.x; dim < D; dim += blockDim.x) {
+    const float o = (group_sum[0][dim] + group_sum[1][dim]) + (group_sum[2][dim] + group_sum[3][dim]);
     p.out[(size_t)(q0 + tok) * p.out_stride + head * D + dim] = f32_to_bf16(o / total);
   }
 }
@@ -231,7 +263,7 @@ static void launch_attn(const AttnParams& p, hipStream_t stream) {
   dim3 grid((p.num_tiles + ATTN_WAVES - 1) / ATTN_WAVES, p.n_kv, p.num_splits);
   attn_mfma_kernel<D><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
   if (p.num_splits > 1) {
-    dim3 mgrid(p.num_tiles, p.n_kv);
+    dim3 mgrid(p.num_tiles, p.n_kv, 16);
     attn_merge_kernel<D><<<mgrid, 256, 0, stream>>>(p);
   }
 }
@@ -256,7 +288,7 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
              "attention (matrix cores): head size %d / page size %d not supported; head sizes "
              "32, 64, 96, 128, 192, 256 and pages of 16 or more are",
              d, page_size);
-  MK_REQUIRE(num_splits >= 1 && num_splits <= 65535 && n_kv <= 65535, "attention: bad grid");
+  MK_REQUIRE(num_splits >= 1 && num_splits <= 1024 && n_kv <= 65535, "attention: bad grid");
   MK_REQUIRE(num_splits == 1 || (part_o && part_ml), "attention: key splits need a workspace");
   MK_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0,
              "attention: row strides %d/%d break 16-byte alignment", q_stride, out_stride);

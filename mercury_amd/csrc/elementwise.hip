@@ -38,6 +38,20 @@ extern "C" int mk_embed(const int* ids, const void* table, int dtype, float* out
 
 // --------------------------------------------------------------------------------- RMSNorm
 
+// Sum of p[0], p[stride], ..., p[(n-1) stride], four loads in flight at a time; the order of
+// the additions is fixed: ((p0 + p1) + (p2 + p3)) per group, groups in ascending order.
+__device__ __forceinline__ float sum_partials(const float* __restrict__ p, int n, size_t stride) {
+  float total = 0.f;
+  int k = 0;
+  for (; k + 4 <= n; k += 4) {
+    const float a = p[(size_t)k * stride], b = p[(size_t)(k + 1) * stride];
+    const float c = p[(size_t)(k + 2) * stride], d = p[(size_t)(k + 3) * stride];
+    total += (a + b) + (c + d);
+  }
+  for (; k < n; ++k) total += p[(size_t)k * stride];
+  return total;
+}
+
 // One block per output row.  h is the float32 residual stream.  When `partials` is given,
 // the P partial sums of the preceding projection are first added into h (in the order
 // 0..P-1) and written back, so the residual sum and the norm are one pass.
@@ -57,8 +71,7 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ 
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
     float v = x[i];
     if (num_partials > 0) {
-      const float* p = partials + (size_t)in_row * hidden + i;
-      for (int k = 0; k < num_partials; ++k) v += p[(size_t)k * partial_stride];
+      v += sum_partials(partials + (size_t)in_row * hidden + i, num_partials, partial_stride);
       x[i] = v;
     }
     sq += v * v;
@@ -77,7 +90,8 @@ static int launch_rmsnorm(float* h, const float* partials, int num_partials,
                           size_t partial_stride, const void* weight, int weight_dtype, float eps,
                           const int* rows, TO* out, int out_rows, int hidden,
                           hipStream_t stream) {
-  const int threads = hidden >= 1024 ? 256 : (hidden >= 256 ? 128 : 64);
+  // Few rows (decoding): more threads per row, so that every thread has few loads to wait for.
+  const int threads = hidden >= 512 ? 256 : (hidden >= 256 ? 128 : 64);
   if (weight_dtype == MK_F32)
     rmsnorm_kernel<TO, float><<<out_rows, threads, 0, stream>>>(
         h, partials, num_partials, partial_stride, (const float*)weight, eps, rows, out, hidden);
@@ -255,11 +269,8 @@ __global__ void silu_mul_partials_kernel(const float* __restrict__ partials, int
     const size_t t = idx / inter;
     const int i = (int)(idx - t * inter);
     const float* row = partials + t * 2 * (size_t)inter;
-    float g = 0.f, u = 0.f;
-    for (int p = 0; p < num_partials; ++p) {
-      g += row[p * partial_stride + i];
-      u += row[p * partial_stride + inter + i];
-    }
+    float g = sum_partials(row + i, num_partials, partial_stride);
+    float u = sum_partials(row + inter + i, num_partials, partial_stride);
     // The reference rounds both projections to the storage type before gating.
     g = Elem<T>::round(g);
     u = Elem<T>::round(u);
@@ -302,6 +313,7 @@ __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_pa
                                   T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   int page_shift, int n_q, int n_kv, int d, int rot,
                                   int write_kv) {
+  extern __shared__ float vals[];  // the token's summed, biased, rounded projection row
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = rot / 2;
@@ -309,23 +321,21 @@ __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_pa
   const float* sn = sin_table + (size_t)pos * half;
   const int width = (n_q + 2 * n_kv) * d;
   const float* row = partials + (size_t)t * width;
-  auto value = [&](int col) {
-    float v = 0.f;
-    for (int p = 0; p < num_partials; ++p) v += row[p * partial_stride + col];
+  for (int col = threadIdx.x; col < width; col += blockDim.x) {
+    float v = sum_partials(row + col, num_partials, partial_stride);
     if (bias) v += Elem<TB>::load(bias + col);
-    return Elem<T>::round(v);
-  };
+    vals[col] = Elem<T>::round(v);
+  }
+  __syncthreads();
 
+  auto rotated = [&](int base, int j) {
+    if (j < half) return vals[base + j] * cs[j] - vals[base + j + half] * sn[j];
+    if (j < rot) return vals[base + j] * cs[j - half] + vals[base + j - half] * sn[j - half];
+    return vals[base + j];
+  };
   for (int idx = threadIdx.x; idx < n_q * d; idx += blockDim.x) {
     const int head = idx / d, j = idx - head * d;
-    float y;
-    if (j < half)
-      y = value(idx) * cs[j] - value(idx + half) * sn[j];
-    else if (j < rot)
-      y = value(idx) * cs[j - half] + value(idx - half) * sn[j - half];
-    else
-      y = value(idx);
-    Elem<T>::store(q_out + (size_t)t * n_q * d + idx, y);
+    Elem<T>::store(q_out + (size_t)t * n_q * d + idx, rotated(head * d, j));
   }
   if (!write_kv) return;
 
@@ -336,16 +346,10 @@ __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_pa
   const int k0 = n_q * d, v0 = (n_q + n_kv) * d;
   for (int idx = threadIdx.x; idx < n_kv * d; idx += blockDim.x) {
     const int head = idx / d, j = idx - head * d;
-    float y;
-    if (j < half)
-      y = value(k0 + idx) * cs[j] - value(k0 + idx + half) * sn[j];
-    else if (j < rot)
-      y = value(k0 + idx) * cs[j - half] + value(k0 + idx - half) * sn[j - half];
-    else
-      y = value(k0 + idx);
-    Elem<T>::store(k_cache + (((size_t)page * n_kv + head) * page_size + off) * d + j, y);
+    Elem<T>::store(k_cache + (((size_t)page * n_kv + head) * page_size + off) * d + j,
+                   rotated(k0 + head * d, j));
     Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * d + j) * page_size + off,
-                   value(v0 + idx));
+                   vals[v0 + idx]);
   }
 }
 
@@ -364,8 +368,11 @@ extern "C" int mk_qkv_finish(const float* partials, int num_partials, long long 
   MK_REQUIRE(dtype == MK_BF16 || dtype == MK_F32, "qkv_finish: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   const int shift = mk_log2(page_size);
+  const size_t lds_bytes = (size_t)(n_q + 2 * n_kv) * d * sizeof(float);
+  MK_REQUIRE(lds_bytes <= 64 * 1024, "qkv_finish: a projection row of %zu bytes exceeds LDS",
+             lds_bytes);
 #define QKV_LAUNCH(T, TB)                                                                      \
-  qkv_finish_kernel<T, TB><<<tokens, 256, 0, stream>>>(                                        \
+  qkv_finish_kernel<T, TB><<<tokens, 256, lds_bytes, stream>>>(                                        \
       partials, num_partials, (size_t)partial_stride, (const TB*)bias, (T*)q_out, cos_table,   \
       sin_table, positions, token_seq, block_table, table_stride, (T*)k_cache, (T*)v_cache,    \
       shift, n_q, n_kv, d, rot, write_kv)
