@@ -90,8 +90,10 @@ static int launch_rmsnorm(float* h, const float* partials, int num_partials,
                           size_t partial_stride, const void* weight, int weight_dtype, float eps,
                           const int* rows, TO* out, int out_rows, int hidden,
                           hipStream_t stream) {
-  // Few rows (decoding): more threads per row, so that every thread has few loads to wait for.
-  const int threads = hidden >= 512 ? 256 : (hidden >= 256 ? 128 : 64);
+  // Few rows (decoding): as many threads per row as it has elements, so that every thread
+  // waits for one group of loads only.
+  int threads = hidden >= 512 ? 256 : (hidden >= 256 ? 128 : 64);
+  if (out_rows <= 64 && num_partials > 0) threads = hidden >= 1024 ? 1024 : (hidden + 63) / 64 * 64;
   if (weight_dtype == MK_F32)
     rmsnorm_kernel<TO, float><<<out_rows, threads, 0, stream>>>(
         h, partials, num_partials, partial_stride, (const float*)weight, eps, rows, out, hidden);
@@ -369,10 +371,11 @@ extern "C" int mk_qkv_finish(const float* partials, int num_partials, long long 
   if (tokens == 0) return 0;
   const int shift = mk_log2(page_size);
   const size_t lds_bytes = (size_t)(n_q + 2 * n_kv) * d * sizeof(float);
+  const int threads = tokens <= 64 ? 1024 : 256;
   MK_REQUIRE(lds_bytes <= 64 * 1024, "qkv_finish: a projection row of %zu bytes exceeds LDS",
              lds_bytes);
 #define QKV_LAUNCH(T, TB)                                                                      \
-  qkv_finish_kernel<T, TB><<<tokens, 256, lds_bytes, stream>>>(                                        \
+  qkv_finish_kernel<T, TB><<<tokens, threads, lds_bytes, stream>>>(                                        \
       partials, num_partials, (size_t)partial_stride, (const TB*)bias, (T*)q_out, cos_table,   \
       sin_table, positions, token_seq, block_table, table_stride, (T*)k_cache, (T*)v_cache,    \
       shift, n_q, n_kv, d, rot, write_kv)

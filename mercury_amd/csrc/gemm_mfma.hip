@@ -4,11 +4,13 @@
 //
 //  * skinny (M <= 64, decoding): the weights are read once, straight from HBM into the A
 //    operand of v_mfma_f32_16x16x32_bf16 (16 rows of W by 32 k per instruction); the few rows
-//    of x are the B operand and come out of the L2.  One wavefront owns 32 rows of W and one
-//    slice of K.  Splitting K gives the small matrices of a small model enough wavefronts to
-//    pull their bytes; every slice writes its own float32 partial result [slice, M, N], and
-//    whichever kernel consumes the projection (RMSNorm, rotary + cache write, SiLU gating)
-//    adds the slices up in slice order, so results are reproducible.
+//    of x are the B operand and come out of the L2.  A workgroup owns 32 rows of W and one
+//    slice of K, its wavefronts taking the slice's k-steps in turn.  Splitting K gives the
+//    small matrices of a small model enough wavefronts to pull their bytes; every slice
+//    writes its own float32 partial result [slice, M, N], and whichever kernel consumes the
+//    projection (RMSNorm, rotary + cache write) adds the slices up in slice order, so results
+//    are reproducible.  The gate/up projection keeps all of K in one workgroup and gates in
+//    its epilogue.
 //
 //  * tiled (M > 64, prompts): 128 x 128 tiles of y per workgroup, K in steps of 32 through
 //    LDS with the next step's global loads in flight during the current step's products;
@@ -33,23 +35,33 @@ __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *(const uint4*)p
 
 // ------------------------------------------------------------------------------ skinny
 
-#define SK_NT 2  // 16-row tiles of W per wavefront
+#define SK_NT 2     // 16-row tiles of W per workgroup
+#define SK_WAVES 4  // wavefronts of a workgroup; they share the rows and split the k-steps
 
-// out[(slice * M + m) * N + n]; K % 8 == 0; a slice covers k_per_slice (a multiple of 128).
-template <int MT>
-__global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restrict__ x,
-                                                          const bf16_t* __restrict__ w,
-                                                          float* __restrict__ out, int M, int N,
-                                                          int K, int k_per_slice) {
-  const int lane = threadIdx.x & 63, r = lane & 15, g4 = lane >> 4;
-  const int n0 = (blockIdx.x * 4 + (threadIdx.x >> 6)) * (16 * SK_NT);
-  if (n0 >= N) return;
+// Each workgroup owns 32 rows of W (two 16-row tiles) and one slice of K; its four wavefronts
+// take the slice's 128-wide k-steps in turn (wave w: steps w, w + 4, ...) and add their
+// results up through LDS in wave order, so a slice yields one partial result.
+//   GATED = 0: out[(slice * M + m) * N + n] float32, tiles are rows n0.. and n0 + 16..
+//   GATED = 1: W is [gate rows | up rows] of N each; the two tiles are gate rows n0.. and the
+//              matching up rows N + n0.., the slice must be all of K, and the epilogue writes
+//              act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
+template <int MT, int GATED>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(
+    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out_, int M,
+    int N, int K, int steps_per_slice) {
+  __shared__ float red[SK_WAVES - 1][SK_NT * MT * 4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g4 = lane >> 4;
+  const int n0 = blockIdx.x * (GATED ? 16 : 16 * SK_NT);
   const int slice = blockIdx.y;
-  const int k_begin = slice * k_per_slice, k_end = min(K, k_begin + k_per_slice);
+  const int step_begin = slice * steps_per_slice;
+  const int step_end = min((K + 127) / 128, step_begin + steps_per_slice);
 
   const bf16_t* wrow[SK_NT];
 #pragma unroll
-  for (int t = 0; t < SK_NT; ++t) wrow[t] = w + (size_t)min(n0 + t * 16 + r, N - 1) * K;
+  for (int t = 0; t < SK_NT; ++t) {
+    const int row = GATED ? t * N + min(n0 + r, N - 1) : min(n0 + t * 16 + r, N - 1);
+    wrow[t] = w + (size_t)row * K;
+  }
   const bf16_t* xrow[MT];
 #pragma unroll
   for (int t = 0; t < MT; ++t) xrow[t] = x + (size_t)min(t * 16 + r, M - 1) * K;
@@ -60,12 +72,12 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
 #pragma unroll
     for (int b = 0; b < MT; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  for (int k0 = k_begin; k0 < k_end; k0 += 128) {
-    const int kk = k0 + g4 * 32;  // this lane's 32 k of the 128
+  for (int step = step_begin + wave; step < step_end; step += SK_WAVES) {
+    const int kk = step * 128 + g4 * 32;  // this lane's 32 k of the step's 128
     Frag a[SK_NT][4], b[MT][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const bool ok = kk + j * 8 < k_end;
+      const bool ok = kk + j * 8 < K;
 #pragma unroll
       for (int t = 0; t < SK_NT; ++t)
         a[t][j].u = ok ? ld16(wrow[t] + kk + j * 8) : make_uint4(0, 0, 0, 0);
@@ -83,40 +95,89 @@ __global__ __launch_bounds__(256) void gemm_skinny_kernel(const bf16_t* __restri
                                                                 acc[ta][tb], 0, 0, 0);
   }
 
-  // acc[ta][tb][i] = y[m = tb*16 + r][n = n0 + ta*16 + g4*4 + i]
+  if (wave > 0) {
+#pragma unroll
+    for (int ta = 0; ta < SK_NT; ++ta)
+#pragma unroll
+      for (int tb = 0; tb < MT; ++tb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) red[wave - 1][(ta * MT + tb) * 4 + i][lane] = acc[ta][tb][i];
+  }
+  __syncthreads();
+  if (wave > 0) return;
+#pragma unroll
+  for (int v = 0; v < SK_WAVES - 1; ++v)
+#pragma unroll
+    for (int ta = 0; ta < SK_NT; ++ta)
+#pragma unroll
+      for (int tb = 0; tb < MT; ++tb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i) acc[ta][tb][i] += red[v][(ta * MT + tb) * 4 + i][lane];
+
+  // acc[ta][tb][i] = y[m = tb*16 + r][column g4*4 + i of tile ta]
 #pragma unroll
   for (int tb = 0; tb < MT; ++tb) {
     const int m = tb * 16 + r;
     if (m >= M) continue;
-    float* dst = out + ((size_t)slice * M + m) * N;
+    if (GATED) {
+      bf16_t* dst = (bf16_t*)out_ + (size_t)m * N;
+      const int n = n0 + g4 * 4;
+      bf16_t o[4];
 #pragma unroll
-    for (int ta = 0; ta < SK_NT; ++ta) {
-      const int n = n0 + ta * 16 + g4 * 4;
+      for (int i = 0; i < 4; ++i) {
+        const float g = Elem<bf16_t>::round(acc[0][tb][i]), u = Elem<bf16_t>::round(acc[1][tb][i]);
+        o[i] = f32_to_bf16(Elem<bf16_t>::round(g / (1.f + expf(-g))) * u);
+      }
       if (n + 3 < N && (N & 3) == 0) {
-        *(float4*)(dst + n) =
-            make_float4(acc[ta][tb][0], acc[ta][tb][1], acc[ta][tb][2], acc[ta][tb][3]);
+        *(ushort4*)(dst + n) = make_ushort4(o[0], o[1], o[2], o[3]);
       } else {
 #pragma unroll
         for (int i = 0; i < 4; ++i)
-          if (n + i < N) dst[n + i] = acc[ta][tb][i];
+          if (n + i < N) dst[n + i] = o[i];
+      }
+    } else {
+      float* dst = (float*)out_ + ((size_t)slice * M + m) * N;
+#pragma unroll
+      for (int ta = 0; ta < SK_NT; ++ta) {
+        const int n = n0 + ta * 16 + g4 * 4;
+        if (n + 3 < N && (N & 3) == 0) {
+          *(float4*)(dst + n) =
+              make_float4(acc[ta][tb][0], acc[ta][tb][1], acc[ta][tb][2], acc[ta][tb][3]);
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) dst[n + i] = acc[ta][tb][i];
+        }
       }
     }
   }
 }
 
+// Slices of K for the plain skinny projection: enough workgroups to fill the chip (about
+// 512), every wavefront of a workgroup with at least one k-step, and no more partial results
+// than the weights are worth (slices * M * 4 bytes per output column against K * 2).
 extern "C" int mk_linear_skinny_slices(int M, int N, int K) {
-  // Enough slices of K (each a multiple of 128) for about 1024 wavefronts, but no more
-  // partial results than the weights are worth: slices * M * 4 bytes per output column
-  // against K * 2 bytes of weights.
   const int tiles = (N + 16 * SK_NT - 1) / (16 * SK_NT);
   const int steps = (K + 127) / 128;
-  int slices = (1024 + tiles - 1) / tiles;
-  if (slices > steps) slices = steps;
+  int slices = (512 + tiles - 1) / tiles;
+  const int by_steps = (steps + SK_WAVES - 1) / SK_WAVES;
+  if (slices > by_steps) slices = by_steps;
   const int cap = K / (8 * (M > 0 ? M : 1));
   if (slices > cap) slices = cap;
   if (slices < 1) slices = 1;
-  const int per = ((steps + slices - 1) / slices);
+  const int per = (steps + slices - 1) / slices;
   return (steps + per - 1) / per;
+}
+
+template <int GATED>
+static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K,
+                          int per, dim3 grid, hipStream_t stream) {
+  switch ((M + 15) / 16) {
+    case 1: gemm_skinny_kernel<1, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
+    case 2: gemm_skinny_kernel<2, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
+    case 3: gemm_skinny_kernel<3, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
+    default: gemm_skinny_kernel<4, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
+  }
 }
 
 extern "C" int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int K,
@@ -129,16 +190,23 @@ extern "C" int mk_linear_skinny(const void* x, const void* w, float* out, int M,
   const int per = (steps + slices - 1) / slices;
   MK_REQUIRE((per * (slices - 1)) < steps, "skinny projection: an empty slice");
   const int tiles = (N + 16 * SK_NT - 1) / (16 * SK_NT);
-  dim3 grid((tiles + 3) / 4, slices);
-  const bf16_t* xp = (const bf16_t*)x;
-  const bf16_t* wp = (const bf16_t*)w;
-  switch ((M + 15) / 16) {
-    case 1: gemm_skinny_kernel<1><<<grid, 256, 0, stream>>>(xp, wp, out, M, N, K, per * 128); break;
-    case 2: gemm_skinny_kernel<2><<<grid, 256, 0, stream>>>(xp, wp, out, M, N, K, per * 128); break;
-    case 3: gemm_skinny_kernel<3><<<grid, 256, 0, stream>>>(xp, wp, out, M, N, K, per * 128); break;
-    default: gemm_skinny_kernel<4><<<grid, 256, 0, stream>>>(xp, wp, out, M, N, K, per * 128); break;
-  }
+  MK_REQUIRE(slices <= 65535, "skinny projection: too many slices");
+  launch_skinny<0>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, per, dim3(tiles, slices),
+                   stream);
   MK_LAUNCH_CHECK("linear_skinny");
+  return 0;
+}
+
+// act[M, I] = silu(x Wg^T) * (x Wu^T) for W = [Wg | Wu] stacked as [2 I, K], 1 <= M <= 64.
+extern "C" int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
+                               hipStream_t stream) {
+  MK_REQUIRE(M >= 1 && M <= 64, "gated projection: M=%d outside 1..64", M);
+  MK_REQUIRE(inter > 0 && K > 0 && K % 8 == 0, "gated projection: K=%d must be a multiple of 8",
+             K);
+  const int steps = (K + 127) / 128;
+  launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, act, M, inter, K, steps,
+                   dim3((inter + 15) / 16, 1), stream);
+  MK_LAUNCH_CHECK("gated_skinny");
   return 0;
 }
 

@@ -71,6 +71,10 @@ int mk_linear_skinny_slices(int M, int N, int K);
 int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int K, int slices,
                      hipStream_t stream);
 
+// act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K].
+int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
+                    hipStream_t stream);
+
 // y = x W^T (+ bias) for any M, tiled through LDS; output bfloat16 or float32, or float32
 // accumulated into `out`.
 int mk_linear_tiled(const void* x, const void* w, const void* bias, int bias_dtype, void* out,

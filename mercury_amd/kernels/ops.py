@@ -164,6 +164,21 @@ def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+    """act = silu(x Wg^T) * (x Wu^T) for few rows of bfloat16 x and W = [Wg | Wu] stacked
+    [2 I, K]: one kernel, the gating in the projection's epilogue."""
+    _dev(x, w_gate_up)
+    if not wants_partials(x, w_gate_up) or x.shape[1] != w_gate_up.shape[1] or w_gate_up.shape[0] % 2:
+        raise KernelArgumentError("gated_projection: operands not eligible")
+    m, k = x.shape
+    inter = w_gate_up.shape[0] // 2
+    act = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
+    lib = _lib.load("mfma")
+    _lib.check(lib, lib.mk_gated_skinny(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream()),
+               "gated_projection")
+    return act
+
+
 def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
            out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
            accumulate: bool = False, kernel: str = "auto") -> torch.Tensor:

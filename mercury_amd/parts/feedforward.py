@@ -42,7 +42,7 @@ class GatedMLP(FeedForward):
 
     def forward(self, x, step, accum):
         if ops.wants_partials(x, self.w_gate_up):
-            act = ops.silu_mul(ops.linear_partials(x, self.w_gate_up), out_dtype=x.dtype)
+            act = ops.gated_projection(x, self.w_gate_up)     # few rows: gated in the epilogue
         else:
             act = ops.silu_mul(ops.linear(x, self.w_gate_up))
         if ops.wants_partials(act, self.w_down):

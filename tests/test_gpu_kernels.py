@@ -178,6 +178,20 @@ def test_tiled_projection(m, n, k):
     torch.testing.assert_close(acc_d.cpu(), acc + want, atol=5e-4, rtol=1e-4)
 
 
+@pytest.mark.parametrize("m,inter,k", [(1, 4864, 896), (8, 410, 168), (33, 704, 256), (64, 176, 64)])
+def test_gated_projection_few_rows(m, inter, k):
+    """silu(x Wg^T) * (x Wu^T) with the gating in the projection's epilogue equals the gating
+    kernel applied to the stored projection."""
+    x_h, x_d = as_dtype(rnd(m, k, seed=31), torch.bfloat16)
+    w_h, w_d = as_dtype(rnd(2 * inter, k, seed=32, scale=0.1), torch.bfloat16)
+    got = ops().gated_projection(x_d, w_d)
+    stored = (x_h.double() @ w_h.double().T).float().to(torch.bfloat16)
+    want = ops().silu_mul(stored.to(DEV))
+    torch.testing.assert_close(got.float().cpu(), want.float().cpu(), atol=2e-3, rtol=1.6e-2)
+    plain_want = plain.gated_mlp(x_h, w_h[:inter], w_h[inter:], torch.eye(inter))
+    torch.testing.assert_close(got.float().cpu(), plain_want, **tol(torch.bfloat16))
+
+
 def test_matrix_core_projection_refuses_what_it_cannot_do():
     from mercury_amd.kernels.ops import KernelArgumentError
 
