@@ -38,8 +38,8 @@ struct AttnParams {
   int q_stride;
   bf16_t* out;
   int out_stride;
-  float* part_o;   // [tile, kv head, split, 16, D]
-  float* part_ml;  // [tile, kv head, split, 16, 2]
+  float* part_o;   // [tile, kv head, split, tile_rows, D]
+  float* part_ml;  // [tile, kv head, split, tile_rows, 2]
   const bf16_t* k_cache;
   const bf16_t* v_cache;
   const int* tile_seq;
@@ -55,15 +55,163 @@ struct AttnParams {
   int window;
   int num_tiles;
   int num_splits;
+  int split_blocks;  // key blocks per split; 0: each tile's range divided evenly
+  int tile_rows;     // rows per tile: 16, 32 or 64
 };
 
 #define ATTN_WAVES 4
+// Blocks of keys in flight beyond the one being used, per tile width (16, 32, 64 rows).
+#ifndef ATTN_AHEAD_16
+#define ATTN_AHEAD_16 1
+#define ATTN_AHEAD_32 1
+#define ATTN_AHEAD_64 0
+#endif
 
+// The keys and values of one block of 32 keys, as MFMA operands of this lane.
 template <int D>
+struct KeyBlock {
+  Frag kf[2][D / 32];
+  Frag vf[D / 16];
+  bool live[2];
+};
+
+// The wavefront's view of its sequence's block table: 64 entries at a time, one per lane,
+// handed out by lane index, so that finding a block's page costs no trip to memory.
+struct TableWindow {
+  const int* table;
+  int width, base, mine;
+  __device__ __forceinline__ int page(int index, int lane) {
+    if (index < base || index >= base + 64) {  // uniform: every lane asks for the same index
+      base = index;
+      mine = index + lane < width ? table[index + lane] : 0;
+    }
+    return __builtin_amdgcn_readlane(mine, index - base);
+  }
+};
+
+// Loads are unconditional: a half that is not live (outside the keys the tile sees, or past
+// the split's end while prefetching) reads page 0, which always exists, and its keys are
+// masked in the scores.  Addresses are a wavefront-uniform base plus a 32-bit lane offset.
+template <int D>
+__device__ __forceinline__ void load_key_block(KeyBlock<D>& blk, const AttnParams& p,
+                                               TableWindow& tw, int b, int b_end, int kmin,
+                                               int kmax, int kvh, int lane) {
+  const int r = lane & 15, g4 = lane >> 4;
+  const int ps = 1 << p.page_shift;
+  const uint32_t k_lane = (uint32_t)(r * D + g4 * 8) * 2u;   // bytes
+  const uint32_t v_lane = (uint32_t)(r * ps + g4 * 4) * 2u;
+  const char* kbase[2];
+  const char* vbase[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int kh = (b << 5) + h * 16;
+    blk.live[h] = b < b_end && kh <= kmax && kh + 15 >= kmin;  // wavefront-uniform
+    const int page = blk.live[h] ? tw.page(kh >> p.page_shift, lane) : 0;
+    const int off = kh & (ps - 1);
+    const size_t head_bytes = ((size_t)page * p.n_kv + kvh) * ((size_t)ps * D * 2);
+    kbase[h] = (const char*)p.k_cache + head_bytes + (size_t)off * D * 2;
+    vbase[h] = (const char*)p.v_cache + head_bytes + (size_t)off * 2;
+  }
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+      blk.kf[h][c].u = *(const uint4*)(kbase[h] + (k_lane + (uint32_t)c * 64u));
+#pragma unroll
+  for (int dt = 0; dt < D / 16; ++dt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      blk.vf[dt].u2[h] = *(const uint2*)(vbase[h] + (v_lane + (uint32_t)(dt * 32 * ps)));
+}
+
+// The running state of RT tiles of 16 rows: this lane's row of each tile.
+template <int D, int RT>
+struct TileState {
+  Frag qf[RT][D / 32];
+  f32x4 acc[RT][D / 16];
+  float m[RT], lsum[RT];
+  int pos[RT], lo[RT];
+  bool row_ok[RT];
+};
+
+// One block of 32 keys against the tiles: scores, online softmax, weighted values.  Scores
+// are kept in the base-2 domain (`c` = scale * log2 e), so every exponential is one
+// instruction.  MASKED is for blocks that some row of the tiles cannot see in full (the
+// causal edge, the window's edge, the end of the sequence); inside, nothing is tested.
+template <int D, int RT, bool MASKED>
+__device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBlock<D>& blk,
+                                             int key0, float c, int g4) {
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    float s[8];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+      for (int k = 0; k < D / 32; ++k)
+        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[h][k].v, st.qf[t][k].v, sc, 0, 0, 0);
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        float v = sc[i] * c;
+        if (MASKED) {
+          const int key = key0 + h * 16 + g4 * 4 + i;
+          const bool ok = blk.live[h] && st.row_ok[t] && key <= st.pos[t] && key >= st.lo[t];
+          v = ok ? v : -INFINITY;
+        }
+        s[h * 4 + i] = v;
+      }
+    }
+    float bm = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                     fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    // The four lanes of a row exchange their maxima, and what is accumulated is rescaled,
+    // only when some lane saw a score above its row's running maximum: rare once a row has
+    // seen a few blocks.
+    if (__builtin_amdgcn_ballot_w64(bm > st.m[t]) != 0) {
+      bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
+      bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+      const float m_new = fmaxf(st.m[t], bm);
+      const float corr = __builtin_amdgcn_exp2f(st.m[t] - (m_new == -INFINITY ? 0.f : m_new));
+      st.lsum[t] *= corr;
+#pragma unroll
+      for (int dt = 0; dt < D / 16; ++dt) st.acc[t][dt] *= corr;
+      st.m[t] = m_new;
+    }
+    const float m_use = (MASKED && st.m[t] == -INFINITY) ? 0.f : st.m[t];
+    float e[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s[j] - m_use);
+    st.lsum[t] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
+    Frag pf;
+    pf.u = make_uint4(pack_bf16x2(e[0], e[1]), pack_bf16x2(e[2], e[3]), pack_bf16x2(e[4], e[5]),
+                      pack_bf16x2(e[6], e[7]));
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt)
+      st.acc[t][dt] =
+          __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.vf[dt].v, pf.v, st.acc[t][dt], 0, 0, 0);
+  }
+}
+
+// Blocks wholly inside what every row of the tiles sees take the unmasked path.
+template <int D, int RT>
+__device__ __forceinline__ void attend(TileState<D, RT>& st, const KeyBlock<D>& blk, int key0,
+                                       float c, int g4, int all_see_upto, int all_see_from) {
+  if (key0 + 31 <= all_see_upto && key0 >= all_see_from)
+    attend_block<D, RT, false>(st, blk, key0, c, g4);
+  else
+    attend_block<D, RT, true>(st, blk, key0, c, g4);
+}
+
+// RT: 16-row tiles per wavefront.  A decoded token's heads fill one tile (RT = 1, and the
+// keys may be split); a prompt portion may give each wavefront RT consecutive tiles, which
+// share every key and value fragment the wavefront loads.  AHEAD: how many blocks of keys
+// are in flight beyond the one in the matrix cores (0, 1 or 2).
+template <int D, int RT, int AHEAD>
 __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p) {
   const int lane = threadIdx.x & 63;
-  const int tile = blockIdx.x * ATTN_WAVES + (threadIdx.x >> 6);
-  if (tile >= p.num_tiles) return;
+  // Tiles are taken from the last: under a causal mask the later tiles of a prompt read the
+  // most keys, and the longest work should start first.
+  const int tile = p.num_tiles - 1 - (blockIdx.x * ATTN_WAVES + (threadIdx.x >> 6));
+  if (tile < 0) return;
   const int kvh = blockIdx.y, split = blockIdx.z;
   const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
@@ -72,132 +220,109 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p
   const int rows_total = q_len * G;
   const int r = lane & 15, g4 = lane >> 4;
 
-  // The row this lane stands for as a column of S^T and O^T.
-  const int flat = row0 + r;
-  const bool row_ok = flat < rows_total;
-  const int tok = row_ok ? flat / G : 0;
-  const int head = kvh * G + (row_ok ? flat % G : 0);
-  const int pos = pos0 + tok;
-  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+  // The rows this lane stands for as a column of S^T and O^T, one per tile.
+  TileState<D, RT> st;
+  int tok[RT], head[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const int flat = row0 + t * 16 + r;
+    st.row_ok[t] = flat < rows_total;
+    tok[t] = st.row_ok[t] ? flat / G : 0;
+    head[t] = kvh * G + (st.row_ok[t] ? flat % G : 0);
+    st.pos[t] = pos0 + tok[t];
+    st.lo[t] = p.window > 0 ? max(0, st.pos[t] - p.window + 1) : 0;
+    st.m[t] = -INFINITY;
+    st.lsum[t] = 0.f;
+    const bf16_t* qrow = p.q + (size_t)(q0 + tok[t]) * p.q_stride + head[t] * D + g4 * 8;
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+      st.qf[t][c].u = st.row_ok[t] ? *(const uint4*)(qrow + c * 32) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt) st.acc[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
 
-  // Keys any row of the tile can see, in blocks of 32, and this split's share of them.
-  const int last_flat = min(row0 + 15, rows_total - 1);
+  // Keys any row of the tiles can see, in blocks of 32, and this split's share of them.
+  const int last_flat = min(row0 + 16 * RT - 1, rows_total - 1);
   const int kmax = pos0 + last_flat / G;
   const int kmin = p.window > 0 ? max(0, pos0 + row0 / G - p.window + 1) : 0;
   const int blk_lo = kmin >> 5, blk_hi = (kmax >> 5) + 1;
-  const int per = (blk_hi - blk_lo + p.num_splits - 1) / p.num_splits;
+  const int per = p.split_blocks > 0 ? p.split_blocks
+                                     : (blk_hi - blk_lo + p.num_splits - 1) / p.num_splits;
   const int b0 = blk_lo + split * per, b1 = min(blk_hi, b0 + per);
+  // Keys [see_from, see_upto] are visible to every valid row of the tiles.
+  const int see_upto = pos0 + row0 / G;
+  const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
+  const float c = p.scale * 1.44269504088896340736f;
 
-  Frag qf[D / 32];
-  {
-    const bf16_t* qrow = p.q + (size_t)(q0 + tok) * p.q_stride + head * D + g4 * 8;
-#pragma unroll
-    for (int c = 0; c < D / 32; ++c)
-      qf[c].u = row_ok ? *(const uint4*)(qrow + c * 32) : make_uint4(0, 0, 0, 0);
-  }
-
-  f32x4 acc[D / 16];
-#pragma unroll
-  for (int dt = 0; dt < D / 16; ++dt) acc[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  float m = -INFINITY, lsum = 0.f;
-  const int ps = 1 << p.page_shift;
-  const int* table = p.block_table + (size_t)seq * p.table_stride;
-
-  for (int b = b0; b < b1; ++b) {
-    const int key0 = b << 5;
-    // Addresses first, then every load of the block (keys and values) before any use, so
-    // that one trip to memory covers them all.
-    bool live[2];
-    const bf16_t* krow[2];
-    const bf16_t* vrow[2];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const int kh = key0 + h * 16;
-      live[h] = kh <= kmax && kh + 15 >= kmin;  // the same for the whole wavefront
-      const int page = live[h] ? table[kh >> p.page_shift] : 0;
-      const int off = kh & (ps - 1);
-      const size_t head_base = (size_t)page * p.n_kv + kvh;
-      krow[h] = p.k_cache + (head_base * ps + off + r) * D + g4 * 8;
-      vrow[h] = p.v_cache + head_base * ps * D + off + (size_t)r * ps + g4 * 4;
+  TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
+  if (AHEAD == 0) {
+    KeyBlock<D> blk;
+    for (int b = b0; b < b1; ++b) {
+      load_key_block<D>(blk, p, tw, b, b1, kmin, kmax, kvh, lane);
+      attend<D, RT>(st, blk, b << 5, c, g4, see_upto, see_from);
     }
-    Frag kf[2][D / 32], vf[D / 16];
-#pragma unroll
-    for (int h = 0; h < 2; ++h)
-#pragma unroll
-      for (int c = 0; c < D / 32; ++c)
-        kf[h][c].u = live[h] ? *(const uint4*)(krow[h] + c * 32) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt)
-#pragma unroll
-      for (int h = 0; h < 2; ++h)
-        vf[dt].u2[h] = live[h] ? *(const uint2*)(vrow[h] + (size_t)dt * 16 * ps) : make_uint2(0, 0);
-
-    float s[8];
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      f32x4 sc = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll
-      for (int c = 0; c < D / 32; ++c)
-        sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kf[h][c].v, qf[c].v, sc, 0, 0, 0);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        const int key = key0 + h * 16 + g4 * 4 + i;
-        const bool ok = live[h] && row_ok && key <= pos && key >= lo;
-        s[h * 4 + i] = ok ? sc[i] * p.scale : -INFINITY;
+  } else if (AHEAD == 1) {
+    KeyBlock<D> x, y;
+    load_key_block<D>(x, p, tw, b0, b1, kmin, kmax, kvh, lane);
+    for (int b = b0; b < b1; b += 2) {
+      load_key_block<D>(y, p, tw, b + 1, b1, kmin, kmax, kvh, lane);
+      attend<D, RT>(st, x, b << 5, c, g4, see_upto, see_from);
+      if (b + 1 < b1) {
+        load_key_block<D>(x, p, tw, b + 2, b1, kmin, kmax, kvh, lane);
+        attend<D, RT>(st, y, (b + 1) << 5, c, g4, see_upto, see_from);
       }
     }
-
-    float bm = s[0];
-#pragma unroll
-    for (int j = 1; j < 8; ++j) bm = fmaxf(bm, s[j]);
-    bm = fmaxf(bm, __shfl_xor(bm, 16, 64));
-    bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
-    const float m_new = fmaxf(m, bm);
-    const float m_use = m_new == -INFINITY ? 0.f : m_new;
-    const float corr = __expf(m - m_use);
-    Frag pf;
-    float psum = 0.f;
-#pragma unroll
-    for (int j = 0; j < 8; ++j) {
-      const bf16_t e = f32_to_bf16(__expf(s[j] - m_use));
-      pf.h[j] = e;
-      psum += bf16_to_f32(e);
-    }
-    lsum = lsum * corr + psum;
-    m = m_new;
-#pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt) {
-      acc[dt] *= corr;
-      acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(vf[dt].v, pf.v, acc[dt], 0, 0, 0);
+  } else {
+    KeyBlock<D> x, y, z;
+    load_key_block<D>(x, p, tw, b0, b1, kmin, kmax, kvh, lane);
+    load_key_block<D>(y, p, tw, b0 + 1, b1, kmin, kmax, kvh, lane);
+    for (int b = b0; b < b1; b += 3) {
+      load_key_block<D>(z, p, tw, b + 2, b1, kmin, kmax, kvh, lane);
+      attend<D, RT>(st, x, b << 5, c, g4, see_upto, see_from);
+      if (b + 1 < b1) {
+        load_key_block<D>(x, p, tw, b + 3, b1, kmin, kmax, kvh, lane);
+        attend<D, RT>(st, y, (b + 1) << 5, c, g4, see_upto, see_from);
+      }
+      if (b + 2 < b1) {
+        load_key_block<D>(y, p, tw, b + 4, b1, kmin, kmax, kvh, lane);
+        attend<D, RT>(st, z, (b + 2) << 5, c, g4, see_upto, see_from);
+      }
     }
   }
 
-  lsum += __shfl_xor(lsum, 16, 64);
-  lsum += __shfl_xor(lsum, 32, 64);
-
-  // acc[dt][i] is O^T[dim = dt*16 + g4*4 + i][row r].
-  if (p.num_splits == 1) {
-    if (!row_ok) return;
-    const float inv = 1.f / lsum;
-    bf16_t* dst = p.out + (size_t)(q0 + tok) * p.out_stride + head * D + g4 * 4;
 #pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt) {
-      ushort4 o;
-      o.x = f32_to_bf16(acc[dt][0] * inv);
-      o.y = f32_to_bf16(acc[dt][1] * inv);
-      o.z = f32_to_bf16(acc[dt][2] * inv);
-      o.w = f32_to_bf16(acc[dt][3] * inv);
-      *(ushort4*)(dst + dt * 16) = o;
-    }
-  } else {
-    const size_t slot = (((size_t)tile * p.n_kv + kvh) * p.num_splits + split) * 16 + r;
-    float* po = p.part_o + slot * D + g4 * 4;
+  for (int t = 0; t < RT; ++t) {
+    float l = st.lsum[t];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    // acc[t][dt][i] is O^T[dim = dt*16 + g4*4 + i][row r of tile t].
+    if (p.num_splits == 1) {
+      if (!st.row_ok[t]) continue;
+      const float inv = 1.f / l;
+      bf16_t* dst = p.out + (size_t)(q0 + tok[t]) * p.out_stride + head[t] * D + g4 * 4;
 #pragma unroll
-    for (int dt = 0; dt < D / 16; ++dt)
-      *(float4*)(po + dt * 16) = make_float4(acc[dt][0], acc[dt][1], acc[dt][2], acc[dt][3]);
-    if (g4 == 0) {
-      p.part_ml[slot * 2] = m;
-      p.part_ml[slot * 2 + 1] = lsum;
+      for (int dt = 0; dt < D / 16; ++dt) {
+        ushort4 o;
+        o.x = f32_to_bf16(st.acc[t][dt][0] * inv);
+        o.y = f32_to_bf16(st.acc[t][dt][1] * inv);
+        o.z = f32_to_bf16(st.acc[t][dt][2] * inv);
+        o.w = f32_to_bf16(st.acc[t][dt][3] * inv);
+        *(ushort4*)(dst + dt * 16) = o;
+      }
+    } else {
+      const size_t slot =
+          (((size_t)tile * p.n_kv + kvh) * p.num_splits + split) * (16 * RT) + t * 16 + r;
+      if (b0 < b1) {  // an empty split only records that it is empty
+        float* po = p.part_o + slot * D + g4 * 4;
+#pragma unroll
+        for (int dt = 0; dt < D / 16; ++dt)
+          *(float4*)(po + dt * 16) = make_float4(st.acc[t][dt][0], st.acc[t][dt][1],
+                                                 st.acc[t][dt][2], st.acc[t][dt][3]);
+      }
+      if (g4 == 0) {
+        p.part_ml[slot * 2] = st.m[t];
+        p.part_ml[slot * 2 + 1] = l;
+      }
     }
   }
 }
@@ -211,7 +336,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   __shared__ float weight[1024];
   __shared__ float group_sum[4][D];
   __shared__ float scratch[16];
-  const int tile = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z;
+  const int tile = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z, R = p.tile_rows;
   const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
   const int G = p.group;
@@ -222,13 +347,13 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
 
   float mx = -INFINITY;
   for (int s = threadIdx.x; s < S; s += blockDim.x)
-    mx = fmaxf(mx, p.part_ml[((base + s) * 16 + r) * 2]);
+    mx = fmaxf(mx, p.part_ml[((base + s) * R + r) * 2]);
   mx = block_max(mx, scratch);
   float part = 0.f;
   for (int s = threadIdx.x; s < S; s += blockDim.x) {
-    const size_t slot = (base + s) * 16 + r;
+    const size_t slot = (base + s) * R + r;
     const float ms = p.part_ml[slot * 2];
-    const float w = ms == -INFINITY ? 0.f : __expf(ms - mx);
+    const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mx);  // base-2 maxima
     weight[s] = w;
     part += p.part_ml[slot * 2 + 1] * w;
   }
@@ -236,18 +361,17 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
 
   const int g = threadIdx.x >> 6;
   for (int dim = threadIdx.x & 63; dim < D; dim += 64) {
-    const float* src = p.part_o + ((base * 16) + r) * D + dim;
-    const size_t stride = (size_t)16 * D;
+    const float* src = p.part_o + ((base * R) + r) * D + dim;
+    const size_t stride = (size_t)R * D;
+    // An empty split has weight 0 and holds nothing: it is not read.
+    auto term = [&](int s) { return weight[s] > 0.f ? src[(size_t)s * stride] * weight[s] : 0.f; };
     float o = 0.f;
     int s = g;
     for (; s + 12 < S; s += 16) {
-      const float a = src[(size_t)s * stride] * weight[s];
-      const float b = src[(size_t)(s + 4) * stride] * weight[s + 4];
-      const float c = src[(size_t)(s + 8) * stride] * weight[s + 8];
-      const float d = src[(size_t)(s + 12) * stride] * weight[s + 12];
+      const float a = term(s), b = term(s + 4), c = term(s + 8), d = term(s + 12);
       o += (a + b) + (c + d);
     }
-    for (; s < S; s += 4) o += src[(size_t)s * stride] * weight[s];
+    for (; s < S; s += 4) o += term(s);
     group_sum[g][dim] = o;
   }
   __syncthreads();
@@ -259,13 +383,26 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
 }
 
 template <int D>
-static void launch_attn(const AttnParams& p, hipStream_t stream) {
+static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stream) {
   dim3 grid((p.num_tiles + ATTN_WAVES - 1) / ATTN_WAVES, p.n_kv, p.num_splits);
-  attn_mfma_kernel<D><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
+  const int threads = 64 * ATTN_WAVES;
+  if (rows_per_tile == 16) {
+    attn_mfma_kernel<D, 1, ATTN_AHEAD_16><<<grid, threads, 0, stream>>>(p);
+  } else if (rows_per_tile == 32) {
+    if constexpr (D <= 128) attn_mfma_kernel<D, 2, ATTN_AHEAD_32><<<grid, threads, 0, stream>>>(p);
+  } else {
+    // 64 rows: only instantiated where the accumulators fit the register file
+    if constexpr (D <= 64) attn_mfma_kernel<D, 4, ATTN_AHEAD_64><<<grid, threads, 0, stream>>>(p);
+  }
   if (p.num_splits > 1) {
-    dim3 mgrid(p.num_tiles, p.n_kv, 16);
+    dim3 mgrid(p.num_tiles, p.n_kv, p.tile_rows);
     attn_merge_kernel<D><<<mgrid, 256, 0, stream>>>(p);
   }
+}
+
+// The most rows (16, 32 or 64) one wavefront can take for this head size.
+extern "C" int mk_attention_mfma_max_rows(int head_dim) {
+  return head_dim <= 64 ? 64 : (head_dim <= 128 ? 32 : 16);
 }
 
 extern "C" int mk_attention_mfma_supported(int head_dim, int page_size) {
@@ -279,8 +416,8 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
                                  const int* tile_row0, int num_tiles, const int* cu_q,
                                  const int* kv_len, const int* block_table, int table_stride,
                                  int page_size, int n_q, int n_kv, int d, float scale, int window,
-                                 int num_splits, float* part_o, float* part_ml,
-                                 hipStream_t stream) {
+                                 int rows_per_tile, int num_splits, int split_blocks,
+                                 float* part_o, float* part_ml, hipStream_t stream) {
   MK_REQUIRE(num_tiles >= 0 && n_q > 0 && n_kv > 0, "attention: bad sizes");
   MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
              n_q, n_kv);
@@ -293,6 +430,11 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   MK_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0,
              "attention: row strides %d/%d break 16-byte alignment", q_stride, out_stride);
   MK_REQUIRE(window >= 0, "attention: negative window");
+  MK_REQUIRE(rows_per_tile == 16 || rows_per_tile == 32 || rows_per_tile == 64,
+             "attention: %d rows per tile", rows_per_tile);
+  MK_REQUIRE(rows_per_tile <= mk_attention_mfma_max_rows(d),
+             "attention: %d rows per tile are too many for head size %d", rows_per_tile, d);
+  MK_REQUIRE(split_blocks >= 0, "attention: negative split size");
   if (num_tiles == 0) return 0;
   AttnParams p;
   p.q = (const bf16_t*)q;
@@ -316,13 +458,15 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   p.window = window;
   p.num_tiles = num_tiles;
   p.num_splits = num_splits;
+  p.split_blocks = split_blocks;
+  p.tile_rows = rows_per_tile;
   switch (d) {
-    case 32: launch_attn<32>(p, stream); break;
-    case 64: launch_attn<64>(p, stream); break;
-    case 96: launch_attn<96>(p, stream); break;
-    case 128: launch_attn<128>(p, stream); break;
-    case 192: launch_attn<192>(p, stream); break;
-    case 256: launch_attn<256>(p, stream); break;
+    case 32: launch_attn<32>(p, rows_per_tile, stream); break;
+    case 64: launch_attn<64>(p, rows_per_tile, stream); break;
+    case 96: launch_attn<96>(p, rows_per_tile, stream); break;
+    case 128: launch_attn<128>(p, rows_per_tile, stream); break;
+    case 192: launch_attn<192>(p, rows_per_tile, stream); break;
+    case 256: launch_attn<256>(p, rows_per_tile, stream); break;
   }
   MK_LAUNCH_CHECK("attention_mfma");
   return 0;

@@ -40,12 +40,19 @@ __device__ __forceinline__ float bf16_to_f32(bf16_t x) {
   return __uint_as_float(((uint32_t)x) << 16);
 }
 
-// Round to nearest, ties to even; NaN stays NaN.
+// Round to nearest, ties to even; NaN stays NaN (v_cvt_pk_bf16_f32 on gfx950).
 __device__ __forceinline__ bf16_t f32_to_bf16(float f) {
-  uint32_t u = __float_as_uint(f);
-  if ((u & 0x7fffffffu) > 0x7f800000u) return (bf16_t)((u >> 16) | 0x40u);
-  u += 0x7fffu + ((u >> 16) & 1u);
-  return (bf16_t)(u >> 16);
+  const __bf16 b = (__bf16)f;
+  return __builtin_bit_cast(bf16_t, b);
+}
+
+// Two floats rounded to bfloat16 in one 32-bit word, `a` in the low half.
+__device__ __forceinline__ uint32_t pack_bf16x2(float a, float b) {
+  typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+  bf16x2_t v;
+  v[0] = (__bf16)a;
+  v[1] = (__bf16)b;
+  return __builtin_bit_cast(uint32_t, v);
 }
 
 template <typename T>

@@ -84,18 +84,22 @@ int mk_linear_tiled(const void* x, const void* w, const void* bias, int bias_dty
 // Whether mk_attention_mfma takes this head size and page size.
 int mk_attention_mfma_supported(int head_dim, int page_size);
 
-// The same attention on the matrix cores.  The caller cuts the step into tiles of 16 rows
-// (row f of a sequence = token f / G, head kvh * G + f % G): tile_seq / tile_row0 name each
-// tile's sequence and first row.  cu_q [S+1] are the prefix sums of the sequences' token
+// The most rows per tile (16, 32 or 64) mk_attention_mfma takes for this head size.
+int mk_attention_mfma_max_rows(int head_dim);
+
+// The same attention on the matrix cores.  The caller cuts the step into tiles of
+// rows_per_tile rows (row f of a sequence = token f / G, head kvh * G + f % G):
+// tile_seq / tile_row0 name each tile's sequence and first row.  cu_q [S+1] are the prefix sums of the sequences' token
 // counts, kv_len [S] their lengths once this step's tokens are written.  With num_splits > 1
-// the keys are split and part_o [tiles, n_kv, splits, 16, d] / part_ml [.., 16, 2] hold the
-// partial results.
+// the keys are split, split_blocks blocks of 32 keys per split (0: each tile's own range in
+// num_splits equal parts), and part_o [tiles, n_kv, splits, rows_per_tile, d] /
+// part_ml [.., rows_per_tile, 2] hold the partial results.
 int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       const void* k_cache, const void* v_cache, const int* tile_seq,
                       const int* tile_row0, int num_tiles, const int* cu_q, const int* kv_len,
                       const int* block_table, int table_stride, int page_size, int n_q, int n_kv,
-                      int d, float scale, int window, int num_splits, float* part_o,
-                      float* part_ml, hipStream_t stream);
+                      int d, float scale, int window, int rows_per_tile, int num_splits,
+                      int split_blocks, float* part_o, float* part_ml, hipStream_t stream);
 
 // ---- library "core" again
 

@@ -55,26 +55,22 @@ class StepContext:
         self.fresh_slots: list = []
         self._tiles: dict = {}
 
-    def tiles(self, group: int):
-        """(tile_seq, tile_row0, count) for attention tiles of 16 rows, a row being a
+    def tiles(self, group: int, rows: int = 16):
+        """(tile_seq, tile_row0, count) for attention tiles of `rows` rows, a row being a
         (token, head within a group of `group` query heads) pair: sequence s with n tokens
-        this step has ceil(n * group / 16) tiles."""
-        cached = self._tiles.get(group)
+        this step has ceil(n * group / rows) tiles."""
+        cached = self._tiles.get((group, rows))
         if cached is None:
-            seqs, rows = [], []
+            seqs, firsts = [], []
             for s, (_first, count, _start) in enumerate(self.spans):
-                n = -(-count * group // 16)
+                n = -(-count * group // rows)
                 seqs.extend([s] * n)
-                rows.extend(range(0, 16 * n, 16))
+                firsts.extend(range(0, rows * n, rows))
             device = self.token_ids.device
-            both = torch.tensor([seqs, rows], dtype=torch.int32).to(device, non_blocking=True)
+            both = torch.tensor([seqs, firsts], dtype=torch.int32).to(device, non_blocking=True)
             cached = (both[0], both[1], len(seqs))
-            self._tiles[group] = cached
+            self._tiles[(group, rows)] = cached
         return cached
-
-
-class BatchError(ValueError):
-    pass
 
 
 def context_from_spans(spans: list, device, token_ids=None) -> StepContext:

@@ -35,7 +35,8 @@ _SIGNATURES = {
         "mk_gated_skinny": [P, P, P, I, I, I, P],
         "mk_linear_tiled": [P, P, P, I, P, I, I, I, I, I, I, P],
         "mk_attention_mfma_supported": [I, I],
-        "mk_attention_mfma": [P, I, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P, P, P],
+        "mk_attention_mfma_max_rows": [I],
+        "mk_attention_mfma": [P, I, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, P, P, P],
     },
 }
 

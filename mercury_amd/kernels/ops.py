@@ -328,7 +328,8 @@ def _qkv_finish(parts, cos, sin, positions, token_seq, block_table, k_cache, v_c
 def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
               step, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int, scale: float,
               window: int | None = None, out: torch.Tensor | None = None,
-              kernel: str = "auto") -> torch.Tensor:
+              kernel: str = "auto", tile_rows: int | None = None,
+              split_override: tuple | None = None) -> torch.Tensor:
     """Causal grouped-query attention of every token of the step over its sequence's cached
     keys; q is read from rows of `q` with stride `q_stride` (the fused qkv buffer).
     `step` describes the batch (positions, token_seq, cu_q, kv_len, spans, tiles());
@@ -336,6 +337,9 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
 
     kernel: "auto" takes the matrix-core kernel for bfloat16 where it covers the head and page
     size and the float32-arithmetic kernel otherwise; "generic" and "mfma" force one.
+    tile_rows (16, 32 or 64) overrides how many rows a wavefront of the matrix-core kernel
+    takes, split_override = (splits, key blocks per split) how the keys are split; by
+    default the step's size decides both.
     """
     _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out)
     _i32(block_table, "block_table")
@@ -362,26 +366,48 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
         raise KernelArgumentError("attention: the matrix-core kernel takes bfloat16 only")
     lib = _lib.load("mfma")
     group = n_q // n_kv
-    tile_seq, tile_row0, num_tiles = step.tiles(group)
-    # Split the keys when the tiles alone would leave most of the chip idle: aim at about a
-    # thousand wavefronts, each with at least one block of 32 keys.
+    # Tiles of 16 rows, the keys split when the tiles alone would leave most of the chip idle
+    # (decoding); wider tiles, whose rows share every key fragment a wavefront loads, when
+    # there are plenty (prompts).
     span = step.max_kv_len if not window else min(step.max_kv_len, window + step.max_q_len)
     blocks = max(1, -(-span // 32))
+    rows = 16
+    total_rows = sum(count for _first, count, _start in step.spans) * group
+    max_rows = lib.mk_attention_mfma_max_rows(head_dim)
+    while rows < max_rows and (total_rows // (rows * 2)) * n_kv >= ATTENTION_WIDE_TILE_WAVES:
+        rows *= 2
+    if tile_rows is not None:
+        rows = tile_rows
+    tile_seq, tile_row0, num_tiles = step.tiles(group, rows)
+    splits, split_blocks = 1, 0
     waves = max(1, num_tiles * n_kv)
-    splits = max(1, min(blocks // ATTENTION_MIN_BLOCKS_PER_SPLIT or 1, -(-ATTENTION_TARGET_WAVES // waves)))
+    if waves < ATTENTION_TARGET_WAVES and step.max_q_len == 1:
+        # decoding: every sequence's own range in equal parts
+        splits = max(1, min(blocks // ATTENTION_MIN_BLOCKS_PER_SPLIT or 1,
+                            -(-ATTENTION_TARGET_WAVES // waves), 1024))
+    elif blocks > ATTENTION_PROMPT_SPLIT_BLOCKS:
+        # prompts: no wavefront walks more than a fixed stretch of keys, so the tiles at the
+        # end of a long causal prompt do not outlast all the others
+        split_blocks = ATTENTION_PROMPT_SPLIT_BLOCKS
+        splits = -(-blocks // split_blocks)
+    if split_override is not None:
+        splits, split_blocks = split_override
     part_o = part_ml = None
     if splits > 1:
-        part_o = torch.empty((num_tiles, n_kv, splits, 16, head_dim), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((num_tiles, n_kv, splits, 16, 2), dtype=torch.float32, device=q.device)
+        part_o = torch.empty((num_tiles, n_kv, splits, rows, head_dim), dtype=torch.float32, device=q.device)
+        part_ml = torch.empty((num_tiles, n_kv, splits, rows, 2), dtype=torch.float32, device=q.device)
     _lib.check(lib, lib.mk_attention_mfma(
         _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
         _ptr(tile_seq), _ptr(tile_row0), num_tiles, _ptr(step.cu_q), _ptr(step.kv_len),
         _ptr(block_table), block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
-        int(window or 0), splits, _ptr(part_o), _ptr(part_ml), _stream()), "attention")
+        int(window or 0), rows, splits, split_blocks, _ptr(part_o), _ptr(part_ml), _stream()),
+        "attention")
     return out
 
 
 ATTENTION_TARGET_WAVES = 1024
+ATTENTION_WIDE_TILE_WAVES = 400
+ATTENTION_PROMPT_SPLIT_BLOCKS = 1 << 30   # prompts are not split: the merge costs what the split gains
 ATTENTION_MIN_BLOCKS_PER_SPLIT = 2
 
 

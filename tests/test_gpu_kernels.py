@@ -350,7 +350,8 @@ def test_rotary_scores_depend_on_distance_only():
 
 
 def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens, q_lens, scale,
-                  window=None, poison=None, kernel="auto", hide_before=None):
+                  window=None, poison=None, kernel="auto", hide_before=None, tile_rows=None,
+                  split_override=None):
     """q_h: list per sequence of [q_len, n_q, d] (the last q_len positions of the sequence);
     k_h/v_h: list per sequence of [seq_len, n_kv, d].  `hide_before`: per sequence, the number
     of leading pages to drop from the table (-1) and to poison, as after a window passed."""
@@ -378,7 +379,8 @@ def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens
     q_flat = torch.cat([q.reshape(q.shape[0], n_q * d) for q in q_h]).to(dtype).to(DEV)
     v_cache = v_cache.transpose(2, 3).contiguous()      # values lie transposed within a page
     out = ops().attention(q_flat, n_q * d, k_cache.to(DEV), v_cache.to(DEV), step, table.to(DEV),
-                          n_q, n_kv, d, scale, window, kernel=kernel)
+                          n_q, n_kv, d, scale, window, kernel=kernel, tile_rows=tile_rows,
+                          split_override=split_override)
     return out.float().cpu().view(-1, n_q, d)
 
 
@@ -494,6 +496,31 @@ def test_attention_window_edge(d, page, dtype, kernel, window):
                         window=window, kernel=kernel, hide_before=[gone])
     want = plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-q_len:]
     torch.testing.assert_close(got, want, **tol(dtype))
+
+
+@pytest.mark.parametrize("tile_rows,d,n_q,n_kv", [(32, 64, 14, 2), (64, 64, 14, 2), (32, 128, 8, 2),
+                                                  (64, 32, 6, 6), (32, 96, 3, 1), (16, 64, 14, 2)])
+@pytest.mark.parametrize("window", [None, 40])
+@pytest.mark.parametrize("split", [None, (3, 2), (5, 1), (4, 0)])
+def test_attention_wide_tiles_for_prompts(tile_rows, d, n_q, n_kv, window, split):
+    """Wavefronts that take 32 or 64 rows (several tiles sharing the key fragments): two prompt
+    portions of different length, one over a cached prefix, beside a decoded token; with the
+    keys unsplit, split into fixed stretches of blocks (some splits then empty), and split
+    evenly."""
+    page = 16
+    lens, q_lens = [150, 77, 90], [150, 33, 1]
+    qs, ks, vs = [], [], []
+    for i, s in enumerate(lens):
+        ks.append(rounded(rnd(s, n_kv, d, seed=500 + i), torch.bfloat16))
+        vs.append(rounded(rnd(s, n_kv, d, seed=510 + i), torch.bfloat16))
+        qs.append(rounded(rnd(s, n_q, d, seed=520 + i), torch.bfloat16))
+    pages = [list(range(0, 10)), list(range(20, 25)), list(range(30, 36))]
+    got = run_attention([q[-ql:] for q, ql in zip(qs, q_lens)], ks, vs, torch.bfloat16, pages, page,
+                        40, lens, q_lens, d ** -0.5, window=window, poison=1e4, kernel="mfma",
+                        tile_rows=tile_rows, split_override=split)
+    want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-ql:]
+                      for q, k, v, ql in zip(qs, ks, vs, q_lens)])
+    torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
 @pytest.mark.parametrize("batch,context", [(1, 4096), (3, 1500), (64, 300)])
