@@ -12,10 +12,11 @@
 //    are reproducible.  The gate/up projection keeps all of K in one workgroup and gates in
 //    its epilogue.
 //
-//  * tiled (M > 64, prompts): 128 x 128 tiles of y per workgroup, K in steps of 32 through
-//    LDS with the next step's global loads in flight during the current step's products;
-//    4 wavefronts as 2 x 2, each 64 x 64 = 4 x 4 MFMA tiles.  Epilogues: bfloat16 store with
-//    bias, float32 store, or float32 accumulate into the residual stream.
+//  * tiled (M > 64, prompts): tiles of y per workgroup of four wavefronts (128 x 128, or
+//    smaller when the matrix would otherwise leave compute units idle), K in stages through
+//    two LDS buffers with the next stage's global loads in flight during the current stage's
+//    products.  Epilogues: bfloat16 store with bias, float32 store, or float32 accumulate
+//    into the residual stream.
 //
 // In both, lane l of a wavefront holds row (l % 16) and k-slots (l / 16) * 8 .. + 8 of an
 // operand; which k a slot means is free as long as A and B agree, and the skinny kernel uses
@@ -212,56 +213,75 @@ extern "C" int mk_gated_skinny(const void* x, const void* w, void* act, int M, i
 
 // ------------------------------------------------------------------------------- tiled
 
-#define TB 128  // tile of y, both ways
-#define TK 32   // k per LDS stage
-#define TLD 40  // LDS row stride in elements (80 bytes: conflict-free 16-byte reads)
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3 };
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2 };
-
-template <int EPI, typename TBIAS>
+// One workgroup of 4 wavefronts (WM x WN) computes a BM x BN tile of y; K advances TK per
+// stage through two LDS buffers, the next stage's global loads in flight during the current
+// stage's products.  Rows of a tile lie in LDS with a stride of TK + 8 elements, which keeps
+// 16-byte reads of 16 consecutive rows on distinct banks.
+// EPI_GATED: W is [gate rows | up rows] of N each; a tile holds BN / 2 gate rows and the BN / 2
+// matching up rows, every wavefront spans the tile's whole width (WN = 1), and the epilogue
+// writes act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
+template <int BM, int BN, int TK, int WM, int WN, int EPI, typename TBIAS>
 __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
                                                          const bf16_t* __restrict__ w,
                                                          const TBIAS* __restrict__ bias,
                                                          void* __restrict__ out_, int M, int N,
                                                          int K, int ldo) {
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][TB * TLD];
-  __shared__ __attribute__((aligned(16))) bf16_t ws[2][TB * TLD];
+  static_assert(WM * WN == 4, "four wavefronts");
+  static_assert(EPI != EPI_GATED || WN == 1, "gating needs both halves in one wavefront");
+  constexpr int LD = TK + 8;
+  constexpr int TM = BM / WM / 16, TN = BN / WN / 16;       // MFMA tiles per wavefront
+  constexpr int CHUNKS_ROW = TK / 8;                        // 16-byte chunks per tile row
+  constexpr int XCH = BM * CHUNKS_ROW / 256, WCH = BN * CHUNKS_ROW / 256;  // per thread
+  static_assert(XCH >= 1 && WCH >= 1, "tile too small for 256 threads");
+  __shared__ __attribute__((aligned(16))) bf16_t xs[2][BM * LD];
+  __shared__ __attribute__((aligned(16))) bf16_t ws[2][BN * LD];
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g4 = lane >> 4;
-  const int wm = (wave >> 1) * 64, wn = (wave & 1) * 64;
-  const int m0 = blockIdx.y * TB, n0 = blockIdx.x * TB;
+  const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
+  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * (EPI == EPI_GATED ? BN / 2 : BN);
 
-  // Staging: 128 rows x 32 k = 512 chunks of 16 bytes per operand, two per thread.
-  const int srow = tid >> 2, sk = (tid & 3) * 8;
-  const bf16_t* xg[2];
-  const bf16_t* wg[2];
+  // Staging: thread t moves chunk t, t + 256, ... of each operand's tile.
+  const bf16_t* xg[XCH];
+  const bf16_t* wg[WCH];
+  int xo[XCH], wo[WCH];
+  const int sk = (tid % CHUNKS_ROW) * 8;
 #pragma unroll
-  for (int i = 0; i < 2; ++i) {
-    xg[i] = x + (size_t)min(m0 + srow + i * 64, M - 1) * K + sk;
-    wg[i] = w + (size_t)min(n0 + srow + i * 64, N - 1) * K + sk;
+  for (int i = 0; i < XCH; ++i) {
+    const int row = (tid + i * 256) / CHUNKS_ROW;
+    xg[i] = x + (size_t)min(m0 + row, M - 1) * K + sk;
+    xo[i] = row * LD + sk;
+  }
+#pragma unroll
+  for (int i = 0; i < WCH; ++i) {
+    const int row = (tid + i * 256) / CHUNKS_ROW;
+    int wrow = min(n0 + row, N - 1);
+    if (EPI == EPI_GATED)  // tile rows [0, BN/2) are gate rows, [BN/2, BN) the matching up rows
+      wrow = row < BN / 2 ? min(n0 + row, N - 1) : N + min(n0 + row - BN / 2, N - 1);
+    wg[i] = w + (size_t)wrow * K + sk;
+    wo[i] = row * LD + sk;
   }
 
-  f32x4 acc[4][4];
+  f32x4 acc[TM][TN];
 #pragma unroll
-  for (int a = 0; a < 4; ++a)
+  for (int a = 0; a < TM; ++a)
 #pragma unroll
-    for (int b = 0; b < 4; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    for (int b = 0; b < TN; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  uint4 xr[2], wr[2];
+  uint4 xr[XCH], wr[WCH];
   auto fetch = [&](int k0) {
     const bool ok = k0 + sk < K;
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      xr[i] = ok ? ld16(xg[i] + k0) : make_uint4(0, 0, 0, 0);
-      wr[i] = ok ? ld16(wg[i] + k0) : make_uint4(0, 0, 0, 0);
-    }
+    for (int i = 0; i < XCH; ++i) xr[i] = ok ? ld16(xg[i] + k0) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int i = 0; i < WCH; ++i) wr[i] = ok ? ld16(wg[i] + k0) : make_uint4(0, 0, 0, 0);
   };
   auto stash = [&](int buf) {
 #pragma unroll
-    for (int i = 0; i < 2; ++i) {
-      *(uint4*)(&xs[buf][(srow + i * 64) * TLD + sk]) = xr[i];
-      *(uint4*)(&ws[buf][(srow + i * 64) * TLD + sk]) = wr[i];
-    }
+    for (int i = 0; i < XCH; ++i) *(uint4*)(&xs[buf][xo[i]]) = xr[i];
+#pragma unroll
+    for (int i = 0; i < WCH; ++i) *(uint4*)(&ws[buf][wo[i]]) = wr[i];
   };
 
   const int steps = (K + TK - 1) / TK;
@@ -271,30 +291,56 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   for (int s = 0; s < steps; ++s) {
     const int buf = s & 1;
     if (s + 1 < steps) fetch((s + 1) * TK);
-    Frag a[4], b[4];
 #pragma unroll
-    for (int t = 0; t < 4; ++t) {
-      a[t].u = *(const uint4*)(&xs[buf][(wm + t * 16 + r) * TLD + g4 * 8]);
-      b[t].u = *(const uint4*)(&ws[buf][(wn + t * 16 + r) * TLD + g4 * 8]);
+    for (int kk = 0; kk < TK; kk += 32) {
+      Frag a[TM], b[TN];
+#pragma unroll
+      for (int t = 0; t < TM; ++t)
+        a[t].u = *(const uint4*)(&xs[buf][(wm + t * 16 + r) * LD + kk + g4 * 8]);
+#pragma unroll
+      for (int t = 0; t < TN; ++t)
+        b[t].u = *(const uint4*)(&ws[buf][(wn + t * 16 + r) * LD + kk + g4 * 8]);
+#pragma unroll
+      for (int ta = 0; ta < TM; ++ta)
+#pragma unroll
+        for (int tb = 0; tb < TN; ++tb)
+          // A = W rows (n), B = x rows (m): the result holds 4 consecutive n per lane.
+          acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[tb].v, a[ta].v, acc[ta][tb],
+                                                                0, 0, 0);
     }
-#pragma unroll
-    for (int ta = 0; ta < 4; ++ta)
-#pragma unroll
-      for (int tb = 0; tb < 4; ++tb)
-        // A = W rows (n), B = x rows (m): the result holds 4 consecutive n per lane.
-        acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[tb].v, a[ta].v, acc[ta][tb], 0,
-                                                              0, 0);
     if (s + 1 < steps) stash(buf ^ 1);
     __syncthreads();
   }
 
   // acc[ta][tb][i] = y[m = m0 + wm + ta*16 + r][n = n0 + wn + tb*16 + g4*4 + i]
 #pragma unroll
-  for (int ta = 0; ta < 4; ++ta) {
+  for (int ta = 0; ta < TM; ++ta) {
     const int m = m0 + wm + ta * 16 + r;
     if (m >= M) continue;
+    if (EPI == EPI_GATED) {
 #pragma unroll
-    for (int tb = 0; tb < 4; ++tb) {
+      for (int tb = 0; tb < TN / 2; ++tb) {
+        const int n = n0 + tb * 16 + g4 * 4;
+        bf16_t* dst = (bf16_t*)out_ + (size_t)m * ldo + n;
+        float o[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float g = Elem<bf16_t>::round(acc[ta][tb][i]);
+          const float u = Elem<bf16_t>::round(acc[ta][tb + TN / 2][i]);
+          o[i] = Elem<bf16_t>::round(g / (1.f + expf(-g))) * u;
+        }
+        if (n + 3 < N && (ldo & 3) == 0) {
+          *(uint2*)dst = make_uint2(pack_bf16x2(o[0], o[1]), pack_bf16x2(o[2], o[3]));
+        } else {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (n + i < N) dst[i] = f32_to_bf16(o[i]);
+        }
+      }
+      continue;
+    }
+#pragma unroll
+    for (int tb = 0; tb < TN; ++tb) {
       const int n = n0 + wn + tb * 16 + g4 * 4;
       float v[4];
 #pragma unroll
@@ -306,12 +352,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       if (EPI == EPI_BF16) {
         bf16_t* dst = (bf16_t*)out_ + (size_t)m * ldo + n;
         if (whole) {
-          ushort4 o;
-          o.x = f32_to_bf16(v[0]);
-          o.y = f32_to_bf16(v[1]);
-          o.z = f32_to_bf16(v[2]);
-          o.w = f32_to_bf16(v[3]);
-          *(ushort4*)dst = o;
+          *(uint2*)dst = make_uint2(pack_bf16x2(v[0], v[1]), pack_bf16x2(v[2], v[3]));
         } else {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
@@ -339,33 +380,69 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   }
 }
 
-template <int EPI>
-static void launch_tiled(const void* x, const void* w, const void* bias, int bias_dtype, void* out,
-                         int M, int N, int K, int ldo, hipStream_t stream) {
-  dim3 grid((N + TB - 1) / TB, (M + TB - 1) / TB);
+template <int BM, int BN, int TK, int WM, int WN, int EPI>
+static void launch_tiled_cfg(const void* x, const void* w, const void* bias, int bias_dtype,
+                             void* out, int M, int N, int K, int ldo, hipStream_t stream) {
+  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
   if (bias && bias_dtype == MK_BF16)
-    gemm_tiled_kernel<EPI, bf16_t><<<grid, 256, 0, stream>>>(
+    gemm_tiled_kernel<BM, BN, TK, WM, WN, EPI, bf16_t><<<grid, 256, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, out, M, N, K, ldo);
   else
-    gemm_tiled_kernel<EPI, float><<<grid, 256, 0, stream>>>(
+    gemm_tiled_kernel<BM, BN, TK, WM, WN, EPI, float><<<grid, 256, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo);
+}
+
+// Tile configurations, by index: 0 = 128x128 (k 64), 1 = 64x128, 2 = 64x64, 3 = 128x128 (k 32).
+#define TILED_CONFIGS 4
+
+template <int EPI>
+static void launch_tiled(int config, const void* x, const void* w, const void* bias,
+                         int bias_dtype, void* out, int M, int N, int K, int ldo,
+                         hipStream_t stream) {
+  switch (config) {
+    case 0: launch_tiled_cfg<128, 128, 64, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 1: launch_tiled_cfg<64, 128, 64, 1, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 2: launch_tiled_cfg<64, 64, 64, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    default: launch_tiled_cfg<128, 128, 32, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+  }
+}
+
+// 128 x 128 tiles when they give every compute unit two workgroups or more, else 64 x 64.
+extern "C" int mk_linear_tiled_config(int M, int N, int K) {
+  const long groups = (long)((M + 127) / 128) * ((N + 127) / 128);
+  return groups >= 512 ? 0 : 2;
+}
+
+// act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K].
+extern "C" int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K,
+                              hipStream_t stream) {
+  MK_REQUIRE(M > 0 && inter > 0 && K > 0 && K % 8 == 0,
+             "gated projection: K=%d must be a multiple of 8 (M=%d I=%d)", K, M, inter);
+  MK_REQUIRE((M + 127) / 128 <= 65535, "gated projection: M=%d too large for one launch", M);
+  dim3 grid((inter + 63) / 64, (M + 127) / 128);
+  gemm_tiled_kernel<128, 128, 64, 4, 1, EPI_GATED, float><<<grid, 256, 0, stream>>>(
+      (const bf16_t*)x, (const bf16_t*)w, (const float*)nullptr, act, M, inter, K, inter);
+  MK_LAUNCH_CHECK("gated_tiled");
+  return 0;
 }
 
 extern "C" int mk_linear_tiled(const void* x, const void* w, const void* bias, int bias_dtype,
                                void* out, int out_dtype, int accumulate, int M, int N, int K,
-                               int ldo, hipStream_t stream) {
+                               int ldo, int config, hipStream_t stream) {
   MK_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0,
              "tiled projection: K=%d must be a multiple of 8 (M=%d N=%d)", K, M, N);
   MK_REQUIRE(ldo >= N, "tiled projection: leading dimension %d smaller than N=%d", ldo, N);
   MK_REQUIRE(!accumulate || out_dtype == MK_F32,
              "tiled projection: accumulation needs a float32 destination");
-  MK_REQUIRE((M + TB - 1) / TB <= 65535, "tiled projection: M=%d too large for one launch", M);
+  MK_REQUIRE((M + 63) / 64 <= 65535, "tiled projection: M=%d too large for one launch", M);
+  if (config < 0) config = mk_linear_tiled_config(M, N, K);
+  MK_REQUIRE(config < TILED_CONFIGS, "tiled projection: no configuration %d", config);
   if (accumulate)
-    launch_tiled<EPI_ACC>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
+    launch_tiled<EPI_ACC>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
   else if (out_dtype == MK_F32)
-    launch_tiled<EPI_F32>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
+    launch_tiled<EPI_F32>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
   else if (out_dtype == MK_BF16)
-    launch_tiled<EPI_BF16>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
+    launch_tiled<EPI_BF16>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
   else
     MK_REQUIRE(false, "tiled projection: unknown out dtype %d", out_dtype);
   MK_LAUNCH_CHECK("linear_tiled");

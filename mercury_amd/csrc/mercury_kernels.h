@@ -75,10 +75,16 @@ int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int
 int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
                     hipStream_t stream);
 
+// The same for any M, tiled through LDS.
+int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K,
+                   hipStream_t stream);
+
 // y = x W^T (+ bias) for any M, tiled through LDS; output bfloat16 or float32, or float32
-// accumulated into `out`.
+// accumulated into `out`.  config: a tile configuration (mk_linear_tiled_config picks one for
+// the shape; -1 does the same).
+int mk_linear_tiled_config(int M, int N, int K);
 int mk_linear_tiled(const void* x, const void* w, const void* bias, int bias_dtype, void* out,
-                    int out_dtype, int accumulate, int M, int N, int K, int ldo,
+                    int out_dtype, int accumulate, int M, int N, int K, int ldo, int config,
                     hipStream_t stream);
 
 // Whether mk_attention_mfma takes this head size and page size.

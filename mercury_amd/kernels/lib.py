@@ -33,7 +33,9 @@ _SIGNATURES = {
         "mk_linear_skinny_slices": [I, I, I],
         "mk_linear_skinny": [P, P, P, I, I, I, I, P],
         "mk_gated_skinny": [P, P, P, I, I, I, P],
-        "mk_linear_tiled": [P, P, P, I, P, I, I, I, I, I, I, P],
+        "mk_gated_tiled": [P, P, P, I, I, I, P],
+        "mk_linear_tiled_config": [I, I, I],
+        "mk_linear_tiled": [P, P, P, I, P, I, I, I, I, I, I, I, P],
         "mk_attention_mfma_supported": [I, I],
         "mk_attention_mfma_max_rows": [I],
         "mk_attention_mfma": [P, I, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, P, P, P],

@@ -164,30 +164,39 @@ def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     return out
 
 
+def fuses_gating(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
+    """Whether `gated_projection` takes these operands (bfloat16, K a multiple of 8)."""
+    return (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
+            and x.shape[0] > 0 and x.shape[1] % 8 == 0 and w_gate_up.shape[0] % 2 == 0)
+
+
 def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
-    """act = silu(x Wg^T) * (x Wu^T) for few rows of bfloat16 x and W = [Wg | Wu] stacked
-    [2 I, K]: one kernel, the gating in the projection's epilogue."""
+    """act = silu(x Wg^T) * (x Wu^T) for bfloat16 x and W = [Wg | Wu] stacked [2 I, K]: one
+    kernel on the matrix cores, the gating in the projection's epilogue (the skinny kernel for
+    few rows, the tiled one for many)."""
     _dev(x, w_gate_up)
-    if not wants_partials(x, w_gate_up) or x.shape[1] != w_gate_up.shape[1] or w_gate_up.shape[0] % 2:
+    if not fuses_gating(x, w_gate_up) or x.shape[1] != w_gate_up.shape[1]:
         raise KernelArgumentError("gated_projection: operands not eligible")
     m, k = x.shape
     inter = w_gate_up.shape[0] // 2
     act = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
     lib = _lib.load("mfma")
-    _lib.check(lib, lib.mk_gated_skinny(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream()),
+    fn = lib.mk_gated_skinny if m <= SKINNY_MAX_ROWS else lib.mk_gated_tiled
+    _lib.check(lib, fn(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream()),
                "gated_projection")
     return act
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
            out: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
-           accumulate: bool = False, kernel: str = "auto") -> torch.Tensor:
+           accumulate: bool = False, kernel: str = "auto", tile_config: int = -1) -> torch.Tensor:
     """y = x W^T (+ bias) for x [M, K], W [N, K].
 
     With `accumulate` the product is added into the float32 tensor `out` (the residual
     stream) instead of being stored.  The result's dtype is `out_dtype` (default: x's).
     kernel: "auto" takes the matrix-core kernels for bfloat16 with K % 8 == 0 and the float32
-    multiply-add kernel otherwise; "generic" and "mfma" force one.
+    multiply-add kernel otherwise; "generic" and "mfma" force one.  tile_config picks the tile
+    shape of the matrix-core kernel for many rows (-1: by the problem's size).
     """
     _dev(x, w, bias, out)
     if x.dim() != 2 or w.dim() != 2 or x.shape[1] != w.shape[1]:
@@ -223,7 +232,8 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
             return out
         _lib.check(lib, lib.mk_linear_tiled(
             _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
-            _ptr(out), dtype_code(out_dtype), int(accumulate), m, n, k, n, _stream()), "linear")
+            _ptr(out), dtype_code(out_dtype), int(accumulate), m, n, k, n, tile_config,
+            _stream()), "linear")
         return out
     lib = _lib.load("core")
     _lib.check(lib, lib.mk_linear_generic(

@@ -41,8 +41,8 @@ class GatedMLP(FeedForward):
         return sum(t.numel() * t.element_size() for t in (self.w_gate_up, self.w_down))
 
     def forward(self, x, step, accum):
-        if ops.wants_partials(x, self.w_gate_up):
-            act = ops.gated_projection(x, self.w_gate_up)     # few rows: gated in the epilogue
+        if ops.fuses_gating(x, self.w_gate_up):
+            act = ops.gated_projection(x, self.w_gate_up)     # gated in the projection's epilogue
         else:
             act = ops.silu_mul(ops.linear(x, self.w_gate_up))
         if ops.wants_partials(act, self.w_down):

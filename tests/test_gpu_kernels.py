@@ -178,8 +178,9 @@ def test_tiled_projection(m, n, k):
     torch.testing.assert_close(acc_d.cpu(), acc + want, atol=5e-4, rtol=1e-4)
 
 
-@pytest.mark.parametrize("m,inter,k", [(1, 4864, 896), (8, 410, 168), (33, 704, 256), (64, 176, 64)])
-def test_gated_projection_few_rows(m, inter, k):
+@pytest.mark.parametrize("m,inter,k", [(1, 4864, 896), (8, 410, 168), (33, 704, 256), (64, 176, 64),
+                                       (65, 410, 168), (300, 4864, 896), (2048, 176, 64), (129, 704, 264)])
+def test_gated_projection(m, inter, k):
     """silu(x Wg^T) * (x Wu^T) with the gating in the projection's epilogue equals the gating
     kernel applied to the stored projection."""
     x_h, x_d = as_dtype(rnd(m, k, seed=31), torch.bfloat16)
