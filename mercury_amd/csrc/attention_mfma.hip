@@ -312,13 +312,12 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p
     } else {
       const size_t slot =
           (((size_t)tile * p.n_kv + kvh) * p.num_splits + split) * (16 * RT) + t * 16 + r;
-      if (b0 < b1) {  // an empty split only records that it is empty
-        float* po = p.part_o + slot * D + g4 * 4;
+      // An empty split writes its zeros too, so that the merge never reads stale memory.
+      float* po = p.part_o + slot * D + g4 * 4;
 #pragma unroll
-        for (int dt = 0; dt < D / 16; ++dt)
-          *(float4*)(po + dt * 16) = make_float4(st.acc[t][dt][0], st.acc[t][dt][1],
-                                                 st.acc[t][dt][2], st.acc[t][dt][3]);
-      }
+      for (int dt = 0; dt < D / 16; ++dt)
+        *(float4*)(po + dt * 16) = make_float4(st.acc[t][dt][0], st.acc[t][dt][1],
+                                               st.acc[t][dt][2], st.acc[t][dt][3]);
       if (g4 == 0) {
         p.part_ml[slot * 2] = st.m[t];
         p.part_ml[slot * 2 + 1] = l;
@@ -363,8 +362,7 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   for (int dim = threadIdx.x & 63; dim < D; dim += 64) {
     const float* src = p.part_o + ((base * R) + r) * D + dim;
     const size_t stride = (size_t)R * D;
-    // An empty split has weight 0 and holds nothing: it is not read.
-    auto term = [&](int s) { return weight[s] > 0.f ? src[(size_t)s * stride] * weight[s] : 0.f; };
+    auto term = [&](int s) { return src[(size_t)s * stride] * weight[s]; };
     float o = 0.f;
     int s = g;
     for (; s + 12 < S; s += 16) {

@@ -19,8 +19,7 @@
 //    into the residual stream.
 //
 // In both, lane l of a wavefront holds row (l % 16) and k-slots (l / 16) * 8 .. + 8 of an
-// operand; which k a slot means is free as long as A and B agree, and the skinny kernel uses
-// that to let each lane read 64 contiguous bytes per 128 k.
+// operand, so the four lanes of a row read 64 contiguous bytes per load instruction.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -74,17 +73,19 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(
     for (int b = 0; b < MT; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
   for (int step = step_begin + wave; step < step_end; step += SK_WAVES) {
-    const int kk = step * 128 + g4 * 32;  // this lane's 32 k of the step's 128
+    // Product j of the step takes k = step*128 + j*32 + g4*8 .. + 8 from this lane, so that
+    // one load instruction reads 64 contiguous bytes of each of its 16 rows.
+    const int kk = step * 128 + g4 * 8;
     Frag a[SK_NT][4], b[MT][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
-      const bool ok = kk + j * 8 < K;
+      const bool ok = kk + j * 32 < K;
 #pragma unroll
       for (int t = 0; t < SK_NT; ++t)
-        a[t][j].u = ok ? ld16(wrow[t] + kk + j * 8) : make_uint4(0, 0, 0, 0);
+        a[t][j].u = ok ? ld16(wrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
 #pragma unroll
       for (int t = 0; t < MT; ++t)
-        b[t][j].u = ok ? ld16(xrow[t] + kk + j * 8) : make_uint4(0, 0, 0, 0);
+        b[t][j].u = ok ? ld16(xrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
     }
 #pragma unroll
     for (int j = 0; j < 4; ++j)

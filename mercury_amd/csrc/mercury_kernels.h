@@ -109,8 +109,10 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
 
 // ---- library "core" again
 
+// parts: optional scratch of rows * 64 * 8 bytes; with it, few rows of a large vocabulary
+// are searched by 64 workgroups per row.
 int mk_argmax(const float* logits, int rows, int vocab, long long row_stride, int* out,
-              hipStream_t stream);
+              void* parts, hipStream_t stream);
 
 int mk_sample(const float* logits, int rows, int vocab, long long row_stride,
               const float* temperatures, const float* top_ps, const float* uniforms,

@@ -55,11 +55,47 @@ __global__ __launch_bounds__(SP_THREADS) void argmax_kernel(const float* __restr
   if (threadIdx.x == 0) out[blockIdx.x] = best.i;
 }
 
+// Two stages for few rows of a large vocabulary: ARGMAX_PARTS workgroups per row each take a
+// stretch of the row, then one wavefront per row picks among their results (lowest index
+// among equals, as in the single-stage kernel).
+#define ARGMAX_PARTS 64
+
+__global__ __launch_bounds__(256) void argmax_part_kernel(const float* __restrict__ logits,
+                                                          int vocab, long long row_stride,
+                                                          MaxIdx* __restrict__ parts) {
+  __shared__ MaxIdx scratch[256 / MK_WAVE];
+  const int row = blockIdx.y, part = blockIdx.x;
+  const int per = (vocab + ARGMAX_PARTS - 1) / ARGMAX_PARTS;
+  const int begin = min(vocab, part * per), count = min(vocab, begin + per) - begin;
+  MaxIdx best = block_argmax(logits + (size_t)row * row_stride + begin, count, scratch);
+  best.i = count > 0 ? best.i + begin : 0x7fffffff;
+  if (count <= 0) best.v = -INFINITY;
+  if (threadIdx.x == 0) parts[row * ARGMAX_PARTS + part] = best;
+}
+
+__global__ __launch_bounds__(MK_WAVE) void argmax_pick_kernel(const MaxIdx* __restrict__ parts,
+                                                              int* __restrict__ out) {
+  MaxIdx best = parts[blockIdx.x * ARGMAX_PARTS + threadIdx.x];
+#pragma unroll
+  for (int m = MK_WAVE / 2; m > 0; m >>= 1) {
+    MaxIdx o = {__shfl_xor(best.v, m, MK_WAVE), __shfl_xor(best.i, m, MK_WAVE)};
+    best = better(best, o);
+  }
+  if (threadIdx.x == 0) out[blockIdx.x] = best.i == 0x7fffffff ? 0 : best.i;
+}
+
 extern "C" int mk_argmax(const float* logits, int rows, int vocab, long long row_stride,
-                         int* out, hipStream_t stream) {
+                         int* out, void* parts, hipStream_t stream) {
   MK_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax: bad sizes");
   if (rows == 0) return 0;
-  argmax_kernel<<<rows, SP_THREADS, 0, stream>>>(logits, vocab, row_stride, out);
+  if (parts != nullptr && rows <= 256 && vocab >= 16384) {
+    static_assert(ARGMAX_PARTS == MK_WAVE, "the pick kernel reads one part per lane");
+    argmax_part_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, stream>>>(logits, vocab, row_stride,
+                                                                      (MaxIdx*)parts);
+    argmax_pick_kernel<<<rows, MK_WAVE, 0, stream>>>((const MaxIdx*)parts, out);
+  } else {
+    argmax_kernel<<<rows, SP_THREADS, 0, stream>>>(logits, vocab, row_stride, out);
+  }
   MK_LAUNCH_CHECK("argmax");
   return 0;
 }

@@ -128,7 +128,10 @@ def pack_step(chunks: list, manager, vocab_size: int, max_positions: int, pinned
 
     cu = np.zeros(num_seqs + 1, dtype=np.int64)
     np.cumsum(counts, out=cu[1:])
-    ids = np.concatenate([np.asarray(c.tokens, dtype=np.int64) for c in chunks])
+    if total == num_seqs:
+        ids = np.fromiter((c.tokens[0] for c in chunks), dtype=np.int64, count=num_seqs)
+    else:
+        ids = np.concatenate([np.asarray(c.tokens, dtype=np.int64) for c in chunks])
     if ids.min() < 0 or ids.max() >= vocab_size:
         raise BatchError(f"token id outside [0, {vocab_size})")
     starts = np.asarray([c.start for c in chunks], dtype=np.int64)
@@ -150,15 +153,16 @@ def pack_step(chunks: list, manager, vocab_size: int, max_positions: int, pinned
     if width < needed:
         raise BatchError(f"block tables of width {width} cannot hold {needed} pages")
     tables = []
+    needs = (-(-kv_len // ps)).tolist()
     for g in range(n_groups):
         t = np.full((num_seqs, width), -1, dtype=np.int64)
         for s, c in enumerate(chunks):
             pages = manager.table(c.key, g)
-            need = -(-int(kv_len[s]) // ps)
+            need = needs[s]
             if len(pages) < need:
                 raise BatchError(
                     f"sequence {c.key!r} holds {len(pages)} pages in group {g} but needs {need}")
-            t[s, :need] = pages[:need]
+            t[s, :need] = pages if len(pages) == need else pages[:need]
         tables.append(t)
 
     parts = [ids, positions, token_seq, cu, kv_len, np.asarray(slots, dtype=np.int64),

@@ -256,7 +256,7 @@ class Engine:
         if token is None:
             return
         index = len(r.out)
-        r.out.append(int(token))
+        r.append(int(token))
         if r.first_token_at is None:
             r.first_token_at = now
         self._emit(r, StreamEvent(rid=r.rid, kind="token", token=int(token), index=index, t=now))

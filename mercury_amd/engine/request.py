@@ -40,6 +40,7 @@ class Request:
     session_id: str | None = None
 
     out: list = field(default_factory=list)
+    tokens: list = field(default_factory=list, repr=False)   # prompt + out, kept in step
     num_computed: int = 0        # tokens whose keys and values are in the cache
     num_cached: int = 0          # of those, how many admission found already cached
     state: RequestState = RequestState.WAITING
@@ -51,13 +52,17 @@ class Request:
     recomputed_tokens: int = 0
     finish_reason: str | None = None
 
-    @property
-    def tokens(self) -> list:
-        return self.prompt + self.out
+    def __post_init__(self) -> None:
+        self.tokens = list(self.prompt) + list(self.out)
+
+    def append(self, token: int) -> None:
+        """Take a generated token."""
+        self.out.append(token)
+        self.tokens.append(token)
 
     @property
     def seq_len(self) -> int:
-        return len(self.prompt) + len(self.out)
+        return len(self.tokens)
 
     @property
     def remaining(self) -> int:

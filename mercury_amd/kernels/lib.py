@@ -26,7 +26,7 @@ _SIGNATURES = {
         "mk_attention_generic": [P, I, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
         "mk_silu_mul_partials": [P, I, L, P, I, I, I, P],
         "mk_qkv_finish": [P, I, L, P, I, P, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
-        "mk_argmax": [P, I, I, L, P, P],
+        "mk_argmax": [P, I, I, L, P, P, P],
         "mk_sample": [P, I, I, L, P, P, P, P, P, P],
     },
     "mfma": {

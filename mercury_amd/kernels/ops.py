@@ -431,9 +431,10 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
         raise KernelArgumentError("argmax: logits must be float32 [n, V]")
     rows, vocab = logits.shape
     out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
+    parts = torch.empty((rows, 64, 2), dtype=torch.int32, device=logits.device)
     lib = _lib.load("core")
-    _lib.check(lib, lib.mk_argmax(_ptr(logits), rows, vocab, vocab, _ptr(out), _stream()),
-               "argmax")
+    _lib.check(lib, lib.mk_argmax(_ptr(logits), rows, vocab, vocab, _ptr(out), _ptr(parts),
+                                  _stream()), "argmax")
     return out
 
 

@@ -563,6 +563,19 @@ def test_argmax_takes_the_lowest_index_among_equals():
     assert got[2] == 77 and got[4] == 1002
 
 
+def test_argmax_in_two_stages_over_a_large_vocabulary():
+    vocab = 151936
+    logits = rnd(9, vocab, seed=103)
+    logits[1, 0] = logits[1, vocab - 1] = 70.0         # equal maxima at both ends
+    logits[2, 2373] = logits[2, 2374] = 70.0           # and across a stage boundary
+    logits[3, vocab - 1] = 80.0
+    logits[4] = -1e30
+    logits[4, 77777] = -1e29
+    got = ops().argmax(logits.to(DEV)).cpu().tolist()
+    assert got == logits.argmax(-1).tolist()
+    assert got[1] == 0 and got[2] == 2373 and got[3] == vocab - 1 and got[4] == 77777
+
+
 def test_sampling_rules():
     """(reference: mercury/sampling.py:17-35)  Greedy rows take the argmax whatever top_p says;
     sampled rows follow the inverse CDF of the plain distribution for their own uniform."""

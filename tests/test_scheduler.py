@@ -38,7 +38,7 @@ def finish_step(plan):
     for w in plan.work:
         w.request.num_computed = w.start + w.count
         if w.emits:
-            w.request.out.append(1)
+            w.request.append(1)
 
 
 def rids(requests):
