@@ -383,7 +383,8 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     blocks = max(1, -(-span // 32))
     rows = 16
     total_rows = sum(count for _first, count, _start in step.spans) * group
-    max_rows = lib.mk_attention_mfma_max_rows(head_dim)
+    # 64-row tiles exist but run at one wavefront per SIMD; 32 rows measured fastest
+    max_rows = min(32, lib.mk_attention_mfma_max_rows(head_dim))
     while rows < max_rows and (total_rows // (rows * 2)) * n_kv >= ATTENTION_WIDE_TILE_WAVES:
         rows *= 2
     if tile_rows is not None:
