@@ -32,6 +32,15 @@ QWEN25_05B = {
     "vocab_size": 151936, "rope_theta": 1000000.0, "rms_norm_eps": 1e-6,
     "tie_word_embeddings": True, "max_position_embeddings": 32768,
 }
+# The larger models of the family, for `--shape`.
+QWEN25_7B = dict(QWEN25_05B, hidden_size=3584, intermediate_size=18944, num_hidden_layers=28,
+                 num_attention_heads=28, num_key_value_heads=4, head_dim=128, vocab_size=152064,
+                 tie_word_embeddings=False)
+QWEN25_32B = dict(QWEN25_05B, hidden_size=5120, intermediate_size=27648, num_hidden_layers=64,
+                  num_attention_heads=40, num_key_value_heads=8, head_dim=128, vocab_size=152064,
+                  tie_word_embeddings=False)
+SHAPES = {"0.5b": ("Qwen2.5-0.5B", QWEN25_05B), "7b": ("Qwen2.5-7B", QWEN25_7B),
+          "32b": ("Qwen2.5-32B", QWEN25_32B)}
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
 BLOCK_SIZE = 16
@@ -45,6 +54,8 @@ def parse_args(argv=None):
     p.add_argument("--steps", type=int, default=64)
     p.add_argument("--warmup", type=int, default=8)
     p.add_argument("--batch", type=int, default=8)
+    p.add_argument("--shape", default="0.5b", choices=sorted(SHAPES),
+                   help="layer sizes of which model of the family")
     p.add_argument("--layers", type=int, default=None, help="run fewer layers than the model has")
     p.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     p.add_argument("--context", type=int, default=CONTEXT)
@@ -74,7 +85,7 @@ class Bench:
         from mercury_amd.engine.executor import GpuExecutor
         from mercury_amd.engine.runner import ModelRunner
         from mercury_amd.sampling import Sampler
-        from mercury_amd.weights import DictSource, load_weights, random_state
+        from mercury_amd.weights import RandomSource, load_weights
 
         self.torch = torch
         self.cfg = cfg
@@ -82,9 +93,7 @@ class Bench:
         t0 = time.time()
         model = build_model(cfg)
         torch_dtype = torch.bfloat16 if dtype == "bfloat16" else torch.float32
-        state = random_state(model, seed, std=0.02, dtype=torch_dtype)
-        load_weights(model, DictSource(state), torch_dtype, device)
-        del state
+        load_weights(model, RandomSource(model, seed, 0.02, torch_dtype, device), torch_dtype, device)
         pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + PREFILL_TOKENS // BLOCK_SIZE + 8
         self.engine_cfg = EngineConfig(
             model="random", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
@@ -170,7 +179,8 @@ def main(argv=None) -> int:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine "
               "has no multi-GPU path)")
         return 2
-    cfg = dict(QWEN25_05B)
+    model_name, shape = SHAPES[args.shape]
+    cfg = dict(shape)
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
@@ -193,7 +203,7 @@ def main(argv=None) -> int:
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     achieved = main_run["bytes"] / (main_run["ms"] * 1e-3) / 1e9
     line = {
-        "metric": "decode tok/s at batch 8, context 4096 (Qwen2.5-0.5B shapes)",
+        "metric": f"decode tok/s at batch {args.batch}, context {args.context} ({model_name} shapes)",
         "value": round(main_run["tok_s"], 1),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -204,9 +214,9 @@ def main(argv=None) -> int:
         "scaling": "weak",
         "vs_baseline": None,
         "dtype": short,
-        "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02)",
+        "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02) drawn on the GPU",
         "config": {
-            "model": "Qwen2.5-0.5B shapes", "layers": cfg["num_hidden_layers"],
+            "model": f"{model_name} shapes", "layers": cfg["num_hidden_layers"],
             "layers_full": full_layers, "hidden": cfg["hidden_size"],
             "heads": cfg["num_attention_heads"], "kv_heads": cfg["num_key_value_heads"],
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"],

@@ -85,13 +85,124 @@ __global__ void rmsnorm_kernel(float* __restrict__ h, const float* __restrict__ 
   }
 }
 
+// The same with 16-byte accesses and the row kept in registers between the two passes: thread
+// t holds chunks t, t + threads, ... (CH of them at most) of four values each, and asks for
+// its weights before it waits for the sum of squares.  Needs H % 4 == 0.
+template <int N>
+struct WeightChunk;
+template <>
+struct WeightChunk<0> {  // float32
+  static __device__ __forceinline__ float4 load(const void* w, int chunk) {
+    return ((const float4*)w)[chunk];
+  }
+};
+template <>
+struct WeightChunk<1> {  // bfloat16
+  static __device__ __forceinline__ float4 load(const void* w, int chunk) {
+    const uint2 u = ((const uint2*)w)[chunk];
+    return make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                       __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+  }
+};
+
+template <typename TO, int WBF16, int CH>
+__global__ void rmsnorm_vec_kernel(float* __restrict__ h, const float* __restrict__ partials,
+                                   int num_partials, size_t partial_stride,
+                                   const void* __restrict__ weight, float eps,
+                                   const int* __restrict__ rows, TO* __restrict__ out,
+                                   int hidden) {
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int in_row = rows ? rows[out_row] : out_row;
+  const int chunks = hidden >> 2;
+  float4* x4 = (float4*)(h + (size_t)in_row * hidden);
+  float4 v[CH], w[CH];
+  float sq = 0.f;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int idx = threadIdx.x + c * blockDim.x;
+    v[c] = make_float4(0.f, 0.f, 0.f, 0.f);
+    w[c] = v[c];
+    if (idx < chunks) {
+      v[c] = x4[idx];
+      w[c] = WeightChunk<WBF16>::load(weight, idx);
+    }
+  }
+  if (num_partials > 0) {
+#pragma unroll
+    for (int c = 0; c < CH; ++c) {
+      const int idx = threadIdx.x + c * blockDim.x;
+      if (idx >= chunks) continue;
+      const float4* p4 = (const float4*)(partials + (size_t)in_row * hidden) + idx;
+      const size_t stride4 = partial_stride >> 2;
+      float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
+      int k = 0;
+      for (; k + 4 <= num_partials; k += 4) {
+        const float4 a = p4[(size_t)k * stride4], b = p4[(size_t)(k + 1) * stride4];
+        const float4 cc = p4[(size_t)(k + 2) * stride4], d = p4[(size_t)(k + 3) * stride4];
+        t.x += (a.x + b.x) + (cc.x + d.x);
+        t.y += (a.y + b.y) + (cc.y + d.y);
+        t.z += (a.z + b.z) + (cc.z + d.z);
+        t.w += (a.w + b.w) + (cc.w + d.w);
+      }
+      for (; k < num_partials; ++k) {
+        const float4 a = p4[(size_t)k * stride4];
+        t.x += a.x;
+        t.y += a.y;
+        t.z += a.z;
+        t.w += a.w;
+      }
+      v[c] = make_float4(v[c].x + t.x, v[c].y + t.y, v[c].z + t.z, v[c].w + t.w);
+      x4[idx] = v[c];
+    }
+  }
+#pragma unroll
+  for (int c = 0; c < CH; ++c)
+    sq += (v[c].x * v[c].x + v[c].y * v[c].y) + (v[c].z * v[c].z + v[c].w * v[c].w);
+  const float total = block_sum(sq, scratch);
+  const float rstd = rsqrtf(total / (float)hidden + eps);
+  TO* dst = out + (size_t)out_row * hidden;
+#pragma unroll
+  for (int c = 0; c < CH; ++c) {
+    const int idx = threadIdx.x + c * blockDim.x;
+    if (idx >= chunks) continue;
+    const float a = Elem<TO>::round(v[c].x * rstd) * w[c].x, b = Elem<TO>::round(v[c].y * rstd) * w[c].y;
+    const float cc = Elem<TO>::round(v[c].z * rstd) * w[c].z, d = Elem<TO>::round(v[c].w * rstd) * w[c].w;
+    if constexpr (sizeof(TO) == 2) {
+      *(uint2*)(dst + 4 * idx) = make_uint2(pack_bf16x2(a, b), pack_bf16x2(cc, d));
+    } else {
+      *(float4*)(dst + 4 * idx) = make_float4(a, b, cc, d);
+    }
+  }
+}
+
 template <typename TO>
 static int launch_rmsnorm(float* h, const float* partials, int num_partials,
                           size_t partial_stride, const void* weight, int weight_dtype, float eps,
                           const int* rows, TO* out, int out_rows, int hidden,
                           hipStream_t stream) {
-  // Few rows (decoding): as many threads per row as it has elements, so that every thread
-  // waits for one group of loads only.
+  // Few rows (decoding): as many threads per row as it has chunks of four, so that every
+  // thread waits for one group of loads only; many rows: 256 threads each.
+  if (hidden % 4 == 0 && (num_partials == 0 || partial_stride % 4 == 0)) {
+    const int chunks = hidden / 4;
+    int threads = out_rows <= 256 ? (chunks + 63) / 64 * 64 : 256;
+    if (threads > 1024) threads = 1024;
+    const int ch = (chunks + threads - 1) / threads;
+#define RMS_VEC(CH)                                                                            \
+  do {                                                                                         \
+    if (weight_dtype == MK_F32)                                                                \
+      rmsnorm_vec_kernel<TO, 0, CH><<<out_rows, threads, 0, stream>>>(                         \
+          h, partials, num_partials, partial_stride, weight, eps, rows, out, hidden);          \
+    else                                                                                       \
+      rmsnorm_vec_kernel<TO, 1, CH><<<out_rows, threads, 0, stream>>>(                         \
+          h, partials, num_partials, partial_stride, weight, eps, rows, out, hidden);          \
+    return 0;                                                                                  \
+  } while (0)
+    if (ch == 1) RMS_VEC(1);
+    if (ch == 2) RMS_VEC(2);
+    if (ch <= 4) RMS_VEC(4);
+#undef RMS_VEC
+  }
   int threads = hidden >= 512 ? 256 : (hidden >= 256 ? 128 : 64);
   if (out_rows <= 64 && num_partials > 0) threads = hidden >= 1024 ? 1024 : (hidden + 63) / 64 * 64;
   if (weight_dtype == MK_F32)

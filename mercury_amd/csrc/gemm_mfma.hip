@@ -4,13 +4,15 @@
 //
 //  * skinny (M <= 64, decoding): the weights are read once, straight from HBM into the A
 //    operand of v_mfma_f32_16x16x32_bf16 (16 rows of W by 32 k per instruction); the few rows
-//    of x are the B operand and come out of the L2.  A workgroup owns 32 rows of W and one
-//    slice of K, its wavefronts taking the slice's k-steps in turn.  Splitting K gives the
-//    small matrices of a small model enough wavefronts to pull their bytes; every slice
-//    writes its own float32 partial result [slice, M, N], and whichever kernel consumes the
-//    projection (RMSNorm, rotary + cache write) adds the slices up in slice order, so results
-//    are reproducible.  The gate/up projection keeps all of K in one workgroup and gates in
-//    its epilogue.
+//    of x are the B operand and come out of the L2.  A workgroup owns 16 or 32 rows of W, its
+//    wavefronts taking the k-steps in turn.  Where those workgroups occupy the chip, or the
+//    matrix is too small for bandwidth to matter, a workgroup keeps all of K and finishes the
+//    job in its epilogue: adds into the float32 residual stream, gates (gate/up projection),
+//    or adds the bias, rotates and writes q and the paged cache (q/k/v projection).
+//    Otherwise K is split:
+//    every slice writes its own float32 partial result [slice, M, N], and whichever kernel
+//    consumes the projection (RMSNorm, rotary + cache write) adds the slices up in slice
+//    order, so results are reproducible.
 //
 //  * tiled (M > 64, prompts): tiles of y per workgroup of four wavefronts (128 x 128, or
 //    smaller when the matrix would otherwise leave compute units idle), K in stages through
@@ -35,71 +37,170 @@ __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *(const uint4*)p
 
 // ------------------------------------------------------------------------------ skinny
 
-#define SK_NT 2     // 16-row tiles of W per workgroup
 #define SK_WAVES 4  // wavefronts of a workgroup; they share the rows and split the k-steps
 
-// Each workgroup owns 32 rows of W (two 16-row tiles) and one slice of K; its four wavefronts
-// take the slice's 128-wide k-steps in turn (wave w: steps w, w + 4, ...) and add their
-// results up through LDS in wave order, so a slice yields one partial result.
-//   GATED = 0: out[(slice * M + m) * N + n] float32, tiles are rows n0.. and n0 + 16..
-//   GATED = 1: W is [gate rows | up rows] of N each; the two tiles are gate rows n0.. and the
-//              matching up rows N + n0.., the slice must be all of K, and the epilogue writes
-//              act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
-template <int MT, int GATED>
-__global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(
-    const bf16_t* __restrict__ x, const bf16_t* __restrict__ w, void* __restrict__ out_, int M,
-    int N, int K, int steps_per_slice) {
-  __shared__ float red[SK_WAVES - 1][SK_NT * MT * 4][64];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g4 = lane >> 4;
-  const int n0 = blockIdx.x * (GATED ? 16 : 16 * SK_NT);
-  const int slice = blockIdx.y;
-  const int step_begin = slice * steps_per_slice;
-  const int step_end = min((K + 127) / 128, step_begin + steps_per_slice);
+// What a workgroup's rows of W are and what becomes of the result:
+//   SK_PARTIAL  rows n0.. of W; out[(slice * M + m) * N + n] float32, one slice of K each.
+//   SK_GATED    W is [gate rows | up rows] of N each; tile 0 is gate rows n0.., tile 1 the
+//               matching up rows N + n0..; act[m][n] = silu(g) * u in bfloat16
+//               (reference: mercury/model/qwen2.py:42).  All of K in the workgroup.
+//   SK_ACC      rows n0.. of W; out[m][n] += y (+ bias) in float32: the residual stream takes
+//               the projection directly.  All of K in the workgroup.
+//   SK_QKV      W is [q heads | k heads | v heads] of d rows each; tile 0 is rows j*16.. of a
+//               head's first half and tile 1 the same rows of its second half, so every lane
+//               holds both members of a rotation pair: bias, rounding, rotation by the token's
+//               position, q to `q_out`, k and v into the paged cache.  All of K.
+enum { SK_PARTIAL = 0, SK_GATED = 1, SK_ACC = 2, SK_QKV = 3 };
 
-  const bf16_t* wrow[SK_NT];
+struct SkinnyArgs {
+  const bf16_t* x;  // [M, K]
+  const bf16_t* w;
+  void* out;
+  int M, N, K, steps_per_slice;
+  const void* bias;  // SK_ACC, SK_QKV: [N] or null
+  int bias_bf16;
+  // SK_QKV
+  bf16_t* q_out;
+  const float* cos_table;
+  const float* sin_table;
+  const int* positions;
+  const int* token_seq;
+  const int* block_table;
+  int table_stride;
+  bf16_t* k_cache;
+  bf16_t* v_cache;
+  int page_shift, n_q, n_kv, d, rotate;
+};
+
+__device__ __forceinline__ float load_scalar(const void* p, int is_bf16, int i) {
+  return is_bf16 ? bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
+}
+
+// One workgroup: NT tiles of 16 rows of W, its four wavefronts taking the slice's 128-wide
+// k-steps in turn (wave w: steps w, w + 4, ...), the next step's loads in flight during the
+// current step's products; the wavefronts' results are added through LDS in wave order.
+// Product j of a step takes k = step*128 + j*32 + g4*8 .. + 8 from a lane, so that one load
+// instruction reads 64 contiguous bytes of each of its 16 rows.
+template <int MT, int NT, int EPI>
+__global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
+  static_assert((EPI != SK_GATED && EPI != SK_QKV) || NT == 2, "paired tiles");
+  __shared__ float red[SK_WAVES - 1][NT * MT * 4][64];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g4 = lane >> 4;
+  const int M = p.M, N = p.N, K = p.K;
+  const int slice = blockIdx.y;
+  const int step_begin = slice * p.steps_per_slice;
+  const int step_end = min((K + 127) / 128, step_begin + p.steps_per_slice);
+
+  // SK_QKV: the head and the 16-row stretch of its halves this workgroup owns.
+  const int per_head = EPI == SK_QKV ? p.d / 32 : 1;
+  const int head = EPI == SK_QKV ? blockIdx.x / per_head : 0;
+  const int dd0 = EPI == SK_QKV ? (blockIdx.x - head * per_head) * 16 : 0;
+  const int n0 = EPI == SK_QKV ? head * p.d + dd0 : blockIdx.x * (EPI == SK_GATED ? 16 : 16 * NT);
+
+  const bf16_t* wrow[NT];
 #pragma unroll
-  for (int t = 0; t < SK_NT; ++t) {
-    const int row = GATED ? t * N + min(n0 + r, N - 1) : min(n0 + t * 16 + r, N - 1);
-    wrow[t] = w + (size_t)row * K;
+  for (int t = 0; t < NT; ++t) {
+    int row;
+    if (EPI == SK_GATED) row = t * N + min(n0 + r, N - 1);
+    else if (EPI == SK_QKV) row = n0 + t * (p.d / 2) + r;
+    else row = min(n0 + t * 16 + r, N - 1);
+    wrow[t] = p.w + (size_t)row * K;
   }
   const bf16_t* xrow[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xrow[t] = x + (size_t)min(t * 16 + r, M - 1) * K;
+  for (int t = 0; t < MT; ++t) xrow[t] = p.x + (size_t)min(t * 16 + r, M - 1) * K;
 
-  f32x4 acc[SK_NT][MT];
-#pragma unroll
-  for (int a = 0; a < SK_NT; ++a)
-#pragma unroll
-    for (int b = 0; b < MT; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
-
-  for (int step = step_begin + wave; step < step_end; step += SK_WAVES) {
-    // Product j of the step takes k = step*128 + j*32 + g4*8 .. + 8 from this lane, so that
-    // one load instruction reads 64 contiguous bytes of each of its 16 rows.
+  Frag a[2][NT][4], b[2][MT][4];
+  auto load_w = [&](int buf, int step) {
     const int kk = step * 128 + g4 * 8;
-    Frag a[SK_NT][4], b[MT][4];
 #pragma unroll
     for (int j = 0; j < 4; ++j) {
       const bool ok = kk + j * 32 < K;
 #pragma unroll
-      for (int t = 0; t < SK_NT; ++t)
-        a[t][j].u = ok ? ld16(wrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
+      for (int t = 0; t < NT; ++t)
+        a[buf][t][j].u = ok ? ld16(wrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
+    }
+  };
+  auto load_x = [&](int buf, int step) {
+    const int kk = step * 128 + g4 * 8;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const bool ok = kk + j * 32 < K;
 #pragma unroll
       for (int t = 0; t < MT; ++t)
-        b[t][j].u = ok ? ld16(xrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
+        b[buf][t][j].u = ok ? ld16(xrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
     }
+  };
+
+  int step = step_begin + wave;
+  if (step < step_end) load_w(0, step);
+
+  // SK_ACC: the values the result is added to are asked for now, by the wavefront that will
+  // write them, so that the epilogue does not wait for them.
+  const bool vec_out = (N & 3) == 0;
+  float4 old[NT][MT];
+  if constexpr (EPI == SK_ACC) {
+    if (wave == 0 && vec_out) {
+#pragma unroll
+      for (int ta = 0; ta < NT; ++ta)
+#pragma unroll
+        for (int tb = 0; tb < MT; ++tb) {
+          const int m = tb * 16 + r, n = n0 + ta * 16 + g4 * 4;
+          old[ta][tb] = (m < M && n + 3 < N) ? *(const float4*)((const float*)p.out + (size_t)m * N + n)
+                                             : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+    }
+  }
+
+  if (step < step_end) load_x(0, step);
+
+  f32x4 acc[NT][MT];
+#pragma unroll
+  for (int ta = 0; ta < NT; ++ta)
+#pragma unroll
+    for (int tb = 0; tb < MT; ++tb) acc[ta][tb] = (f32x4){0.f, 0.f, 0.f, 0.f};
+
+  auto products = [&](int buf) {
 #pragma unroll
     for (int j = 0; j < 4; ++j)
 #pragma unroll
-      for (int ta = 0; ta < SK_NT; ++ta)
+      for (int ta = 0; ta < NT; ++ta)
 #pragma unroll
         for (int tb = 0; tb < MT; ++tb)
-          acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[ta][j].v, b[tb][j].v,
+          acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[buf][ta][j].v, b[buf][tb][j].v,
                                                                 acc[ta][tb], 0, 0, 0);
+  };
+  // Two steps in flight where the registers allow four wavefronts a SIMD; with three or four
+  // tiles of x rows the second buffer would halve that, and one step at a time is faster.
+  constexpr bool PIPELINED = MT <= 2;
+  if constexpr (!PIPELINED) {
+    for (; step < step_end; step += SK_WAVES) {
+      products(0);
+      if (step + SK_WAVES < step_end) {
+        load_w(0, step + SK_WAVES);
+        load_x(0, step + SK_WAVES);
+      }
+    }
+  }
+  for (; step < step_end; step += 2 * SK_WAVES) {
+    const bool more = step + SK_WAVES < step_end;
+    if (more) {
+      load_w(1, step + SK_WAVES);
+      load_x(1, step + SK_WAVES);
+    }
+    products(0);
+    if (more) {
+      if (step + 2 * SK_WAVES < step_end) {
+        load_w(0, step + 2 * SK_WAVES);
+        load_x(0, step + 2 * SK_WAVES);
+      }
+      products(1);
+    }
   }
 
   if (wave > 0) {
 #pragma unroll
-    for (int ta = 0; ta < SK_NT; ++ta)
+    for (int ta = 0; ta < NT; ++ta)
 #pragma unroll
       for (int tb = 0; tb < MT; ++tb)
 #pragma unroll
@@ -110,19 +211,19 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(
 #pragma unroll
   for (int v = 0; v < SK_WAVES - 1; ++v)
 #pragma unroll
-    for (int ta = 0; ta < SK_NT; ++ta)
+    for (int ta = 0; ta < NT; ++ta)
 #pragma unroll
       for (int tb = 0; tb < MT; ++tb)
 #pragma unroll
         for (int i = 0; i < 4; ++i) acc[ta][tb][i] += red[v][(ta * MT + tb) * 4 + i][lane];
 
-  // acc[ta][tb][i] = y[m = tb*16 + r][column g4*4 + i of tile ta]
+  // acc[ta][tb][i] = y[m = tb*16 + r][row g4*4 + i of tile ta]
 #pragma unroll
   for (int tb = 0; tb < MT; ++tb) {
     const int m = tb * 16 + r;
     if (m >= M) continue;
-    if (GATED) {
-      bf16_t* dst = (bf16_t*)out_ + (size_t)m * N;
+    if constexpr (EPI == SK_GATED) {
+      bf16_t* dst = (bf16_t*)p.out + (size_t)m * N;
       const int n = n0 + g4 * 4;
       bf16_t o[4];
 #pragma unroll
@@ -137,18 +238,84 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(
         for (int i = 0; i < 4; ++i)
           if (n + i < N) dst[n + i] = o[i];
       }
-    } else {
-      float* dst = (float*)out_ + ((size_t)slice * M + m) * N;
+    } else if constexpr (EPI == SK_QKV) {
+      // Both halves of 4 rotation pairs of one head: dims dd.. and dd + d/2..
+      const int d = p.d, half = d / 2, dd = dd0 + g4 * 4;
+      const int pos = p.positions[m];
+      float lo[4], hi[4];
 #pragma unroll
-      for (int ta = 0; ta < SK_NT; ++ta) {
+      for (int i = 0; i < 4; ++i) {
+        float u = acc[0][tb][i], v = acc[1][tb][i];
+        if (p.bias) {
+          u += load_scalar(p.bias, p.bias_bf16, n0 + g4 * 4 + i);
+          v += load_scalar(p.bias, p.bias_bf16, n0 + half + g4 * 4 + i);
+        }
+        lo[i] = Elem<bf16_t>::round(u);
+        hi[i] = Elem<bf16_t>::round(v);
+      }
+      const bool is_v = head >= p.n_q + p.n_kv;
+      if (p.rotate && !is_v) {
+        const float4 c = *(const float4*)(p.cos_table + (size_t)pos * half + dd);
+        const float4 s = *(const float4*)(p.sin_table + (size_t)pos * half + dd);
+        const float cs[4] = {c.x, c.y, c.z, c.w}, sn[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          const float u = lo[i], v = hi[i];
+          lo[i] = u * cs[i] - v * sn[i];
+          hi[i] = v * cs[i] + u * sn[i];
+        }
+      }
+      const ushort4 lo4 = make_ushort4(f32_to_bf16(lo[0]), f32_to_bf16(lo[1]), f32_to_bf16(lo[2]),
+                                       f32_to_bf16(lo[3]));
+      const ushort4 hi4 = make_ushort4(f32_to_bf16(hi[0]), f32_to_bf16(hi[1]), f32_to_bf16(hi[2]),
+                                       f32_to_bf16(hi[3]));
+      if (head < p.n_q) {
+        bf16_t* dst = p.q_out + (size_t)m * p.n_q * d + head * d + dd;
+        *(ushort4*)dst = lo4;
+        *(ushort4*)(dst + half) = hi4;
+      } else {
+        const int page = p.block_table[(size_t)p.token_seq[m] * p.table_stride + (pos >> p.page_shift)];
+        if (page < 0) continue;
+        const int ps = 1 << p.page_shift, off = pos & (ps - 1);
+        if (!is_v) {
+          const int kh = head - p.n_q;
+          bf16_t* dst = p.k_cache + (((size_t)page * p.n_kv + kh) * ps + off) * d + dd;
+          *(ushort4*)dst = lo4;
+          *(ushort4*)(dst + half) = hi4;
+        } else {
+          const int vh = head - p.n_q - p.n_kv;
+          bf16_t* dst = p.v_cache + (((size_t)page * p.n_kv + vh) * d + dd) * ps + off;
+          const bf16_t l[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, h4[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
+#pragma unroll
+          for (int i = 0; i < 4; ++i) {
+            dst[(size_t)i * ps] = l[i];
+            dst[(size_t)(half + i) * ps] = h4[i];
+          }
+        }
+      }
+    } else {
+      float* dst = (float*)p.out + ((size_t)(EPI == SK_PARTIAL ? slice : 0) * M + m) * N;
+#pragma unroll
+      for (int ta = 0; ta < NT; ++ta) {
         const int n = n0 + ta * 16 + g4 * 4;
-        if (n + 3 < N && (N & 3) == 0) {
-          *(float4*)(dst + n) =
-              make_float4(acc[ta][tb][0], acc[ta][tb][1], acc[ta][tb][2], acc[ta][tb][3]);
+        float y[4] = {acc[ta][tb][0], acc[ta][tb][1], acc[ta][tb][2], acc[ta][tb][3]};
+        if constexpr (EPI == SK_ACC) {
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            if (p.bias && n + i < N) y[i] += load_scalar(p.bias, p.bias_bf16, n + i);
+        }
+        if (n + 3 < N && vec_out) {
+          float4* q = (float4*)(dst + n);
+          if constexpr (EPI == SK_ACC) {
+            const float4 o = old[ta][tb];
+            *q = make_float4(o.x + y[0], o.y + y[1], o.z + y[2], o.w + y[3]);
+          } else {
+            *q = make_float4(y[0], y[1], y[2], y[3]);
+          }
         } else {
 #pragma unroll
           for (int i = 0; i < 4; ++i)
-            if (n + i < N) dst[n + i] = acc[ta][tb][i];
+            if (n + i < N) dst[n + i] = EPI == SK_ACC ? dst[n + i] + y[i] : y[i];
         }
       }
     }
@@ -159,7 +326,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(
 // 512), every wavefront of a workgroup with at least one k-step, and no more partial results
 // than the weights are worth (slices * M * 4 bytes per output column against K * 2).
 extern "C" int mk_linear_skinny_slices(int M, int N, int K) {
-  const int tiles = (N + 16 * SK_NT - 1) / (16 * SK_NT);
+  const int tiles = (N + 31) / 32;
   const int steps = (K + 127) / 128;
   int slices = (512 + tiles - 1) / tiles;
   const int by_steps = (steps + SK_WAVES - 1) / SK_WAVES;
@@ -171,15 +338,37 @@ extern "C" int mk_linear_skinny_slices(int M, int N, int K) {
   return (steps + per - 1) / per;
 }
 
-template <int GATED>
-static void launch_skinny(const bf16_t* x, const bf16_t* w, void* out, int M, int N, int K,
-                          int per, dim3 grid, hipStream_t stream) {
-  switch ((M + 15) / 16) {
-    case 1: gemm_skinny_kernel<1, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
-    case 2: gemm_skinny_kernel<2, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
-    case 3: gemm_skinny_kernel<3, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
-    default: gemm_skinny_kernel<4, GATED><<<grid, 64 * SK_WAVES, 0, stream>>>(x, w, out, M, N, K, per); break;
+// Whether a projection added straight into the residual stream should keep all of K in one
+// workgroup (no partial results, one kernel less to wait for): when 16-row workgroups alone
+// occupy most of the chip, or when the matrix is so small that latency, not bandwidth, is
+// what its kernel costs.  One workgroup alone pulls about 35 GB/s.
+extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
+  (void)M;
+  const int tiles16 = (N + 15) / 16;
+  return tiles16 >= 192 || (double)N * K * 2.0 <= 4.0e6;
+}
+
+template <int NT, int EPI>
+static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream) {
+  switch ((a.M + 15) / 16) {
+    case 1: gemm_skinny_kernel<1, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
+    case 2: gemm_skinny_kernel<2, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
+    case 3: gemm_skinny_kernel<3, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
+    default: gemm_skinny_kernel<4, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
   }
+}
+
+static SkinnyArgs skinny_args(const void* x, const void* w, void* out, int M, int N, int K,
+                              int steps_per_slice) {
+  SkinnyArgs a = {};
+  a.x = (const bf16_t*)x;
+  a.w = (const bf16_t*)w;
+  a.out = out;
+  a.M = M;
+  a.N = N;
+  a.K = K;
+  a.steps_per_slice = steps_per_slice;
+  return a;
 }
 
 extern "C" int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int K,
@@ -191,11 +380,29 @@ extern "C" int mk_linear_skinny(const void* x, const void* w, float* out, int M,
              steps);
   const int per = (steps + slices - 1) / slices;
   MK_REQUIRE((per * (slices - 1)) < steps, "skinny projection: an empty slice");
-  const int tiles = (N + 16 * SK_NT - 1) / (16 * SK_NT);
   MK_REQUIRE(slices <= 65535, "skinny projection: too many slices");
-  launch_skinny<0>((const bf16_t*)x, (const bf16_t*)w, out, M, N, K, per, dim3(tiles, slices),
-                   stream);
+  launch_skinny<2, SK_PARTIAL>(skinny_args(x, w, out, M, N, K, per),
+                                      dim3((N + 31) / 32, slices), stream);
   MK_LAUNCH_CHECK("linear_skinny");
+  return 0;
+}
+
+// out[M, N] (float32) += x W^T (+ bias), 1 <= M <= 64, all of K in each workgroup.
+extern "C" int mk_linear_skinny_acc(const void* x, const void* w, const void* bias,
+                                    int bias_dtype, float* out, int M, int N, int K,
+                                    hipStream_t stream) {
+  MK_REQUIRE(M >= 1 && M <= 64, "skinny projection: M=%d outside 1..64", M);
+  MK_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny projection: K=%d must be a multiple of 8", K);
+  MK_REQUIRE(bias_dtype == MK_F32 || bias_dtype == MK_BF16, "skinny projection: bias dtype");
+  SkinnyArgs a = skinny_args(x, w, out, M, N, K, (K + 127) / 128);
+  a.bias = bias;
+  a.bias_bf16 = bias_dtype == MK_BF16;
+  // 16 rows a workgroup until those alone are more workgroups than the chip holds at once
+  if ((N + 15) / 16 <= 1024)
+    launch_skinny<1, SK_ACC>(a, dim3((N + 15) / 16, 1), stream);
+  else
+    launch_skinny<2, SK_ACC>(a, dim3((N + 31) / 32, 1), stream);
+  MK_LAUNCH_CHECK("linear_skinny_acc");
   return 0;
 }
 
@@ -205,10 +412,52 @@ extern "C" int mk_gated_skinny(const void* x, const void* w, void* act, int M, i
   MK_REQUIRE(M >= 1 && M <= 64, "gated projection: M=%d outside 1..64", M);
   MK_REQUIRE(inter > 0 && K > 0 && K % 8 == 0, "gated projection: K=%d must be a multiple of 8",
              K);
-  const int steps = (K + 127) / 128;
-  launch_skinny<1>((const bf16_t*)x, (const bf16_t*)w, act, M, inter, K, steps,
-                   dim3((inter + 15) / 16, 1), stream);
+  launch_skinny<2, SK_GATED>(skinny_args(x, w, act, M, inter, K, (K + 127) / 128),
+                             dim3((inter + 15) / 16, 1), stream);
   MK_LAUNCH_CHECK("gated_skinny");
+  return 0;
+}
+
+// The q/k/v projection of 1 <= M <= 64 tokens with everything that follows it: bias, rotation
+// of q and k by the token's position (full head width, or none), q [M, n_q d] out, k and v
+// into the paged cache (n_kv = 0: queries only).  W is [(n_q + 2 n_kv) d, K].
+// Formulas: reference mercury/model/qwen2.py:57-64, mercury/model/rope.py:19-29.
+extern "C" int mk_qkv_skinny(const void* x, const void* w, const void* bias, int bias_dtype,
+                             void* q_out, const float* cos_table, const float* sin_table,
+                             int table_positions, const int* positions, const int* token_seq,
+                             const int* block_table, int table_stride, void* k_cache,
+                             void* v_cache, int page_size, int n_q, int n_kv, int d, int rotate,
+                             int M, int K, hipStream_t stream) {
+  MK_REQUIRE(M >= 1 && M <= 64, "qkv projection: M=%d outside 1..64", M);
+  MK_REQUIRE(n_q > 0 && n_kv >= 0 && d > 0 && d % 32 == 0,
+             "qkv projection: head size %d is not a multiple of 32", d);
+  MK_REQUIRE(K > 0 && K % 8 == 0, "qkv projection: K=%d must be a multiple of 8", K);
+  MK_REQUIRE(!rotate || (cos_table && sin_table && table_positions > 0),
+             "qkv projection: rotation needs the angle tables");
+  MK_REQUIRE(n_kv == 0 || (k_cache && v_cache && block_table && mk_is_pow2(page_size)),
+             "qkv projection: the cache and a power-of-two page size are required");
+  MK_REQUIRE(bias_dtype == MK_F32 || bias_dtype == MK_BF16, "qkv projection: bias dtype");
+  const int N = (n_q + 2 * n_kv) * d;
+  SkinnyArgs a = skinny_args(x, w, nullptr, M, N, K, (K + 127) / 128);
+  a.bias = bias;
+  a.bias_bf16 = bias_dtype == MK_BF16;
+  a.q_out = (bf16_t*)q_out;
+  a.cos_table = cos_table;
+  a.sin_table = sin_table;
+  a.positions = positions;
+  a.token_seq = token_seq;
+  a.block_table = block_table;
+  a.table_stride = table_stride;
+  a.k_cache = (bf16_t*)k_cache;
+  a.v_cache = (bf16_t*)v_cache;
+  a.page_shift = mk_log2(page_size > 0 ? page_size : 1);
+  a.n_q = n_q;
+  a.n_kv = n_kv;
+  a.d = d;
+  a.rotate = rotate;
+  const dim3 grid((n_q + 2 * n_kv) * (d / 32), 1);
+  launch_skinny<2, SK_QKV>(a, grid, stream);
+  MK_LAUNCH_CHECK("qkv_skinny");
   return 0;
 }
 

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 1
+#define MK_ABI_VERSION 2
 
 #ifdef __cplusplus
 extern "C" {
@@ -71,9 +71,25 @@ int mk_linear_skinny_slices(int M, int N, int K);
 int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int K, int slices,
                      hipStream_t stream);
 
-// act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K].
+// out[M, N] (float32) += x W^T (+ bias) for 1 <= M <= 64, all of K in each workgroup;
+// mk_linear_skinny_unsplit says whether that keeps the chip busy for the shape.
+int mk_linear_skinny_unsplit(int M, int N, int K);
+int mk_linear_skinny_acc(const void* x, const void* w, const void* bias, int bias_dtype,
+                         float* out, int M, int N, int K, hipStream_t stream);
+
+// act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K],
+// 1 <= M <= 64.
 int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
                     hipStream_t stream);
+
+// The q/k/v projection of 1 <= M <= 64 tokens, w = [(n_q + 2 n_kv) d, K], with bias, rotation
+// of q and k over the whole head (rotate != 0), q [M, n_q d] out and k, v written to the
+// paged cache; n_kv = 0 projects the queries only.  d must be a multiple of 32.
+int mk_qkv_skinny(const void* x, const void* w, const void* bias, int bias_dtype, void* q_out,
+                  const float* cos_table, const float* sin_table, int table_positions,
+                  const int* positions, const int* token_seq, const int* block_table,
+                  int table_stride, void* k_cache, void* v_cache, int page_size, int n_q,
+                  int n_kv, int d, int rotate, int M, int K, hipStream_t stream);
 
 // The same for any M, tiled through LDS.
 int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K,

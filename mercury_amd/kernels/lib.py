@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 
 from . import build
 
-ABI_VERSION = 1
+ABI_VERSION = 2
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -32,7 +32,10 @@ _SIGNATURES = {
     "mfma": {
         "mk_linear_skinny_slices": [I, I, I],
         "mk_linear_skinny": [P, P, P, I, I, I, I, P],
+        "mk_linear_skinny_unsplit": [I, I, I],
+        "mk_linear_skinny_acc": [P, P, P, I, P, I, I, I, P],
         "mk_gated_skinny": [P, P, P, I, I, I, P],
+        "mk_qkv_skinny": [P, P, P, I, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_gated_tiled": [P, P, P, I, I, I, P],
         "mk_linear_tiled_config": [I, I, I],
         "mk_linear_tiled": [P, P, P, I, P, I, I, I, I, I, I, I, P],

@@ -144,6 +144,12 @@ def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether x W^T is best computed as K-split float32 partial sums (`linear_partials`):
     few rows of bfloat16 x, where the weights are the traffic and the chip needs the split to
     have enough wavefronts in flight."""
+    if not _skinny_eligible(x, w):
+        return False
+    return not _lib.load("mfma").mk_linear_skinny_unsplit(x.shape[0], w.shape[0], w.shape[1])
+
+
+def _skinny_eligible(x, w: torch.Tensor) -> bool:
     return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
             and 0 < x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0)
 
@@ -152,7 +158,7 @@ def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """Float32 partial sums [P, M, N] of x W^T over P slices of K; the consumer (rmsnorm,
     rope_kv_write, silu_mul: their `partials` forms) adds them up in slice order."""
     _dev(x, w)
-    if not wants_partials(x, w) or x.shape[1] != w.shape[1]:
+    if not _skinny_eligible(x, w) or x.shape[1] != w.shape[1]:
         raise KernelArgumentError(f"linear_partials: x {tuple(x.shape)} / W {tuple(w.shape)} not eligible")
     m, k = x.shape
     n = w.shape[0]
@@ -229,6 +235,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
         if m <= SKINNY_MAX_ROWS and out_dtype == torch.float32 and bias is None and not accumulate:
             _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, 1, _stream()),
                        "linear")
+            return out
+        if m <= SKINNY_MAX_ROWS and accumulate:
+            _lib.check(lib, lib.mk_linear_skinny_acc(
+                _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
+                _ptr(out), m, n, k, _stream()), "linear")
             return out
         _lib.check(lib, lib.mk_linear_tiled(
             _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
@@ -332,6 +343,64 @@ def _qkv_finish(parts, cos, sin, positions, token_seq, block_table, k_cache, v_c
         _ptr(block_table), block_table.shape[1], _ptr(k_cache), _ptr(v_cache), page_size, n_q,
         n_kv if write_kv else 0, head_dim, rotary_dim, int(write_kv), tokens, _stream()),
         "qkv_finish")
+    return q
+
+
+def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
+    """Whether `qkv_project` runs as one kernel: few bfloat16 rows, K a multiple of 8, heads a multiple of 32 wide and rotated over their whole width or not at
+    all, pages a power of two."""
+    return (_skinny_eligible(x, w) and head_dim % 32 == 0 and rotary_dim in (0, head_dim)
+            and page_size > 0 and page_size & (page_size - 1) == 0)
+
+
+def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor | None,
+                sin: torch.Tensor | None, positions: torch.Tensor, token_seq: torch.Tensor,
+                block_table: torch.Tensor, k_cache: torch.Tensor | None,
+                v_cache: torch.Tensor | None, n_q: int, n_kv: int, head_dim: int,
+                rotary_dim: int, write_kv: bool = True) -> torch.Tensor:
+    """q, k, v = x W^T + bias for W = [q heads | k heads | v heads]; q and k rotated by their
+    positions; k and v written to the paged cache (`write_kv`; otherwise W holds the query
+    heads only).  Returns the rotated q [T, n_q d].
+
+    Few rows take one kernel (projection, bias, rotation and cache write in its epilogue);
+    otherwise the projection is followed by `rope_kv_write`."""
+    heads_kv = n_kv if write_kv else 0
+    width = (n_q + 2 * heads_kv) * head_dim
+    if w.shape[0] != width or w.shape[1] != x.shape[1]:
+        raise KernelArgumentError(f"qkv_project: W {tuple(w.shape)} is not [{width}, {x.shape[1]}]")
+    page_size = k_cache.shape[2] if write_kv and k_cache is not None else 1
+    if not fuses_qkv(x, w, head_dim, rotary_dim, page_size):
+        if wants_partials(x, w):
+            return rope_kv_write(linear_partials(x, w), cos, sin, positions, token_seq,
+                                 block_table, k_cache, v_cache, n_q, heads_kv, head_dim,
+                                 rotary_dim, write_kv, bias=bias, out_dtype=x.dtype)
+        return rope_kv_write(linear(x, w, bias), cos, sin, positions, token_seq, block_table,
+                             k_cache, v_cache, n_q, heads_kv, head_dim, rotary_dim, write_kv)
+    tokens, k = x.shape
+    _dev(x, w, bias, cos, sin, positions, token_seq, block_table, k_cache, v_cache)
+    _i32(positions, "positions")
+    _i32(token_seq, "token_seq")
+    _i32(block_table, "block_table")
+    if positions.shape[0] != tokens or token_seq.shape[0] != tokens:
+        raise KernelArgumentError("qkv_project: positions/token_seq must have one entry per token")
+    if bias is not None and bias.shape != (width,):
+        raise KernelArgumentError("qkv_project: bias does not match the projection width")
+    table_positions = 0
+    if rotary_dim:
+        if cos is None or sin is None or cos.dtype != torch.float32 or cos.shape != sin.shape \
+                or cos.shape[1] != rotary_dim // 2:
+            raise KernelArgumentError("qkv_project: float32 cos and sin tables of the rotary width are required")
+        table_positions = cos.shape[0]
+    if write_kv:
+        _check_caches("qkv_project", k_cache, v_cache, n_kv, head_dim, torch.bfloat16)
+    q = torch.empty((tokens, n_q * head_dim), dtype=torch.bfloat16, device=w.device)
+    lib = _lib.load("mfma")
+    _lib.check(lib, lib.mk_qkv_skinny(
+        _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32, _ptr(q),
+        _ptr(cos), _ptr(sin), table_positions, _ptr(positions), _ptr(token_seq),
+        _ptr(block_table), block_table.shape[1], _ptr(k_cache) if write_kv else 0,
+        _ptr(v_cache) if write_kv else 0, page_size, n_q, heads_kv, head_dim,
+        int(rotary_dim > 0), tokens, k, _stream()), "qkv_project")
     return q
 
 

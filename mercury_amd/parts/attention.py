@@ -87,16 +87,8 @@ class Attention(Mixer):
             # Reads a cache another entry fills: only the queries are projected.
             w, b = w[:n_q * d], None if b is None else b[:n_q * d]
         k_cache, v_cache = (cache.k, cache.v) if cache.writes else (None, None)
-        heads_kv = n_kv if cache.writes else 0
-        if ops.wants_partials(x, w):
-            # Few rows: K-split partial sums, added up by the rotary kernel.
-            q = ops.rope_kv_write(ops.linear_partials(x, w), pos.cos, pos.sin, step.positions,
-                                  step.token_seq, table, k_cache, v_cache, n_q, heads_kv, d,
-                                  pos.rotary_dim, cache.writes, bias=b, out_dtype=x.dtype)
-        else:
-            q = ops.rope_kv_write(ops.linear(x, w, b), pos.cos, pos.sin, step.positions,
-                                  step.token_seq, table, k_cache, v_cache, n_q, heads_kv, d,
-                                  pos.rotary_dim, cache.writes)
+        q = ops.qkv_project(x, w, b, pos.cos, pos.sin, step.positions, step.token_seq, table,
+                            k_cache, v_cache, n_q, n_kv, d, pos.rotary_dim, cache.writes)
         attended = ops.attention(q, q.shape[1], cache.k, cache.v, step, table, n_q, n_kv, d,
                                  self.scale, self.window)
         if self.b_o is None and ops.wants_partials(attended, self.w_o):

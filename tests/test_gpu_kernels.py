@@ -147,7 +147,6 @@ def test_skinny_projection_partial_sums(m, n, k):
     """Few rows on the matrix cores: float32 slices over K whose sum is the product."""
     x_h, x_d = as_dtype(rnd(m, k, seed=21), torch.bfloat16)
     w_h, w_d = as_dtype(rnd(n, k, seed=22, scale=0.1), torch.bfloat16)
-    assert ops().wants_partials(x_d, w_d)
     parts = ops().linear_partials(x_d, w_d)
     assert parts.dtype == torch.float32 and parts.shape[1:] == (m, n)
     want = (x_h.double() @ w_h.double().T).float()
@@ -191,6 +190,127 @@ def test_gated_projection(m, inter, k):
     torch.testing.assert_close(got.float().cpu(), want.float().cpu(), atol=2e-3, rtol=1.6e-2)
     plain_want = plain.gated_mlp(x_h, w_h[:inter], w_h[inter:], torch.eye(inter))
     torch.testing.assert_close(got.float().cpu(), plain_want, **tol(torch.bfloat16))
+
+
+def test_which_skinny_projections_are_split():
+    """K is split into partial sums only where the matrix is large and has too few rows to
+    occupy the chip with 16-row workgroups."""
+    def wants(m, n, k):
+        return ops().wants_partials(torch.zeros(m, k, dtype=torch.bfloat16, device=DEV),
+                                    torch.zeros(n, k, dtype=torch.bfloat16, device=DEV))
+    assert wants(8, 896, 4864)             # 8.7 MB behind 56 tiles of rows
+    assert not wants(8, 896, 896)          # small: latency is the cost, not bandwidth
+    assert not wants(8, 3584, 4096)        # 224 tiles of rows are workgroups enough
+    assert not wants(8, 896, 4868)         # K % 8 != 0: not for the matrix cores at all
+
+
+@pytest.mark.parametrize("m,n,k", [(1, 896, 896), (8, 1003, 168), (17, 130, 264), (64, 3584, 1024),
+                                   (33, 20000, 64), (5, 7, 8)])
+@pytest.mark.parametrize("bias_dtype", [None, torch.bfloat16, torch.float32])
+def test_skinny_projection_into_the_stream(m, n, k, bias_dtype):
+    """Few rows, all of K in a workgroup, the product (and a bias) added to the float32
+    stream in the epilogue."""
+    x_h, x_d = as_dtype(rnd(m, k, seed=41), torch.bfloat16)
+    w_h, w_d = as_dtype(rnd(n, k, seed=42, scale=0.1), torch.bfloat16)
+    acc = rnd(m, n, seed=43)
+    acc_d = acc.clone().to(DEV)
+    want = acc + (x_h.double() @ w_h.double().T).float()
+    bias_d = None
+    if bias_dtype is not None:
+        b_h, bias_d = as_dtype(rnd(n, seed=44), bias_dtype)
+        want = want + b_h
+    ops().linear(x_d, w_d, bias_d, out=acc_d, accumulate=True, kernel="mfma")
+    torch.testing.assert_close(acc_d.cpu(), want, atol=2e-4, rtol=1e-4)
+
+
+QKV_CASES = [  # n_q, n_kv, d, page, K, rows
+    (14, 2, 64, 16, 896, 8), (6, 1, 32, 8, 168, 1), (4, 4, 128, 32, 264, 17), (3, 1, 96, 16, 72, 64),
+    (2, 2, 64, 16, 64, 16)]
+
+
+@pytest.mark.parametrize("n_q,n_kv,d,page,k,m", QKV_CASES)
+@pytest.mark.parametrize("mode", ["plain", "unrotated", "queries_only"])
+def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(n_q, n_kv, d, page, k, m, mode):
+    """The fused q/k/v kernel for few rows equals projection, then rotary + cache write, and
+    the plain implementation; tokens sit on page edges, in several sequences, one of them on
+    a page that was given back."""
+    o = ops()
+    write_kv = mode != "queries_only"
+    rot = 0 if mode == "unrotated" else d
+    heads_kv = n_kv if write_kv else 0
+    width = (n_q + 2 * heads_kv) * d
+    theta, max_pos = 10000.0, 8 * page
+    cos, sin = rotary_tables(d, theta, max_pos)
+    w_h, w_d = as_dtype(rnd(width, k, seed=51, scale=0.05), torch.bfloat16)
+    b_h, b_d = as_dtype(rnd(width, seed=52), torch.bfloat16)
+    # positions around page edges, spread over three sequences
+    edge = [page - 1, page, 2 * page - 1, 0, 3 * page, 1]
+    positions = [edge[i % len(edge)] + (i // len(edge)) for i in range(m)]
+    token_seq = [i % 3 for i in range(m)]
+    seen = set()
+    for i in range(m):                       # one slot per (sequence, position)
+        while (token_seq[i], positions[i]) in seen:
+            positions[i] += 1
+        seen.add((token_seq[i], positions[i]))
+    table = torch.arange(1, 1 + 3 * 8, dtype=torch.int32).view(3, 8).contiguous()
+    dropped = None
+    if write_kv and m >= 3:
+        dropped = 2
+        table[token_seq[dropped], positions[dropped] // page] = -1
+    pos_d = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    seq_d = torch.tensor(token_seq, dtype=torch.int32, device=DEV)
+    caches = [[torch.zeros(32, n_kv, page, d, dtype=torch.bfloat16, device=DEV),
+               torch.zeros(32, n_kv, d, page, dtype=torch.bfloat16, device=DEV)] for _ in range(2)]
+    x_h, x_d = as_dtype(rnd(m, k, seed=55), torch.bfloat16)
+    x_in = x_d
+    assert o.fuses_qkv(x_in, w_d, d, rot, page)
+    cos_d, sin_d = (cos.to(DEV), sin.to(DEV)) if rot else (None, None)
+    q_got = o.qkv_project(x_in, w_d, b_d, cos_d, sin_d, pos_d, seq_d, table.to(DEV),
+                          caches[0][0] if write_kv else None, caches[0][1] if write_kv else None,
+                          n_q, n_kv, d, rot, write_kv)
+    assert q_got.shape == (m, n_q * d) and q_got.dtype == torch.bfloat16
+    stored = o.linear(x_d, w_d, b_d, kernel="mfma" if m > 64 else "auto")
+    q_ref = o.rope_kv_write(stored, cos_d, sin_d, pos_d, seq_d, table.to(DEV),
+                            caches[1][0] if write_kv else None, caches[1][1] if write_kv else None,
+                            n_q, heads_kv, d, rot, write_kv)[:, : n_q * d]
+    # q, k and v are rounded to bfloat16 before the rotation mixes two of them: an error of one
+    # rounding of the largest projected value can land on a small rotated one
+    bf = dict(atol=float(stored.float().abs().max()) * 2.0 ** -7, rtol=1.6e-2)
+    torch.testing.assert_close(q_got.float().cpu(), q_ref.float().cpu(), **bf)
+    if write_kv:
+        torch.testing.assert_close(caches[0][0].float().cpu(), caches[1][0].float().cpu(), **bf)
+        torch.testing.assert_close(caches[0][1].float().cpu(), caches[1][1].float().cpu(), **bf)
+        assert (caches[0][0] != 0).eq(caches[1][0] != 0).all()      # the same slots, no others
+        assert (caches[0][1] != 0).eq(caches[1][1] != 0).all()
+        assert caches[0][0].abs().sum() > 0
+    # and the plain implementation, from the formulas
+    y = ((x_h.double() @ w_h.double().T).float() + b_h).to(torch.bfloat16).float()
+    q = y[:, : n_q * d].view(m, n_q, d)
+    if rot:
+        full_cos, full_sin = plain.rotary_table(d, positions, theta)
+        kk = y[:, n_q * d: (n_q + n_kv) * d].view(m, n_kv, d) if write_kv else q[:, :1]
+        q, k_want = plain.apply_rotary(q, kk, full_cos, full_sin)
+    elif write_kv:
+        k_want = y[:, n_q * d: (n_q + n_kv) * d].view(m, n_kv, d)
+    torch.testing.assert_close(q_got.float().cpu().view(m, n_q, d), q, **bf)
+    if write_kv:
+        v_want = y[:, (n_q + n_kv) * d:].view(m, n_kv, d)
+        for t in range(m):
+            pg, off = int(table[token_seq[t], positions[t] // page]), positions[t] % page
+            if t == dropped:
+                assert pg < 0
+                continue
+            torch.testing.assert_close(caches[0][0][pg, :, off].float().cpu(), k_want[t], **bf)
+            torch.testing.assert_close(caches[0][1][pg, :, :, off].float().cpu(), v_want[t], **bf)
+
+
+def test_qkv_projection_falls_back_where_the_fused_kernel_does_not_apply():
+    o = ops()
+    x = torch.zeros(4, 64, dtype=torch.bfloat16, device=DEV)
+    assert not o.fuses_qkv(x, x, 48, 48, 16)          # heads not a multiple of 32 wide
+    assert not o.fuses_qkv(x, x, 64, 32, 16)          # rotation over part of the head
+    assert not o.fuses_qkv(x.float(), x.float(), 64, 64, 16)
+    assert not o.fuses_qkv(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), x, 64, 64, 16)
 
 
 def test_matrix_core_projection_refuses_what_it_cannot_do():
