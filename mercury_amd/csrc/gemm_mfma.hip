@@ -339,13 +339,14 @@ extern "C" int mk_linear_skinny_slices(int M, int N, int K) {
 }
 
 // Whether a projection added straight into the residual stream should keep all of K in one
-// workgroup (no partial results, one kernel less to wait for): when 16-row workgroups alone
-// occupy most of the chip, or when the matrix is so small that latency, not bandwidth, is
-// what its kernel costs.  One workgroup alone pulls about 35 GB/s.
+// workgroup (no partial results, one kernel less to wait for): for at most 16 rows of x,
+// when 16-row workgroups alone occupy most of the chip, or when the matrix is so small that
+// latency, not bandwidth, is what its kernel costs.  One workgroup alone pulls about 35 GB/s;
+// with more rows of x every workgroup re-reads so much of x from the L2 that fewer, larger
+// workgroups over slices of K are faster.
 extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
-  (void)M;
   const int tiles16 = (N + 15) / 16;
-  return tiles16 >= 192 || (double)N * K * 2.0 <= 4.0e6;
+  return M <= 16 && (tiles16 >= 192 || (double)N * K * 2.0 <= 4.0e6);
 }
 
 template <int NT, int EPI>

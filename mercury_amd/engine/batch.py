@@ -15,6 +15,11 @@ import numpy as np
 import torch
 
 
+class BatchError(ValueError):
+    """A step that cannot be run as given: a token id or position out of range, a wanted
+    place outside a sequence's tokens, pages missing from a block table."""
+
+
 @dataclass
 class SeqChunk:
     """The next tokens of one request.

@@ -10,10 +10,12 @@ returns sampled tokens; here one forward takes any mix and returns logits).
 
 from __future__ import annotations
 
+import numpy as np
 import torch
 
 from ..parts.base import LayerCache
-from .batch import SeqChunk, StepContext, build_step, context_from_packed, pack_step
+from .batch import (BatchError, SeqChunk, StepContext, build_step, context_from_packed,
+                    pack_step)
 
 
 class DecodeGraph:
@@ -33,6 +35,20 @@ class DecodeGraph:
         self.ctx = context_from_packed(packed, self.static)
         self.ctx.max_kv_len = kv_bound
         self.ctx.fresh_slots = []
+        # The host's copy of the step, kept between replays: a replay rewrites the few
+        # numbers that change (token ids, positions, lengths, new pages) and copies it whole.
+        self.host = torch.empty(packed.host.shape, dtype=torch.int32, pin_memory=True)
+        self.host.copy_(packed.host)
+        views, offset = [], 0
+        for size in packed.sizes:
+            views.append(self.host.numpy()[offset:offset + size])
+            offset += size
+        self.ids, self.positions, _seq, _cu, self.kv_len, self.slots, _rows = views[:7]
+        n = packed.num_seqs
+        self.tables = [views[7 + g].reshape(n, w) for g, w in enumerate(packed.widths)]
+        self.row_record = [None] * n                       # whose pages a table row mirrors
+        self.row_pages = [[0] * n for _ in packed.widths]  # and how many of them
+        self.appendable = [g.spec.window is None for g in runner.manager.groups]
         # Once outside the capture: loads libraries, fills the context's tile tables.
         side = torch.cuda.Stream(device=runner.device)
         side.wait_stream(torch.cuda.current_stream(runner.device))
@@ -44,8 +60,44 @@ class DecodeGraph:
         with torch.cuda.graph(self.graph):
             self.logits = runner.model.forward(self.ctx, runner.caches, runner.states)
 
-    def replay(self, packed) -> torch.Tensor:
-        self.static.copy_(packed.host, non_blocking=True)
+    def refill(self, chunks: list, manager, vocab_size: int, max_positions: int) -> None:
+        """Write this step's numbers into the host copy.  The previous replay's copy to the
+        device has finished: its logits have been read since."""
+        n = len(chunks)
+        self.ids[:] = [c.tokens[0] for c in chunks]
+        self.positions[:] = [c.start for c in chunks]
+        if self.ids.min() < 0 or self.ids.max() >= vocab_size:
+            raise BatchError(f"token id outside [0, {vocab_size})")
+        if self.positions.min() < 0 or self.positions.max() >= max_positions:
+            raise BatchError(f"a sequence would pass the limit of {max_positions} tokens")
+        np.add(self.positions, 1, out=self.kv_len)
+        ps = manager.page_size
+        requests = manager.requests
+        for s in range(n):
+            c = chunks[s]
+            record = requests[c.key]
+            need = c.start // ps + 1
+            same = record is self.row_record[s]
+            if not same:
+                self.row_record[s] = record
+                self.slots[s] = record.state_slot
+            for g, table in enumerate(self.tables):
+                have = self.row_pages[g][s]
+                if same and self.appendable[g] and have == need:
+                    continue
+                pages = record.tables[g]
+                if len(pages) < need:
+                    raise BatchError(
+                        f"sequence {c.key!r} holds {len(pages)} pages in group {g} but needs {need}")
+                if same and self.appendable[g] and have < need:
+                    table[s, have:need] = pages[have:need]
+                else:
+                    table[s, :need] = pages[:need]
+                    table[s, need:] = -1
+                self.row_pages[g][s] = need
+
+    def replay(self) -> torch.Tensor:
+        self.static.copy_(self.host, non_blocking=True)
         self.graph.replay()
         return self.logits
 
@@ -131,21 +183,23 @@ class ModelRunner:
     def step_graphed(self, chunks: list, started: float | None = None) -> torch.Tensor:
         """A decode-only step through a captured graph (captured on first use for this number
         of sequences and length bound)."""
-        width = -(-self.max_model_len // self.page_size)
-        packed = pack_step(chunks, self.manager, self.model.vocab_size, self.max_model_len,
-                           pinned=True, table_width=width)
         bound = 256
-        while bound < packed.max_kv_len:
+        longest = max(c.start for c in chunks) + 1
+        while bound < longest:
             bound *= 2
         key = (len(chunks), bound)
         graph = self.graphs.get(key)
         if graph is None:
+            width = -(-self.max_model_len // self.page_size)
+            packed = pack_step(chunks, self.manager, self.model.vocab_size, self.max_model_len,
+                               pinned=True, table_width=width)
             graph = self.graphs[key] = DecodeGraph(self, packed, bound)
+        graph.refill(chunks, self.manager, self.model.vocab_size, self.max_model_len)
         if started is not None:
             import time
 
             self.last_prepare_seconds = time.perf_counter() - started
-        return graph.replay(packed)
+        return graph.replay()
 
     @torch.inference_mode()
     def run(self, ctx: StepContext) -> torch.Tensor:

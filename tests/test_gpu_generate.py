@@ -172,3 +172,36 @@ def test_captured_decode_graphs_replay_like_eager_steps(dtype):
     # the same graphs again, after unrelated work in between
     assert generate(graphed_engine, prompts[:2], 20) == [e[:20] for e in eager[:2]]
     assert generate(graphed_engine, prompts, 40) == eager
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_a_graph_row_changes_its_owner(dtype):
+    """With two requests running at a time and five waiting in turn, the rows of the
+    two-sequence graph pass from request to request, and with few pages a preempted request
+    comes back under its own key with other pages: the graph's host copy of the block tables
+    has to follow.  The tokens are those of an engine that never captures."""
+    from mercury_amd import SamplingParams
+
+    prompts = [PROMPT[:40], OTHER[:30], PROMPT[:9], OTHER[:50], PROMPT[:25]]
+    lengths = [30, 12, 44, 7, 21]
+
+    def run(**kw):
+        eng = engine(dtype=dtype, max_running=2, **kw)
+        outs = {i: [] for i in range(len(prompts))}
+        for i, (p, n) in enumerate(zip(prompts, lengths)):
+            eng.submit(f"r{i}", list(p), n, outs[i].append, params=SamplingParams(ignore_eos=True))
+        eng._drain_commands()
+        while eng.sched.has_work():
+            eng.step()
+        assert eng.leaked_blocks() == 0
+        return {i: [e.token for e in ev if e.kind == "token"] for i, ev in outs.items()}, eng
+
+    eager, _ = run(use_graphs=False)
+    graphed, eng = run(use_graphs=True)
+    assert graphed == eager
+    assert any(key[0] == 2 for key in eng.runner.runner.graphs)
+    # 6 pages of 16 tokens hold two requests only until they have grown: the newer one is
+    # preempted and starts over
+    tight, eng = run(use_graphs=True, num_blocks=6, max_model_len=96)
+    assert tight == eager
+    assert eng.sched.stats["preemptions"] > 0

@@ -201,6 +201,7 @@ def test_which_skinny_projections_are_split():
     assert wants(8, 896, 4864)             # 8.7 MB behind 56 tiles of rows
     assert not wants(8, 896, 896)          # small: latency is the cost, not bandwidth
     assert not wants(8, 3584, 4096)        # 224 tiles of rows are workgroups enough
+    assert wants(64, 3584, 4096)           # many rows of x: re-reading them costs more than slices
     assert not wants(8, 896, 4868)         # K % 8 != 0: not for the matrix cores at all
 
 
