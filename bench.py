@@ -60,6 +60,8 @@ def parse_args(argv=None):
     p.add_argument("--dtype", default="bfloat16", choices=("bfloat16", "float32"))
     p.add_argument("--context", type=int, default=CONTEXT)
     p.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 runs")
+    p.add_argument("--no-lookahead", action="store_true",
+                   help="never start a decode step before the previous one's tokens are read")
     p.add_argument("--seed", type=int, default=0)
     return p.parse_args(argv)
 
@@ -76,7 +78,8 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
 
 
 class Bench:
-    def __init__(self, cfg: dict, dtype: str, max_batch: int, context: int, seed: int):
+    def __init__(self, cfg: dict, dtype: str, max_batch: int, context: int, seed: int,
+                 lookahead: bool = True):
         import torch
 
         from mercury_amd.cache import CacheManager, PageHasher
@@ -97,10 +100,11 @@ class Bench:
         pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + PREFILL_TOKENS // BLOCK_SIZE + 8
         self.engine_cfg = EngineConfig(
             model="random", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
-            max_running=max_batch + 1, prefill_budget=8192, max_model_len=context + 128, seed=seed)
+            max_running=max_batch + 1, prefill_budget=8192, max_model_len=context + 128, seed=seed,
+            lookahead=lookahead)
         manager = CacheManager(model.cache_slots, pages, BLOCK_SIZE, max_batch + 1, False)
         runner = ModelRunner(model, manager, torch_dtype, device, context + 128)
-        self.engine = Engine(self.engine_cfg, executor=GpuExecutor(runner, Sampler(seed)),
+        self.engine = Engine(self.engine_cfg, executor=GpuExecutor(runner, Sampler(seed), lookahead=self.engine_cfg.lookahead),
                              manager=manager, eos_token_ids=())
         self.model, self.runner, self.manager = model, runner, manager
         self.rng = torch.Generator().manual_seed(seed)
@@ -120,13 +124,17 @@ class Bench:
         the last timed step."""
         from mercury_amd import SamplingParams
 
-        prompt_len = context - steps - warmup
+        # Prompts enter a few per step (the token budget), so the first admitted request is
+        # some tokens ahead of the last; the untimed steps are counted so that the longest
+        # request reaches `context` exactly at the last timed step.
+        stagger = -(-batch * context // self.engine_cfg.prefill_budget) + 1
+        prompt_len = context - steps - warmup - stagger
         rids = []
         for _ in range(batch):
             rid = f"bench-{self.counter}"
             self.counter += 1
-            self.engine.submit(rid, self.tokens(prompt_len), steps + warmup + batch + 8, lambda e: None,
-                               params=SamplingParams(ignore_eos=True))
+            self.engine.submit(rid, self.tokens(prompt_len), steps + warmup + stagger + batch + 8,
+                               lambda e: None, params=SamplingParams(ignore_eos=True))
             rids.append(rid)
         self.engine._drain_commands()
         t0 = time.time()
@@ -135,7 +143,10 @@ class Bench:
         self.sync()
         fill_s = time.time() - t0
         assert len(self.engine.sched.running) == batch
-        for _ in range(warmup):
+        longest = max(r.num_computed for r in self.engine.sched.running)
+        untimed = context - steps - longest
+        assert untimed >= warmup, (untimed, warmup)
+        for _ in range(untimed):
             self.engine.step()
         self.sync()
         start = time.perf_counter()
@@ -144,6 +155,7 @@ class Bench:
             assert record.num_decode == batch and record.num_prefill == 0
         self.sync()
         elapsed = time.perf_counter() - start
+        assert max(r.num_computed for r in self.engine.sched.running) == context
         kv_tokens = sum(r.num_computed for r in self.engine.sched.running)
         kv_bytes = kv_tokens * self.runner.kv_bytes_per_token()
         for rid in rids:
@@ -152,7 +164,7 @@ class Bench:
         assert self.engine.leaked_blocks() == 0
         ms = 1e3 * elapsed / steps
         return {"tok_s": batch * steps / elapsed, "ms": ms, "fill_s": fill_s,
-                "bytes": self.model.decode_weight_bytes() + kv_bytes}
+                "prompt_len": prompt_len, "bytes": self.model.decode_weight_bytes() + kv_bytes}
 
     def prefill(self, tokens: int, repeats: int = 5) -> dict:
         from mercury_amd import SamplingParams
@@ -185,7 +197,7 @@ def main(argv=None) -> int:
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
     max_batch = args.batch if args.no_points else max(args.batch, 64)
-    bench = Bench(cfg, args.dtype, max_batch, args.context, args.seed)
+    bench = Bench(cfg, args.dtype, max_batch, args.context, args.seed, not args.no_lookahead)
 
     main_run = bench.decode(args.batch, args.context, args.steps, args.warmup)
     print(f"[bench] decode b{args.batch}: {main_run['ms']:.3f} ms/step "
@@ -222,7 +234,7 @@ def main(argv=None) -> int:
             "head_dim": cfg["head_dim"], "intermediate": cfg["intermediate_size"],
             "vocab": cfg["vocab_size"], "tied_embeddings": cfg["tie_word_embeddings"],
             "global_batch": args.batch, "seq_len": args.context,
-            "prompt_len": args.context - args.steps - args.warmup, "block_size": BLOCK_SIZE,
+            "prompt_len": main_run["prompt_len"], "block_size": BLOCK_SIZE,
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
         },
         "prefill": {"value": round(pre["tok_s"], 1), "tokens": PREFILL_TOKENS,

@@ -60,6 +60,9 @@ class EngineConfig:
     max_step_records: int = 500_000
     debug_invariants: bool = False
     use_graphs: bool = True
+    # Start a decode step before the previous one's tokens have been read, when the scheduler
+    # expects the same requests to go on (needs use_graphs).
+    lookahead: bool = True
 
     extra: dict = field(default_factory=dict)
 

@@ -107,7 +107,8 @@ class Engine:
                                has_state)
         runner = ModelRunner(model, manager, cfg.torch_dtype, device, cfg.max_model_len,
                              use_graphs=cfg.use_graphs)
-        return GpuExecutor(runner, Sampler(cfg.seed)), manager, model.eos_token_ids
+        return (GpuExecutor(runner, Sampler(cfg.seed), lookahead=cfg.lookahead), manager,
+                model.eos_token_ids)
 
     # ---------------------------------------------------------------- lifecycle
 

@@ -46,6 +46,7 @@ class DecodeGraph:
         self.ids, self.positions, _seq, _cu, self.kv_len, self.slots, _rows = views[:7]
         n = packed.num_seqs
         self.tables = [views[7 + g].reshape(n, w) for g, w in enumerate(packed.widths)]
+        self.copied = None                                 # the last copy of `host` to the device
         self.row_record = [None] * n                       # whose pages a table row mirrors
         self.row_pages = [[0] * n for _ in packed.widths]  # and how many of them
         self.appendable = [g.spec.window is None for g in runner.manager.groups]
@@ -60,14 +61,18 @@ class DecodeGraph:
         with torch.cuda.graph(self.graph):
             self.logits = runner.model.forward(self.ctx, runner.caches, runner.states)
 
-    def refill(self, chunks: list, manager, vocab_size: int, max_positions: int) -> None:
-        """Write this step's numbers into the host copy.  The previous replay's copy to the
-        device has finished: its logits have been read since."""
+    def refill(self, chunks: list, manager, vocab_size: int, max_positions: int,
+               ids_on_device: bool = False) -> None:
+        """Write this step's numbers into the host copy, once the previous replay's copy to
+        the device has finished.  With `ids_on_device` the token ids are not the chunks'."""
+        if self.copied is not None:
+            self.copied.synchronize()
         n = len(chunks)
-        self.ids[:] = [c.tokens[0] for c in chunks]
+        if not ids_on_device:
+            self.ids[:] = [c.tokens[0] for c in chunks]
+            if self.ids.min() < 0 or self.ids.max() >= vocab_size:
+                raise BatchError(f"token id outside [0, {vocab_size})")
         self.positions[:] = [c.start for c in chunks]
-        if self.ids.min() < 0 or self.ids.max() >= vocab_size:
-            raise BatchError(f"token id outside [0, {vocab_size})")
         if self.positions.min() < 0 or self.positions.max() >= max_positions:
             raise BatchError(f"a sequence would pass the limit of {max_positions} tokens")
         np.add(self.positions, 1, out=self.kv_len)
@@ -96,8 +101,15 @@ class DecodeGraph:
                     table[s, need:] = -1
                 self.row_pages[g][s] = need
 
-    def replay(self) -> torch.Tensor:
+    def replay(self, ids: torch.Tensor | None = None) -> torch.Tensor:
+        """Copy the step to the device and run the graph; `ids` (int32 on the device, one per
+        sequence) replace the token ids of the host copy."""
         self.static.copy_(self.host, non_blocking=True)
+        if self.copied is None:
+            self.copied = torch.cuda.Event()
+        self.copied.record()
+        if ids is not None:
+            self.ctx.token_ids.copy_(ids)
         self.graph.replay()
         return self.logits
 
@@ -175,31 +187,43 @@ class ModelRunner:
         self.last_prepare_seconds = time.perf_counter() - started
         return self.run(ctx)
 
+    def captured(self, chunks: list) -> bool:
+        """Whether `step_graphed` would replay a graph it already has for these chunks."""
+        return self._graphable(chunks) and self._graph_key(chunks) in self.graphs
+
+    @staticmethod
+    def _graph_key(chunks: list) -> tuple:
+        bound = 256
+        longest = max(c.start for c in chunks) + 1
+        while bound < longest:
+            bound *= 2
+        return len(chunks), bound
+
     def _graphable(self, chunks: list) -> bool:
         return (self.use_graphs and len(chunks) <= self.max_graph_batch
                 and all(len(c.tokens) == 1 and c.want == [0] and c.start > 0 for c in chunks))
 
     @torch.inference_mode()
-    def step_graphed(self, chunks: list, started: float | None = None) -> torch.Tensor:
+    def step_graphed(self, chunks: list, started: float | None = None,
+                     ids: torch.Tensor | None = None) -> torch.Tensor:
         """A decode-only step through a captured graph (captured on first use for this number
-        of sequences and length bound)."""
-        bound = 256
-        longest = max(c.start for c in chunks) + 1
-        while bound < longest:
-            bound *= 2
-        key = (len(chunks), bound)
+        of sequences and length bound).  `ids`: the token ids, on the device, when the host
+        does not know them yet."""
+        key = self._graph_key(chunks)
+        bound = key[1]
         graph = self.graphs.get(key)
         if graph is None:
             width = -(-self.max_model_len // self.page_size)
             packed = pack_step(chunks, self.manager, self.model.vocab_size, self.max_model_len,
                                pinned=True, table_width=width)
             graph = self.graphs[key] = DecodeGraph(self, packed, bound)
-        graph.refill(chunks, self.manager, self.model.vocab_size, self.max_model_len)
+        graph.refill(chunks, self.manager, self.model.vocab_size, self.max_model_len,
+                     ids_on_device=ids is not None)
         if started is not None:
             import time
 
             self.last_prepare_seconds = time.perf_counter() - started
-        return graph.replay()
+        return graph.replay(ids)
 
     @torch.inference_mode()
     def run(self, ctx: StepContext) -> torch.Tensor:

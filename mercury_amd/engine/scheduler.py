@@ -39,6 +39,11 @@ class Plan:
     preempted: list = field(default_factory=list)
     admitted: list = field(default_factory=list)
     sched_seconds: float = 0.0
+    # The next plan is expected to be this one a token further: every request decodes and
+    # none reaches its length limit with this step's token, and nobody waits for a place that
+    # is free.  (A stop token may still prove it wrong.)  An executor may use it to start the
+    # next step's work early.
+    steady: bool = False
 
     def __bool__(self) -> bool:
         return bool(self.work)
@@ -195,6 +200,11 @@ class Scheduler:
             self.running.extend(plan.admitted)
             self.stats["admissions"] += len(plan.admitted)
 
+        plan.steady = (bool(plan.work) and not plan.preempted
+                       and (not self.waiting or len(self.running) >= self.max_running)
+                       and all(w.count == 1 and w.emits and w.start >= w.request.prompt_len
+                               and len(w.request.out) + 1 < w.request.max_tokens
+                               for w in plan.work))
         plan.sched_seconds = time.perf_counter() - t0
         self.stats["steps"] += 1
         self.stats["sched_seconds"] += plan.sched_seconds

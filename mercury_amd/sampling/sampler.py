@@ -31,15 +31,23 @@ class Sampler:
     def sample(self, logits: torch.Tensor, requests: list) -> list:
         """One token per row of float32 logits [n, V]; row i belongs to requests[i], whose
         next output index is len(request.out)."""
+        if not requests:
+            if logits.shape[0]:
+                raise ValueError(f"{logits.shape[0]} rows of logits for no requests")
+            return []
+        return self.launch(logits, requests).cpu().tolist()
+
+    def launch(self, logits: torch.Tensor, requests: list, ahead: int = 0) -> torch.Tensor:
+        """The same as int32 tokens [n] left on the device, without waiting for them.  `ahead`
+        is how many tokens each request will have got before this one that it has not got
+        yet (for a step started before the previous one's tokens were read)."""
         if logits.shape[0] != len(requests):
             raise ValueError(f"{logits.shape[0]} rows of logits for {len(requests)} requests")
-        if not requests:
-            return []
         if all(r.params.greedy for r in requests):
-            return ops.argmax(logits).cpu().tolist()
+            return ops.argmax(logits)
         temps = [float(r.params.temperature) for r in requests]
         top_ps = [float(r.params.top_p) for r in requests]
-        us = [uniform_for(self.seed if r.params.seed is None else r.params.seed, r.rid, len(r.out))
-              for r in requests]
+        us = [uniform_for(self.seed if r.params.seed is None else r.params.seed, r.rid,
+                          len(r.out) + ahead) for r in requests]
         packed = torch.tensor([temps, top_ps, us], dtype=torch.float32).to(logits.device)
-        return ops.sample(logits, packed[0], packed[1], packed[2]).cpu().tolist()
+        return ops.sample(logits, packed[0], packed[1], packed[2])

@@ -205,3 +205,68 @@ def test_a_graph_row_changes_its_owner(dtype):
     tight, eng = run(use_graphs=True, num_blocks=6, max_model_len=96)
     assert tight == eager
     assert eng.sched.stats["preemptions"] > 0
+
+
+def run_requests(eng, submissions, max_tokens, aborts=(), **params):
+    """Drive the engine by hand: `submissions` maps a step number to the prompts submitted
+    before it, `aborts` a step number to the request ids aborted before it."""
+    from mercury_amd import SamplingParams
+
+    outs, step, count = {}, 0, 0
+    while True:
+        for prompt in submissions.get(step, []):
+            rid = f"r{count}"
+            outs[rid] = []
+            eng.submit(rid, list(prompt), max_tokens, outs[rid].append,
+                       params=SamplingParams(**params))
+            count += 1
+        for rid in dict(aborts).get(step, []):
+            eng.abort(rid)
+        eng._drain_commands()
+        if not eng.sched.has_work() and step > max(submissions):
+            break
+        eng.step()
+        step += 1
+    assert eng.leaked_blocks() == 0
+    return {rid: [e.token for e in ev if e.kind == "token"] for rid, ev in outs.items()}
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_steps_started_ahead_give_the_same_tokens(dtype):
+    """A decode step launched before the previous one's tokens were read (the scheduler
+    expected the same requests to go on) yields what the step launched afterwards yields:
+    greedy and sampled, with requests that arrive, stop at a stop token, reach their length
+    or are aborted while a step runs ahead."""
+    prompts = [PROMPT, OTHER, PROMPT[:33], OTHER[:7]]
+    plain_run = run_requests(engine(dtype=dtype, lookahead=False), {0: prompts}, 40, ignore_eos=True)
+    eng = engine(dtype=dtype, lookahead=True)
+    assert run_requests(eng, {0: prompts}, 40, ignore_eos=True) == plain_run
+    stats = eng.runner.stats
+    assert stats["ahead_used"] >= 30 and stats["ahead_started"] - stats["ahead_used"] <= 2
+
+    sampling = dict(temperature=0.8, top_p=0.9)
+    sampled = run_requests(engine(dtype=dtype, lookahead=False), {0: prompts}, 24, ignore_eos=True,
+                           **sampling)
+    assert run_requests(engine(dtype=dtype, lookahead=True), {0: prompts}, 24, ignore_eos=True,
+                        **sampling) == sampled
+
+    # a token some request first draws a few steps into decoding becomes the stop token: the
+    # request ends there, the others go on, and the step that ran ahead with it is dropped
+    stop = next(tok for toks in sampled.values() for i, tok in enumerate(toks)
+                if i >= 3 and tok not in toks[:i])
+    cut = {rid: (toks[:toks.index(stop) + 1] if stop in toks else toks) for rid, toks in sampled.items()}
+    from mercury_amd import Engine, EngineConfig
+    for look in (False, True):
+        eng = Engine(EngineConfig(model=str(helpers.model_folder("A")), dtype=dtype, num_blocks=64,
+                                  max_model_len=512, lookahead=look), eos_token_ids=[stop])
+        assert run_requests(eng, {0: prompts}, 24, **sampling) == cut
+    assert eng.runner.stats["ahead_started"] > eng.runner.stats["ahead_used"] > 0
+
+    # arrivals and an abort in the middle of decoding
+    late = {0: prompts[:2], 9: prompts[2:3], 15: prompts[3:]}
+    aborts = {12: ["r0"]}
+    want = run_requests(engine(dtype=dtype, lookahead=False), late, 30, aborts, ignore_eos=True)
+    eng = engine(dtype=dtype, lookahead=True)
+    assert run_requests(eng, late, 30, aborts, ignore_eos=True) == want
+    assert len(want["r0"]) < 30 and want["r1"] == plain_run["r1"][:30]
+    assert eng.runner.stats["ahead_used"] > 0

@@ -239,3 +239,27 @@ def test_prefix_aware_order_wins_under_pressure_and_the_deadline_bounds_the_wait
     assert lpm.hit_rate() > fcfs.hit_rate() + 0.05
     assert fcfs.hit_rate() < aged.hit_rate() < lpm.hit_rate()
     assert lpm.stats["evictions"] < fcfs.stats["evictions"]
+
+
+def test_a_plan_says_when_the_next_one_will_be_the_same_a_token_further():
+    """`steady`: every request decodes and none reaches its length with this step's token, and
+    nobody waits for a place that is free."""
+    _, sched = make(64, max_running=2)
+    sched.add(request("a", [1] * 20, 0.0, max_tokens=4))
+    sched.add(request("b", [2] * 5, 1.0, max_tokens=6))
+    plan = sched.schedule(2.0)
+    assert not plan.steady                       # prompts
+    finish_step(plan)
+    plan = sched.schedule(3.0)
+    assert rids(plan.decode) == ["a", "b"] and plan.steady
+    sched.add(request("c", [3] * 5, 3.5))
+    finish_step(plan)
+    plan = sched.schedule(4.0)
+    assert plan.steady                           # c waits, but no place is free
+    sched.max_running = 3
+    finish_step(plan)
+    plan = sched.schedule(5.0)
+    assert rids(plan.admitted) == ["c"] and not plan.steady
+    sched.abort("c")
+    # a has 3 of its 4 tokens: this step's token is its last
+    assert len(sched.running[0].out) == 3 and not sched.schedule(6.0).steady
