@@ -326,6 +326,202 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p
   }
 }
 
+// ---------------------------------------------------------------------- prompts through LDS
+//
+// With many rows per sequence (prompt portions), the four wavefronts of a workgroup take four
+// consecutive stretches of 16 * RT rows of one sequence and one kv head and walk the same
+// blocks of keys together: every block is fetched from the cache once per workgroup, each
+// thread bringing 16 or 32 bytes of the keys and as much of the values, parked in registers
+// for two iterations and then placed in one of two LDS buffers, from which every wavefront
+// reads its operands.  Loads are so two blocks ahead of their use at a quarter of the
+// registers a wavefront fetching for itself would need (deeper did not pay: the loop is bound
+// by the instructions it issues, not by the loads), and the cache is read once, not four
+// times.
+//
+// LDS layout of a block (32 keys): keys [32][D] and values [D][32], the 16-byte chunks of
+// each row permuted so that the rows one operand read touches fall on different banks:
+//   keys    D = 64: rows of 128 bytes, chunk c of key k at c ^ ((k >> 1) & 7)
+//           D a multiple of 128: chunk c of key k at (c & ~15) | ((c ^ k) & 15)
+//           else: at (c & ~7) | ((c ^ k) & 7)
+//   values  rows of 64 bytes (32 keys), 16-byte slot s of dim j at s ^ ((j >> 2) & 3)
+
+template <int D>
+__device__ __forceinline__ int staged_key_offset(int key, int chunk) {  // in 16-byte units
+  if (D == 64) return key * 8 + ((chunk ^ (key >> 1)) & 7);
+  if (D % 128 == 0) return key * (D / 8) + ((chunk & ~15) | ((chunk ^ key) & 15));
+  return key * (D / 8) + ((chunk & ~7) | ((chunk ^ key) & 7));
+}
+
+__device__ __forceinline__ int staged_value_offset(int dim, int slot) {  // in 16-byte units
+  return dim * 4 + ((slot ^ (dim >> 2)) & 3);
+}
+
+// What one thread carries of a block between its global loads and its LDS stores.
+template <int D>
+struct StagedRegs {
+  uint4 k[D / 64], v[D / 64];
+};
+
+template <int D>
+__device__ __forceinline__ StagedRegs<D> staged_fetch(const AttnParams& p, TableWindow& tw, int b,
+                                                      int b_end, int kmin, int kmax, int kvh,
+                                                      int lane) {
+  StagedRegs<D> regs;
+  const int ps = 1 << p.page_shift;
+  const int tid = threadIdx.x;
+  int page[2], off[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int kh = (b << 5) + h * 16;
+    const bool live = b < b_end && kh <= kmax && kh + 15 >= kmin;  // uniform
+    page[h] = live ? tw.page(kh >> p.page_shift, lane) : 0;
+    off[h] = kh & (ps - 1);
+  }
+  const size_t head_elems = (size_t)ps * D;
+#pragma unroll
+  for (int i = 0; i < D / 64; ++i) {
+    // keys: 16-byte chunk `chunk` of key `key` of the block
+    const int idx = tid + i * 256, key = idx / (D / 8), chunk = idx % (D / 8);
+    const bool h = key >= 16;      // per lane: selected, not indexed
+    const bf16_t* kp = p.k_cache + ((size_t)(h ? page[1] : page[0]) * p.n_kv + kvh) * head_elems +
+                       (size_t)((h ? off[1] : off[0]) + (key & 15)) * D + chunk * 8;
+    regs.k[i] = *(const uint4*)kp;
+    // values: 8 keys (slot `slot` of 4) of dim `dim`
+    const int dim = idx >> 2, slot = idx & 3;
+    const bool hv = slot >= 2;
+    const bf16_t* vp = p.v_cache + ((size_t)(hv ? page[1] : page[0]) * p.n_kv + kvh) * head_elems +
+                       (size_t)dim * ps + (hv ? off[1] : off[0]) + (slot & 1) * 8;
+    regs.v[i] = *(const uint4*)vp;
+  }
+  return regs;
+}
+
+template <int D>
+__device__ __forceinline__ void staged_store(const StagedRegs<D>& regs, uint4* lds_k, uint4* lds_v) {
+  const int tid = threadIdx.x;
+#pragma unroll
+  for (int i = 0; i < D / 64; ++i) {
+    const int idx = tid + i * 256;
+    lds_k[staged_key_offset<D>(idx / (D / 8), idx % (D / 8))] = regs.k[i];
+    lds_v[staged_value_offset(idx >> 2, idx & 3)] = regs.v[i];
+  }
+}
+
+// The block's operands of this lane, out of LDS (as load_key_block takes them from the cache).
+template <int D>
+__device__ __forceinline__ void staged_operands(KeyBlock<D>& blk, const uint4* lds_k,
+                                                const uint4* lds_v, int b, int kmin, int kmax,
+                                                int lane) {
+  const int r = lane & 15, g4 = lane >> 4;
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int kh = (b << 5) + h * 16;
+    blk.live[h] = kh <= kmax && kh + 15 >= kmin;
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+      blk.kf[h][c].u = lds_k[staged_key_offset<D>(h * 16 + r, c * 4 + g4)];
+  }
+#pragma unroll
+  for (int dt = 0; dt < D / 16; ++dt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+      // keys h*16 + g4*4 .. + 4 of dim dt*16 + r: half of the 16-byte slot h*2 + g4/2
+      const int dim = dt * 16 + r;
+      const uint2* slot = (const uint2*)(lds_v + staged_value_offset(dim, h * 2 + (g4 >> 1)));
+      blk.vf[dt].u2[h] = slot[g4 & 1];
+    }
+}
+
+template <int D, int RT>
+__global__ __launch_bounds__(64 * ATTN_WAVES) void attn_staged_kernel(AttnParams p) {
+  static_assert(D % 64 == 0, "256 threads bring whole 16-byte chunks of 32 keys");
+  __shared__ uint4 lds_k[2][32 * D / 8];
+  __shared__ uint4 lds_v[2][32 * D / 8];
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int tile = p.num_tiles - 1 - (int)blockIdx.x;   // the longest work first
+  const int kvh = blockIdx.y;
+  const int seq = p.tile_seq[tile];
+  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  const int pos0 = p.kv_len[seq] - q_len;
+  const int G = p.group;
+  const int rows_total = q_len * G;
+  const int r = lane & 15, g4 = lane >> 4;
+  constexpr int WAVE_ROWS = 16 * RT;
+  const int wg_row0 = p.tile_row0[tile];
+  const int row0 = wg_row0 + wave * WAVE_ROWS;          // this wavefront's rows
+  const bool wave_has_rows = row0 < rows_total;
+
+  TileState<D, RT> st;
+  int tok[RT], head[RT];
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    const int flat = row0 + t * 16 + r;
+    st.row_ok[t] = flat < rows_total;
+    tok[t] = st.row_ok[t] ? flat / G : 0;
+    head[t] = kvh * G + (st.row_ok[t] ? flat % G : 0);
+    st.pos[t] = pos0 + tok[t];
+    st.lo[t] = p.window > 0 ? max(0, st.pos[t] - p.window + 1) : 0;
+    st.m[t] = -INFINITY;
+    st.lsum[t] = 0.f;
+    const bf16_t* qrow = p.q + (size_t)(q0 + tok[t]) * p.q_stride + head[t] * D + g4 * 8;
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+      st.qf[t][c].u = st.row_ok[t] ? *(const uint4*)(qrow + c * 32) : make_uint4(0, 0, 0, 0);
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt) st.acc[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  // Keys the workgroup's rows can see, and this wavefront's own share of them.
+  const int wg_last = min(wg_row0 + ATTN_WAVES * WAVE_ROWS - 1, rows_total - 1);
+  const int wg_kmax = pos0 + wg_last / G;
+  const int wg_kmin = p.window > 0 ? max(0, pos0 + wg_row0 / G - p.window + 1) : 0;
+  const int b0 = wg_kmin >> 5, b1 = (wg_kmax >> 5) + 1;
+  const int last_flat = min(row0 + WAVE_ROWS - 1, rows_total - 1);
+  const int kmax = wave_has_rows ? pos0 + last_flat / G : -1;
+  const int kmin = p.window > 0 ? max(0, pos0 + row0 / G - p.window + 1) : 0;
+  const int see_upto = pos0 + row0 / G;
+  const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
+  const float c = p.scale * 1.44269504088896340736f;
+
+  TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
+  StagedRegs<D> ra = staged_fetch<D>(p, tw, b0, b1, wg_kmin, wg_kmax, kvh, lane);
+  StagedRegs<D> rb = staged_fetch<D>(p, tw, b0 + 1, b1, wg_kmin, wg_kmax, kvh, lane);
+  KeyBlock<D> blk;
+  // One block: park what was fetched two iterations ago in LDS, ask for the block two ahead,
+  // and, once every wavefront's share is in place, use the block.  Blocks past this
+  // wavefront's last key or before its first are the others' business.
+#define STAGED_ITERATION(regs, b, buf)                                                  \
+  do {                                                                                  \
+    staged_store<D>(regs, lds_k[buf], lds_v[buf]);                                      \
+    regs = staged_fetch<D>(p, tw, (b) + 2, b1, wg_kmin, wg_kmax, kvh, lane);            \
+    __syncthreads();                                                                    \
+    if (((b) << 5) <= kmax && ((b) << 5) + 31 >= kmin) {                                \
+      staged_operands<D>(blk, lds_k[buf], lds_v[buf], (b), kmin, kmax, lane);           \
+      attend<D, RT>(st, blk, (b) << 5, c, g4, see_upto, see_from);                      \
+    }                                                                                   \
+  } while (0)
+  for (int b = b0; b < b1; b += 2) {
+    STAGED_ITERATION(ra, b, 0);
+    if (b + 1 < b1) STAGED_ITERATION(rb, b + 1, 1);
+  }
+#undef STAGED_ITERATION
+
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    if (!st.row_ok[t]) continue;
+    float l = st.lsum[t];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+    const float inv = 1.f / l;
+    bf16_t* dst = p.out + (size_t)(q0 + tok[t]) * p.out_stride + head[t] * D + g4 * 4;
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt)
+      *(uint2*)(dst + dt * 16) =
+          make_uint2(pack_bf16x2(st.acc[t][dt][0] * inv, st.acc[t][dt][1] * inv),
+                     pack_bf16x2(st.acc[t][dt][2] * inv, st.acc[t][dt][3] * inv));
+  }
+}
+
 // Merge the key splits of one (tile, kv head, row) per workgroup: the maximum of the running
 // maxima, then the sums and the partial results rescaled to it.  Thread (g, dim) adds the
 // splits g, g + 4, ... of its dim, four loads in flight at a time; the four groups are then
@@ -381,6 +577,17 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
 }
 
 template <int D>
+static void launch_staged(const AttnParams& p, int rows_per_tile, hipStream_t stream) {
+  if constexpr (D == 64 || D == 128) {   // wider heads do not fit the register file
+    dim3 grid(p.num_tiles, p.n_kv);
+    if (rows_per_tile == 16)
+      attn_staged_kernel<D, 1><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
+    else
+      attn_staged_kernel<D, 2><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
+  }
+}
+
+template <int D>
 static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stream) {
   dim3 grid((p.num_tiles + ATTN_WAVES - 1) / ATTN_WAVES, p.n_kv, p.num_splits);
   const int threads = 64 * ATTN_WAVES;
@@ -403,6 +610,12 @@ extern "C" int mk_attention_mfma_max_rows(int head_dim) {
   return head_dim <= 64 ? 64 : (head_dim <= 128 ? 32 : 16);
 }
 
+// Whether the kernel that stages keys and values in LDS (workgroups of 4 * rows_per_tile rows
+// of one sequence) takes this head size and tile height.
+extern "C" int mk_attention_mfma_staged(int head_dim, int rows_per_tile) {
+  return (head_dim == 64 || head_dim == 128) && (rows_per_tile == 16 || rows_per_tile == 32);
+}
+
 extern "C" int mk_attention_mfma_supported(int head_dim, int page_size) {
   const bool d_ok = head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 ||
                     head_dim == 192 || head_dim == 256;
@@ -414,7 +627,7 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
                                  const int* tile_row0, int num_tiles, const int* cu_q,
                                  const int* kv_len, const int* block_table, int table_stride,
                                  int page_size, int n_q, int n_kv, int d, float scale, int window,
-                                 int rows_per_tile, int num_splits, int split_blocks,
+                                 int rows_per_tile, int staged, int num_splits, int split_blocks,
                                  float* part_o, float* part_ml, hipStream_t stream) {
   MK_REQUIRE(num_tiles >= 0 && n_q > 0 && n_kv > 0, "attention: bad sizes");
   MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
@@ -433,6 +646,9 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   MK_REQUIRE(rows_per_tile <= mk_attention_mfma_max_rows(d),
              "attention: %d rows per tile are too many for head size %d", rows_per_tile, d);
   MK_REQUIRE(split_blocks >= 0, "attention: negative split size");
+  MK_REQUIRE(!staged || (num_splits == 1 && mk_attention_mfma_staged(d, rows_per_tile)),
+             "attention: staging in LDS takes unsplit keys, head sizes 64 and 128 and 16 or 32 "
+             "rows per wavefront");
   if (num_tiles == 0) return 0;
   AttnParams p;
   p.q = (const bf16_t*)q;
@@ -459,12 +675,12 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   p.split_blocks = split_blocks;
   p.tile_rows = rows_per_tile;
   switch (d) {
-    case 32: launch_attn<32>(p, rows_per_tile, stream); break;
-    case 64: launch_attn<64>(p, rows_per_tile, stream); break;
-    case 96: launch_attn<96>(p, rows_per_tile, stream); break;
-    case 128: launch_attn<128>(p, rows_per_tile, stream); break;
-    case 192: launch_attn<192>(p, rows_per_tile, stream); break;
-    case 256: launch_attn<256>(p, rows_per_tile, stream); break;
+    case 32: staged ? launch_staged<32>(p, rows_per_tile, stream) : launch_attn<32>(p, rows_per_tile, stream); break;
+    case 64: staged ? launch_staged<64>(p, rows_per_tile, stream) : launch_attn<64>(p, rows_per_tile, stream); break;
+    case 96: staged ? launch_staged<96>(p, rows_per_tile, stream) : launch_attn<96>(p, rows_per_tile, stream); break;
+    case 128: staged ? launch_staged<128>(p, rows_per_tile, stream) : launch_attn<128>(p, rows_per_tile, stream); break;
+    case 192: staged ? launch_staged<192>(p, rows_per_tile, stream) : launch_attn<192>(p, rows_per_tile, stream); break;
+    case 256: staged ? launch_staged<256>(p, rows_per_tile, stream) : launch_attn<256>(p, rows_per_tile, stream); break;
   }
   MK_LAUNCH_CHECK("attention_mfma");
   return 0;

@@ -468,8 +468,8 @@ enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3 };
 
 // One workgroup of 4 wavefronts (WM x WN) computes a BM x BN tile of y; K advances TK per
 // stage through two LDS buffers, the next stage's global loads in flight during the current
-// stage's products.  Rows of a tile lie in LDS with a stride of TK + 8 elements, which keeps
-// 16-byte reads of 16 consecutive rows on distinct banks.
+// stage's products.  The 16-byte chunks of a tile row are permuted in LDS (or the row padded)
+// so that operand reads of 16 rows and staging writes of 2 rows hit distinct banks.
 // EPI_GATED: W is [gate rows | up rows] of N each; a tile holds BN / 2 gate rows and the BN / 2
 // matching up rows, every wavefront spans the tile's whole width (WN = 1), and the epilogue
 // writes act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
@@ -481,7 +481,15 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
                                                          int K, int ldo) {
   static_assert(WM * WN == 4, "four wavefronts");
   static_assert(EPI != EPI_GATED || WN == 1, "gating needs both halves in one wavefront");
-  constexpr int LD = TK + 8;
+  constexpr bool SWIZZLED = TK == 64;
+  constexpr int LD = SWIZZLED ? TK : TK + 8;
+  // Where the 8 elements from k (a multiple of 8) of a tile row lie in LDS.  Rows of 64
+  // elements are 128 bytes, half the banks; the 16-byte chunks of a row are permuted by the
+  // row pair's index, so that the 16 rows one operand read touches hit 16 different bank
+  // groups, as do the two rows a staging write fills.  Other widths pad the row instead.
+  auto lds_at = [](int row, int k) {
+    return SWIZZLED ? row * LD + ((((k >> 3) ^ (row >> 1)) & 7) << 3) : row * LD + k;
+  };
   constexpr int TM = BM / WM / 16, TN = BN / WN / 16;       // MFMA tiles per wavefront
   constexpr int CHUNKS_ROW = TK / 8;                        // 16-byte chunks per tile row
   constexpr int XCH = BM * CHUNKS_ROW / 256, WCH = BN * CHUNKS_ROW / 256;  // per thread
@@ -502,7 +510,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   for (int i = 0; i < XCH; ++i) {
     const int row = (tid + i * 256) / CHUNKS_ROW;
     xg[i] = x + (size_t)min(m0 + row, M - 1) * K + sk;
-    xo[i] = row * LD + sk;
+    xo[i] = lds_at(row, sk);
   }
 #pragma unroll
   for (int i = 0; i < WCH; ++i) {
@@ -511,7 +519,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     if (EPI == EPI_GATED)  // tile rows [0, BN/2) are gate rows, [BN/2, BN) the matching up rows
       wrow = row < BN / 2 ? min(n0 + row, N - 1) : N + min(n0 + row - BN / 2, N - 1);
     wg[i] = w + (size_t)wrow * K + sk;
-    wo[i] = row * LD + sk;
+    wo[i] = lds_at(row, sk);
   }
 
   f32x4 acc[TM][TN];
@@ -547,10 +555,10 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
       Frag a[TM], b[TN];
 #pragma unroll
       for (int t = 0; t < TM; ++t)
-        a[t].u = *(const uint4*)(&xs[buf][(wm + t * 16 + r) * LD + kk + g4 * 8]);
+        a[t].u = *(const uint4*)(&xs[buf][lds_at(wm + t * 16 + r, kk + g4 * 8)]);
 #pragma unroll
       for (int t = 0; t < TN; ++t)
-        b[t].u = *(const uint4*)(&ws[buf][(wn + t * 16 + r) * LD + kk + g4 * 8]);
+        b[t].u = *(const uint4*)(&ws[buf][lds_at(wn + t * 16 + r, kk + g4 * 8)]);
 #pragma unroll
       for (int ta = 0; ta < TM; ++ta)
 #pragma unroll
@@ -658,10 +666,12 @@ static void launch_tiled(int config, const void* x, const void* w, const void* b
   }
 }
 
-// 128 x 128 tiles when they give every compute unit two workgroups or more, else 64 x 64.
+// 128 x 128 tiles when they give every compute unit a workgroup, else 64 x 64 (measured:
+// 2048 x 3584 x 18944 runs a quarter faster in 448 large tiles than in 1792 small ones,
+// 2048 x 896 x 4864 a quarter slower in 112 large tiles than in 448 small ones).
 extern "C" int mk_linear_tiled_config(int M, int N, int K) {
   const long groups = (long)((M + 127) / 128) * ((N + 127) / 128);
-  return groups >= 512 ? 0 : 2;
+  return groups >= 256 ? 0 : 2;
 }
 
 // act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K].

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 2
+#define MK_ABI_VERSION 3
 
 #ifdef __cplusplus
 extern "C" {
@@ -115,13 +115,17 @@ int mk_attention_mfma_max_rows(int head_dim);
 // counts, kv_len [S] their lengths once this step's tokens are written.  With num_splits > 1
 // the keys are split, split_blocks blocks of 32 keys per split (0: each tile's own range in
 // num_splits equal parts), and part_o [tiles, n_kv, splits, rows_per_tile, d] /
-// part_ml [.., rows_per_tile, 2] hold the partial results.
+// part_ml [.., rows_per_tile, 2] hold the partial results.  staged != 0 (see
+// mk_attention_mfma_staged): the tiles are of 4 * rows_per_tile rows, one per workgroup, whose
+// wavefronts share the keys and values through LDS; for many rows per sequence, keys unsplit.
+int mk_attention_mfma_staged(int head_dim, int rows_per_tile);
 int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       const void* k_cache, const void* v_cache, const int* tile_seq,
                       const int* tile_row0, int num_tiles, const int* cu_q, const int* kv_len,
                       const int* block_table, int table_stride, int page_size, int n_q, int n_kv,
-                      int d, float scale, int window, int rows_per_tile, int num_splits,
-                      int split_blocks, float* part_o, float* part_ml, hipStream_t stream);
+                      int d, float scale, int window, int rows_per_tile, int staged,
+                      int num_splits, int split_blocks, float* part_o, float* part_ml,
+                      hipStream_t stream);
 
 // ---- library "core" again
 

@@ -408,7 +408,7 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
               step, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int, scale: float,
               window: int | None = None, out: torch.Tensor | None = None,
               kernel: str = "auto", tile_rows: int | None = None,
-              split_override: tuple | None = None) -> torch.Tensor:
+              split_override: tuple | None = None, staged: bool | None = None) -> torch.Tensor:
     """Causal grouped-query attention of every token of the step over its sequence's cached
     keys; q is read from rows of `q` with stride `q_stride` (the fused qkv buffer).
     `step` describes the batch (positions, token_seq, cu_q, kv_len, spans, tiles());
@@ -417,8 +417,9 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     kernel: "auto" takes the matrix-core kernel for bfloat16 where it covers the head and page
     size and the float32-arithmetic kernel otherwise; "generic" and "mfma" force one.
     tile_rows (16, 32 or 64) overrides how many rows a wavefront of the matrix-core kernel
-    takes, split_override = (splits, key blocks per split) how the keys are split; by
-    default the step's size decides both.
+    takes, split_override = (splits, key blocks per split) how the keys are split, staged
+    whether workgroups of four wavefronts share the keys and values of one sequence's rows
+    through LDS; by default the step's size decides all three.
     """
     _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out)
     _i32(block_table, "block_table")
@@ -458,10 +459,21 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
         rows *= 2
     if tile_rows is not None:
         rows = tile_rows
-    tile_seq, tile_row0, num_tiles = step.tiles(group, rows)
+    if staged is None:
+        # prompts: plenty of rows per sequence, enough workgroups of 64 of them; 16 rows a
+        # wavefront measured faster than 32 there
+        staged = (split_override is None and tile_rows is None
+                  and step.max_q_len * group >= 64
+                  and (total_rows // 64) * n_kv >= ATTENTION_STAGED_WORKGROUPS
+                  and bool(lib.mk_attention_mfma_staged(head_dim, 16)))
+        if staged:
+            rows = 16
+    tile_seq, tile_row0, num_tiles = step.tiles(group, rows * 4 if staged else rows)
     splits, split_blocks = 1, 0
     waves = max(1, num_tiles * n_kv)
-    if waves < ATTENTION_TARGET_WAVES and step.max_q_len == 1:
+    if staged:
+        pass
+    elif waves < ATTENTION_TARGET_WAVES and step.max_q_len == 1:
         # decoding: every sequence's own range in equal parts
         splits = max(1, min(blocks // ATTENTION_MIN_BLOCKS_PER_SPLIT or 1,
                             -(-ATTENTION_TARGET_WAVES // waves), 1024))
@@ -480,12 +492,13 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
         _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
         _ptr(tile_seq), _ptr(tile_row0), num_tiles, _ptr(step.cu_q), _ptr(step.kv_len),
         _ptr(block_table), block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
-        int(window or 0), rows, splits, split_blocks, _ptr(part_o), _ptr(part_ml), _stream()),
-        "attention")
+        int(window or 0), rows, int(staged), splits, split_blocks, _ptr(part_o), _ptr(part_ml),
+        _stream()), "attention")
     return out
 
 
 ATTENTION_TARGET_WAVES = 1024
+ATTENTION_STAGED_WORKGROUPS = 128
 ATTENTION_WIDE_TILE_WAVES = 400
 ATTENTION_PROMPT_SPLIT_BLOCKS = 1 << 30   # prompts are not split: the merge costs what the split gains
 ATTENTION_MIN_BLOCKS_PER_SPLIT = 2

@@ -473,7 +473,7 @@ def test_rotary_scores_depend_on_distance_only():
 
 def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens, q_lens, scale,
                   window=None, poison=None, kernel="auto", hide_before=None, tile_rows=None,
-                  split_override=None):
+                  split_override=None, staged=None):
     """q_h: list per sequence of [q_len, n_q, d] (the last q_len positions of the sequence);
     k_h/v_h: list per sequence of [seq_len, n_kv, d].  `hide_before`: per sequence, the number
     of leading pages to drop from the table (-1) and to poison, as after a window passed."""
@@ -502,7 +502,7 @@ def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens
     v_cache = v_cache.transpose(2, 3).contiguous()      # values lie transposed within a page
     out = ops().attention(q_flat, n_q * d, k_cache.to(DEV), v_cache.to(DEV), step, table.to(DEV),
                           n_q, n_kv, d, scale, window, kernel=kernel, tile_rows=tile_rows,
-                          split_override=split_override)
+                          split_override=split_override, staged=staged)
     return out.float().cpu().view(-1, n_q, d)
 
 
@@ -643,6 +643,43 @@ def test_attention_wide_tiles_for_prompts(tile_rows, d, n_q, n_kv, window, split
     want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-ql:]
                       for q, k, v, ql in zip(qs, ks, vs, q_lens)])
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
+
+
+@pytest.mark.parametrize("tile_rows,d,n_q,n_kv,page", [(16, 64, 14, 2, 16), (32, 64, 14, 2, 16),
+                                                       (16, 128, 8, 2, 32), (32, 128, 4, 4, 16),
+                                                       (32, 64, 3, 1, 64)])
+@pytest.mark.parametrize("window", [None, 40])
+def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, window):
+    """Workgroups whose four wavefronts share the keys and values of one sequence through LDS:
+    prompt portions of different length, one over a cached prefix, one ending inside a
+    workgroup's rows, beside a decoded token; pages scattered and poisoned outside."""
+    lens, q_lens = [333, 150, 77, 90], [333, 150, 33, 1]
+    qs, ks, vs = [], [], []
+    for i, s in enumerate(lens):
+        ks.append(rounded(rnd(s, n_kv, d, seed=600 + i), torch.bfloat16))
+        vs.append(rounded(rnd(s, n_kv, d, seed=610 + i), torch.bfloat16))
+        qs.append(rounded(rnd(s, n_q, d, seed=620 + i), torch.bfloat16))
+    per = [-(-s // page) for s in lens]
+    order = torch.randperm(sum(per) + 5, generator=torch.Generator().manual_seed(7)).tolist()
+    pages, at = [], 0
+    for n in per:
+        pages.append(order[at:at + n])
+        at += n
+    got = run_attention([q[-ql:] for q, ql in zip(qs, q_lens)], ks, vs, torch.bfloat16, pages, page,
+                        sum(per) + 5, lens, q_lens, d ** -0.5, window=window, poison=1e4,
+                        kernel="mfma", tile_rows=tile_rows, staged=True)
+    want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-ql:]
+                      for q, k, v, ql in zip(qs, ks, vs, q_lens)])
+    torch.testing.assert_close(got, want, **tol(torch.bfloat16))
+
+
+def test_attention_through_lds_is_refused_where_it_does_not_fit():
+    from mercury_amd.kernels.ops import KernelArgumentError
+
+    q = rounded(rnd(40, 2, 96, seed=1), torch.bfloat16)
+    with pytest.raises((KernelArgumentError, RuntimeError)):
+        run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
+                      kernel="mfma", staged=True)
 
 
 @pytest.mark.parametrize("batch,context", [(1, 4096), (3, 1500), (64, 300)])
