@@ -669,7 +669,9 @@ static void launch_tiled(int config, const void* x, const void* w, const void* b
 // 128 x 128 tiles when they give every compute unit a workgroup, else 64 x 64 (measured:
 // 2048 x 3584 x 18944 runs a quarter faster in 448 large tiles than in 1792 small ones,
 // 2048 x 896 x 4864 a quarter slower in 112 large tiles than in 448 small ones).
+// At most 64 rows: 64 x 128 tiles, no half of a tile idle.
 extern "C" int mk_linear_tiled_config(int M, int N, int K) {
+  if (M <= 64) return 1;
   const long groups = (long)((M + 127) / 128) * ((N + 127) / 128);
   return groups >= 256 ? 0 : 2;
 }

@@ -138,6 +138,9 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None,
 
 
 SKINNY_MAX_ROWS = 64
+WIDE_MATRIX_COLUMNS = 8192
+FUSED_QKV_MIN_WORKGROUPS = 128
+GATED_TILED_MIN_ROWS, GATED_TILED_MIN_WEIGHTS = 33, 16 << 20
 
 
 def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -187,7 +190,11 @@ def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     inter = w_gate_up.shape[0] // 2
     act = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
     lib = _lib.load("mfma")
-    fn = lib.mk_gated_skinny if m <= SKINNY_MAX_ROWS else lib.mk_gated_tiled
+    # 33 to 64 rows of a large matrix: the tiled kernel's shared x beats the skinny one's
+    # re-reads (measured at 18944 x 3584: 75 against 85 to 112 us)
+    skinny = m <= SKINNY_MAX_ROWS and not (m >= GATED_TILED_MIN_ROWS
+                                           and inter * k >= GATED_TILED_MIN_WEIGHTS)
+    fn = lib.mk_gated_skinny if skinny else lib.mk_gated_tiled
     _lib.check(lib, fn(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream()),
                "gated_projection")
     return act
@@ -232,7 +239,11 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
         if x.dtype != torch.bfloat16 or k % 8:
             raise KernelArgumentError("linear: the matrix-core kernels take bfloat16 with K % 8 == 0")
         lib = _lib.load("mfma")
-        if m <= SKINNY_MAX_ROWS and out_dtype == torch.float32 and bias is None and not accumulate:
+        # Few rows straight from HBM into the matrix cores; from 17 rows on, a wide matrix
+        # (the head over the vocabulary) is faster through LDS tiles, which read x once per
+        # 128 columns instead of once per 32.
+        if (m <= SKINNY_MAX_ROWS and out_dtype == torch.float32 and bias is None and not accumulate
+                and (m <= 16 or n < WIDE_MATRIX_COLUMNS)):
             _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, 1, _stream()),
                        "linear")
             return out
@@ -346,30 +357,42 @@ def _qkv_finish(parts, cos, sin, positions, token_seq, block_table, k_cache, v_c
     return q
 
 
-def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
-    """Whether `qkv_project` runs as one kernel: few bfloat16 rows, K a multiple of 8, heads a multiple of 32 wide and rotated over their whole width or not at
-    all, pages a power of two."""
+def _qkv_fusable(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
     return (_skinny_eligible(x, w) and head_dim % 32 == 0 and rotary_dim in (0, head_dim)
             and page_size > 0 and page_size & (page_size - 1) == 0)
+
+
+def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
+    """Whether `qkv_project` runs as one kernel by itself: few bfloat16 rows, K a multiple of
+    8, heads a multiple of 32 wide and rotated over their whole width or not at all, pages a
+    power of two; and, as that kernel has one workgroup per 32 rows of W with all of K, more
+    than 16 rows of x only where those workgroups are many."""
+    return (_qkv_fusable(x, w, head_dim, rotary_dim, page_size)
+            and (x.shape[0] <= 16 or w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS))
 
 
 def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor | None,
                 sin: torch.Tensor | None, positions: torch.Tensor, token_seq: torch.Tensor,
                 block_table: torch.Tensor, k_cache: torch.Tensor | None,
                 v_cache: torch.Tensor | None, n_q: int, n_kv: int, head_dim: int,
-                rotary_dim: int, write_kv: bool = True) -> torch.Tensor:
+                rotary_dim: int, write_kv: bool = True, fused: bool | None = None) -> torch.Tensor:
     """q, k, v = x W^T + bias for W = [q heads | k heads | v heads]; q and k rotated by their
     positions; k and v written to the paged cache (`write_kv`; otherwise W holds the query
     heads only).  Returns the rotated q [T, n_q d].
 
     Few rows take one kernel (projection, bias, rotation and cache write in its epilogue);
-    otherwise the projection is followed by `rope_kv_write`."""
+    otherwise the projection is followed by `rope_kv_write`.  `fused` forces one or the
+    other."""
     heads_kv = n_kv if write_kv else 0
     width = (n_q + 2 * heads_kv) * head_dim
     if w.shape[0] != width or w.shape[1] != x.shape[1]:
         raise KernelArgumentError(f"qkv_project: W {tuple(w.shape)} is not [{width}, {x.shape[1]}]")
     page_size = k_cache.shape[2] if write_kv and k_cache is not None else 1
-    if not fuses_qkv(x, w, head_dim, rotary_dim, page_size):
+    if fused is None:
+        fused = fuses_qkv(x, w, head_dim, rotary_dim, page_size)
+    elif fused and not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
+        raise KernelArgumentError("qkv_project: these operands cannot take the fused kernel")
+    if not fused:
         if wants_partials(x, w):
             return rope_kv_write(linear_partials(x, w), cos, sin, positions, token_seq,
                                  block_table, k_cache, v_cache, n_q, heads_kv, head_dim,
