@@ -37,7 +37,9 @@ __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *(const uint4*)p
 
 // ------------------------------------------------------------------------------ skinny
 
-#define SK_WAVES 4  // wavefronts of a workgroup; they share the rows and split the k-steps
+#define SK_WAVES 4  // wavefronts of a workgroup where the grid has many; they share the rows
+                    // and split the k-steps.  Kernels whose grid is one workgroup per compute
+                    // unit or fewer (SK_ACC, SK_QKV) take 8, for more bytes in flight per unit.
 
 // What a workgroup's rows of W are and what becomes of the result:
 //   SK_PARTIAL  rows n0.. of W; out[(slice * M + m) * N + n] float32, one slice of K each.
@@ -81,10 +83,10 @@ __device__ __forceinline__ float load_scalar(const void* p, int is_bf16, int i) 
 // current step's products; the wavefronts' results are added through LDS in wave order.
 // Product j of a step takes k = step*128 + j*32 + g4*8 .. + 8 from a lane, so that one load
 // instruction reads 64 contiguous bytes of each of its 16 rows.
-template <int MT, int NT, int EPI>
-__global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
+template <int MT, int NT, int EPI, int WAVES>
+__global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   static_assert((EPI != SK_GATED && EPI != SK_QKV) || NT == 2, "paired tiles");
-  __shared__ float red[SK_WAVES - 1][NT * MT * 4][64];
+  __shared__ float red[WAVES - 1][NT * MT * 4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g4 = lane >> 4;
   const int M = p.M, N = p.N, K = p.K;
   const int slice = blockIdx.y;
@@ -174,25 +176,25 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(SkinnyArgs p
   // tiles of x rows the second buffer would halve that, and one step at a time is faster.
   constexpr bool PIPELINED = MT <= 2;
   if constexpr (!PIPELINED) {
-    for (; step < step_end; step += SK_WAVES) {
+    for (; step < step_end; step += WAVES) {
       products(0);
-      if (step + SK_WAVES < step_end) {
-        load_w(0, step + SK_WAVES);
-        load_x(0, step + SK_WAVES);
+      if (step + WAVES < step_end) {
+        load_w(0, step + WAVES);
+        load_x(0, step + WAVES);
       }
     }
   }
-  for (; step < step_end; step += 2 * SK_WAVES) {
-    const bool more = step + SK_WAVES < step_end;
+  for (; step < step_end; step += 2 * WAVES) {
+    const bool more = step + WAVES < step_end;
     if (more) {
-      load_w(1, step + SK_WAVES);
-      load_x(1, step + SK_WAVES);
+      load_w(1, step + WAVES);
+      load_x(1, step + WAVES);
     }
     products(0);
     if (more) {
-      if (step + 2 * SK_WAVES < step_end) {
-        load_w(0, step + 2 * SK_WAVES);
-        load_x(0, step + 2 * SK_WAVES);
+      if (step + 2 * WAVES < step_end) {
+        load_w(0, step + 2 * WAVES);
+        load_x(0, step + 2 * WAVES);
       }
       products(1);
     }
@@ -209,7 +211,7 @@ __global__ __launch_bounds__(64 * SK_WAVES) void gemm_skinny_kernel(SkinnyArgs p
   __syncthreads();
   if (wave > 0) return;
 #pragma unroll
-  for (int v = 0; v < SK_WAVES - 1; ++v)
+  for (int v = 0; v < WAVES - 1; ++v)
 #pragma unroll
     for (int ta = 0; ta < NT; ++ta)
 #pragma unroll
@@ -351,11 +353,14 @@ extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
 
 template <int NT, int EPI>
 static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream) {
+  // 8 wavefronts where the grid is small; with 3 or 4 tiles of x rows they would not fit
+  // the register file.
+  constexpr int W = (EPI == SK_ACC || EPI == SK_QKV) ? 8 : SK_WAVES;
   switch ((a.M + 15) / 16) {
-    case 1: gemm_skinny_kernel<1, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
-    case 2: gemm_skinny_kernel<2, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
-    case 3: gemm_skinny_kernel<3, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
-    default: gemm_skinny_kernel<4, NT, EPI><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
+    case 1: gemm_skinny_kernel<1, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a); break;
+    case 2: gemm_skinny_kernel<2, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a); break;
+    case 3: gemm_skinny_kernel<3, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
+    default: gemm_skinny_kernel<4, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
   }
 }
 
