@@ -112,7 +112,8 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
   for (int t = 0; t < MT; ++t) xrow[t] = p.x + (size_t)min(t * 16 + r, M - 1) * K;
 
-  Frag a[2][NT][4], b[2][MT][4];
+  constexpr int DEPTH = MT == 1 ? 3 : (MT == 2 ? 2 : 1);
+  Frag a[DEPTH][NT][4], b[DEPTH][MT][4];
   auto load_w = [&](int buf, int step) {
     const int kk = step * 128 + g4 * 8;
 #pragma unroll
@@ -172,10 +173,10 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
           acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[buf][ta][j].v, b[buf][tb][j].v,
                                                                 acc[ta][tb], 0, 0, 0);
   };
-  // Two steps in flight where the registers allow four wavefronts a SIMD; with three or four
-  // tiles of x rows the second buffer would halve that, and one step at a time is faster.
-  constexpr bool PIPELINED = MT <= 2;
-  if constexpr (!PIPELINED) {
+  // DEPTH k-steps per wavefront between a load's issue and its use: three for one tile of x
+  // rows, two for two; with three or four tiles of x rows the extra buffers would cost
+  // wavefronts per SIMD, and one step at a time is faster.
+  if constexpr (DEPTH == 1) {
     for (; step < step_end; step += WAVES) {
       products(0);
       if (step + WAVES < step_end) {
@@ -183,20 +184,26 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
         load_x(0, step + WAVES);
       }
     }
-  }
-  for (; step < step_end; step += 2 * WAVES) {
-    const bool more = step + WAVES < step_end;
-    if (more) {
-      load_w(1, step + WAVES);
-      load_x(1, step + WAVES);
-    }
-    products(0);
-    if (more) {
-      if (step + 2 * WAVES < step_end) {
-        load_w(0, step + 2 * WAVES);
-        load_x(0, step + 2 * WAVES);
+  } else {
+#pragma unroll
+    for (int d = 1; d < DEPTH - 1; ++d) {
+      if (step + d * WAVES < step_end) {
+        load_w(d, step + d * WAVES);
+        load_x(d, step + d * WAVES);
       }
-      products(1);
+    }
+    for (; step < step_end; step += DEPTH * WAVES) {
+#pragma unroll
+      for (int d = 0; d < DEPTH; ++d) {
+        const int now = step + d * WAVES, ahead = now + (DEPTH - 1) * WAVES;
+        if (now < step_end) {
+          if (ahead < step_end) {
+            load_w((d + DEPTH - 1) % DEPTH, ahead);
+            load_x((d + DEPTH - 1) % DEPTH, ahead);
+          }
+          products(d);
+        }
+      }
     }
   }
 
