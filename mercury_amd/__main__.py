@@ -39,6 +39,10 @@ def build_parser() -> argparse.ArgumentParser:
     g.add_argument("--scan-limit", type=int, default=128)
     g.add_argument("--cryptographic-hashes", action="store_true")
     g.add_argument("--debug-invariants", action="store_true")
+    g.add_argument("--no-graphs", action="store_true",
+                   help="launch every decode step kernel by kernel instead of replaying a HIP graph")
+    g.add_argument("--no-lookahead", action="store_true",
+                   help="never start a decode step before the previous one's tokens are read")
     g.add_argument("--seed", type=int, default=0)
     g.add_argument("--stats", action="store_true", help="print the engine snapshot to stderr")
 
@@ -76,7 +80,8 @@ def run_generate(args) -> int:
         prefill_budget=args.prefill_budget, max_model_len=args.max_model_len, policy=args.policy,
         aging_tokens_per_s=args.aging_tokens_per_s, max_wait_s=args.max_wait_s,
         scan_limit=args.scan_limit, cryptographic_hashes=args.cryptographic_hashes,
-        debug_invariants=args.debug_invariants, seed=args.seed)
+        debug_invariants=args.debug_invariants, seed=args.seed,
+        use_graphs=not args.no_graphs, lookahead=not args.no_lookahead)
     engine = Engine(cfg)
     params = SamplingParams(temperature=args.temperature, top_p=args.top_p,
                             ignore_eos=args.ignore_eos)

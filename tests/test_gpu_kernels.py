@@ -704,6 +704,27 @@ def test_attention_decode_with_split_keys(batch, context):
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("dtype,kernel", [(torch.float32, "generic"), (torch.bfloat16, "mfma")])
+@pytest.mark.parametrize("q_len", [1, 40])
+def test_attention_over_a_very_long_context(dtype, kernel, q_len):
+    """20,000 cached keys (block tables of 1,250 pages, far more than the 64 entries a
+    wavefront holds at a time), a decoded token or a short portion at the end; one key far
+    back is made to stand out for the last query, so it has to be found."""
+    n_q, n_kv, d, page, s = 4, 2, 64, 16, 20000
+    k = rounded(rnd(s, n_kv, d, seed=701), dtype)
+    v = rounded(rnd(s, n_kv, d, seed=702), dtype)
+    q = rounded(rnd(q_len, n_q, d, seed=703), dtype)
+    far = 1234
+    k[far, 0] = rounded(q[-1, 0] * 4.0, dtype)            # head 0 of the last query looks there
+    v[far, 0] = 7.0
+    pages = torch.randperm(1300, generator=torch.Generator().manual_seed(5)).tolist()[: -(-s // page)]
+    got = run_attention([q], [k], [v], dtype, [pages], page, 1300, [s], [q_len], d ** -0.5,
+                        kernel=kernel)
+    want = plain.causal_attention(q, k, v, d ** -0.5, s - q_len)
+    torch.testing.assert_close(got, want, **tol(dtype))
+    assert got[-1, 0].mean() > 6.0                       # the far value dominates that head
+
+
 def test_attention_gqa_equals_mha_with_repeated_heads():
     n_q, n_kv, d, page, s = 6, 2, 16, 16, 37
     q, k, v = (rnd(s, h, d, seed=90 + i) for i, h in enumerate((n_q, n_kv, n_kv)))
