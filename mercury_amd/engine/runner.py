@@ -129,7 +129,7 @@ class ModelRunner:
         require_gpu(device)
         self.graphs: dict = {}
         self.use_graphs = bool(use_graphs) and all(
-            getattr(layer.mixer, "graph_safe", False) for layer in model.layers)
+            getattr(layer, "graph_safe", False) for layer in model.layers)
         self.max_graph_batch = int(max_graph_batch)
         self.last_prepare_seconds = 0.0
         self.model, self.manager = model, manager

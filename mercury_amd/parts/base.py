@@ -96,6 +96,11 @@ class LayerCache:
 class Part:
     """Base of all parts: declares tensors, receives them."""
 
+    # True when forward() only launches kernels on the current stream (no host reads of device
+    # data, no host-side branching on them), so a decode step through the part can be captured
+    # in a HIP graph and replayed.  A layer is captured only if all of its parts say so.
+    graph_safe = False
+
     def param_specs(self) -> dict:
         return {}
 
@@ -123,11 +128,6 @@ class PositionEncoding(Part):
 
 
 class Mixer(Part):
-    # True when forward() only launches kernels on the current stream (no host reads of device
-    # data, no host-side branching on them), so a decode step through it can be captured in a
-    # HIP graph and replayed.
-    graph_safe = False
-
     def cache_spec(self) -> CacheSpec | None:
         return None
 

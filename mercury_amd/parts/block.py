@@ -27,6 +27,10 @@ class PreNormBlock(Part):
             out += [("ffn", self.ffn), ("norm_ffn", self.norm_ffn)]
         return out
 
+    @property
+    def graph_safe(self) -> bool:
+        return all(part.graph_safe for _, part in self._children())
+
     def param_specs(self) -> dict:
         specs = {}
         for key, part in self._children():

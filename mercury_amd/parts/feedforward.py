@@ -15,6 +15,8 @@ class GatedMLP(FeedForward):
     (reference: mercury/model/qwen2.py:34-42).  Tensor names: ``gate_proj``, ``up_proj``,
     ``down_proj``."""
 
+    graph_safe = True
+
     def __init__(self, hidden: int, intermediate: int, activation: str = "silu"):
         if activation not in ACTIVATIONS:
             raise ValueError(f"activation {activation!r} is not implemented; known: {ACTIVATIONS}")

@@ -16,6 +16,8 @@ class RMSNorm(Norm):
     sums of the preceding projection that are added into the float32 stream in the same pass.
     """
 
+    graph_safe = True
+
     def __init__(self, size: int, eps: float):
         self.size = int(size)
         self.eps = float(eps)
