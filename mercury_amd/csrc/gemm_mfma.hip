@@ -511,7 +511,24 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int r = lane & 15, g4 = lane >> 4;
   const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
-  const int m0 = blockIdx.y * BM, n0 = blockIdx.x * (EPI == EPI_GATED ? BN / 2 : BN);
+  // Which tile: workgroups go to the 8 XCDs in turn, each with an L2 of its own, so the
+  // launch index is first renumbered to give every XCD a contiguous stretch of tiles, and the
+  // stretch is walked in bands of 8 tile rows, column by column, so that the tiles in flight
+  // on an XCD share rows of x and rows of W in its L2.
+  int tile_m, tile_n;
+  {
+    const int gx = gridDim.x, gy = gridDim.y, total = gx * gy;
+    const int id = blockIdx.y * gx + blockIdx.x;
+    const int per = (total + 7) / 8, tall = total % 8;
+    const int xcd = id % 8, local = id / 8;
+    const int renum = (tall == 0 || xcd < tall) ? xcd * per + local
+                                                : tall * per + (xcd - tall) * (per - 1) + local;
+    const int band = 8 * gx, first = renum / band * 8;
+    const int height = min(gy - first, 8), in_band = renum % band;
+    tile_m = first + in_band % height;
+    tile_n = in_band / height;
+  }
+  const int m0 = tile_m * BM, n0 = tile_n * (EPI == EPI_GATED ? BN / 2 : BN);
 
   // Staging: thread t moves chunk t, t + 256, ... of each operand's tile.
   const bf16_t* xg[XCH];
@@ -540,28 +557,28 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 #pragma unroll
     for (int b = 0; b < TN; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  uint4 xr[XCH], wr[WCH];
-  auto fetch = [&](int k0) {
+  // A stage's loads are asked for one or two stages before it is needed, into registers (the
+  // latency of a load is several stages' worth of products), and parked in LDS one stage
+  // before.
+  struct Staged {
+    uint4 x[XCH], w[WCH];
+  };
+  auto fetch = [&](int k0) __attribute__((always_inline)) {
+    Staged r;
     const bool ok = k0 + sk < K;
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) xr[i] = ok ? ld16(xg[i] + k0) : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < XCH; ++i) r.x[i] = ok ? ld16(xg[i] + k0) : make_uint4(0, 0, 0, 0);
 #pragma unroll
-    for (int i = 0; i < WCH; ++i) wr[i] = ok ? ld16(wg[i] + k0) : make_uint4(0, 0, 0, 0);
+    for (int i = 0; i < WCH; ++i) r.w[i] = ok ? ld16(wg[i] + k0) : make_uint4(0, 0, 0, 0);
+    return r;
   };
-  auto stash = [&](int buf) {
+  auto stash = [&](const Staged& r, int buf) __attribute__((always_inline)) {
 #pragma unroll
-    for (int i = 0; i < XCH; ++i) *(uint4*)(&xs[buf][xo[i]]) = xr[i];
+    for (int i = 0; i < XCH; ++i) *(uint4*)(&xs[buf][xo[i]]) = r.x[i];
 #pragma unroll
-    for (int i = 0; i < WCH; ++i) *(uint4*)(&ws[buf][wo[i]]) = wr[i];
+    for (int i = 0; i < WCH; ++i) *(uint4*)(&ws[buf][wo[i]]) = r.w[i];
   };
-
-  const int steps = (K + TK - 1) / TK;
-  fetch(0);
-  stash(0);
-  __syncthreads();
-  for (int s = 0; s < steps; ++s) {
-    const int buf = s & 1;
-    if (s + 1 < steps) fetch((s + 1) * TK);
+  auto products = [&](int buf) __attribute__((always_inline)) {
 #pragma unroll
     for (int kk = 0; kk < TK; kk += 32) {
       Frag a[TM], b[TN];
@@ -579,8 +596,40 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
           acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[tb].v, a[ta].v, acc[ta][tb],
                                                                 0, 0, 0);
     }
-    if (s + 1 < steps) stash(buf ^ 1);
+  };
+
+  const int steps = (K + TK - 1) / TK;
+  // Small tiles have the registers for a second set in flight (the loop is unrolled by two so
+  // that no set is ever copied: a copy would wait for its loads); the 128 x 128 tile would
+  // lose its second workgroup per compute unit to it, and asks one stage ahead only.
+  constexpr bool TWO_AHEAD = BM * BN <= 64 * 128;
+  Staged even = fetch(0);
+  stash(even, 0);
+  if constexpr (TWO_AHEAD) {
+    Staged odd = fetch(TK);          // past K: zeros, never parked
+    even = fetch(2 * TK);
     __syncthreads();
+    for (int s = 0; s < steps; s += 2) {
+      products(0);
+      if (s + 1 < steps) stash(odd, 1);
+      odd = fetch((s + 3) * TK);
+      __syncthreads();
+      if (s + 1 < steps) {
+        products(1);
+        if (s + 2 < steps) stash(even, 0);
+        even = fetch((s + 4) * TK);
+        __syncthreads();
+      }
+    }
+  } else {
+    __syncthreads();
+    for (int s = 0; s < steps; ++s) {   // not unrolled: the loop body's registers are the limit
+      const int buf = s & 1;
+      if (s + 1 < steps) even = fetch((s + 1) * TK);
+      products(buf);
+      if (s + 1 < steps) stash(even, buf ^ 1);
+      __syncthreads();
+    }
   }
 
   // acc[ta][tb][i] = y[m = m0 + wm + ta*16 + r][n = n0 + wn + tb*16 + g4*4 + i]
