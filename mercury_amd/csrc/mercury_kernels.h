@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 3
+#define MK_ABI_VERSION 4
 
 #ifdef __cplusplus
 extern "C" {
@@ -134,9 +134,14 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
 int mk_argmax(const float* logits, int rows, int vocab, long long row_stride, int* out,
               void* parts, hipStream_t stream);
 
+// One token per row: the argmax where temperature <= 0, else an inverse-CDF draw with the
+// row's uniform number from softmax(logits / temperature) restricted to the nucleus top_p
+// (top_ps null: no row restricts it, and the threshold search is skipped).  scratch:
+// mk_sample_scratch_bytes(rows, top_ps != null) bytes, 256-byte aligned.
+long long mk_sample_scratch_bytes(int rows, int nucleus);
 int mk_sample(const float* logits, int rows, int vocab, long long row_stride,
               const float* temperatures, const float* top_ps, const float* uniforms,
-              float* probs_scratch, int* out, hipStream_t stream);
+              void* scratch, int* out, hipStream_t stream);
 
 #ifdef __cplusplus
 }

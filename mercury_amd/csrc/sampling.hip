@@ -9,7 +9,8 @@
 // The reference draws with a generator shared by the whole batch; here the caller passes a
 // uniform number u in [0, 1) per row and the token is the first, in index order, whose
 // inclusive cumulative kept mass exceeds u * total.  Equal probabilities at the nucleus
-// edge are kept together.
+// edge are kept together.  Every pass over a row's vocabulary is shared out over 64
+// workgroups.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -100,119 +101,363 @@ extern "C" int mk_argmax(const float* logits, int rows, int vocab, long long row
   return 0;
 }
 
-// Mass of the probabilities strictly above the threshold.
-__device__ float mass_above(const float* probs, int vocab, float threshold, float* scratch) {
-  float s = 0.f;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float p = probs[i];
-    if (p > threshold) s += p;
+// ------------------------------------------------------------- sampling without a nucleus
+//
+// When no row restricts the nucleus (top_p >= 1) the draw needs no threshold search, and the
+// vocabulary is shared out: SAMPLE_PARTS workgroups per row each take a stretch of it and
+// report its maximum (with the index, for greedy rows) and the sum of exp(x / t - maximum);
+// one workgroup per row then rescales the sums to the row's maximum, finds by their running
+// total (in part order) the stretch in which u * total is crossed, and walks that stretch
+// alone.  The order of every addition is fixed by the layout, not by timing.
+#define SAMPLE_PARTS 64
+
+struct SamplePart {
+  float best_v;  // largest raw logit of the stretch
+  int best_i;
+  float m;       // largest scaled logit (x / t)
+  float z;       // sum of exp(x / t - m)
+};
+
+__global__ __launch_bounds__(256) void sample_parts_kernel(const float* __restrict__ logits,
+                                                           int vocab, long long row_stride,
+                                                           const float* __restrict__ temperatures,
+                                                           SamplePart* __restrict__ parts) {
+  __shared__ MaxIdx mi_scratch[256 / MK_WAVE];
+  __shared__ float scratch[16];
+  const int row = blockIdx.y, part = blockIdx.x;
+  const int per = (vocab + SAMPLE_PARTS - 1) / SAMPLE_PARTS;
+  const int begin = min(vocab, part * per), count = min(vocab, begin + per) - begin;
+  const float* x = logits + (size_t)row * row_stride + begin;
+  MaxIdx best = block_argmax(x, count, mi_scratch);
+  SamplePart out;
+  out.best_v = count > 0 ? best.v : -INFINITY;
+  out.best_i = count > 0 ? best.i + begin : 0x7fffffff;
+  const float t = temperatures[row];
+  out.m = -INFINITY;
+  out.z = 0.f;
+  if (t > 0.f && count > 0) {
+    const float inv_t = 1.f / fmaxf(t, 1e-5f);
+    out.m = best.v * inv_t;
+    float z = 0.f;
+    for (int i = threadIdx.x; i < count; i += blockDim.x) z += expf(x[i] * inv_t - out.m);
+    out.z = block_sum(z, scratch);
   }
-  return block_sum(s, scratch);
+  if (threadIdx.x == 0) parts[row * SAMPLE_PARTS + part] = out;
 }
 
-__global__ __launch_bounds__(SP_THREADS) void sample_kernel(
-    const float* __restrict__ logits, int vocab, long long row_stride,
-    const float* __restrict__ temperatures, const float* __restrict__ top_ps,
-    const float* __restrict__ uniforms, float* __restrict__ probs_all, int* __restrict__ out) {
-  __shared__ MaxIdx mi_scratch[SP_THREADS / MK_WAVE];
-  __shared__ float scratch[SP_THREADS / MK_WAVE];
-  __shared__ float chunk_sum[SP_THREADS];
-  __shared__ int chosen;
-  const int r = blockIdx.x;
-  const float* row = logits + (size_t)r * row_stride;
-  float* probs = probs_all + (size_t)r * vocab;
-  const float temperature = temperatures[r];
+// The value a token weighs in a row's draw, and whether the nucleus keeps it: kept are the
+// tokens whose weight's bit pattern is at least `keep_from` (weights are positive floats, so
+// their patterns order as they do).
+__device__ __forceinline__ float draw_weight(float x, float inv_t, float m, unsigned keep_from) {
+  const float e = expf(x * inv_t - m);
+  return __float_as_uint(e) >= keep_from ? e : 0.f;
+}
 
-  const MaxIdx best = block_argmax(row, vocab, mi_scratch);
-  if (temperature <= 0.f) {
-    if (threadIdx.x == 0) out[r] = best.i;
+__global__ __launch_bounds__(256) void sample_pick_kernel(const float* __restrict__ logits,
+                                                          int vocab, long long row_stride,
+                                                          const float* __restrict__ temperatures,
+                                                          const float* __restrict__ uniforms,
+                                                          const SamplePart* __restrict__ parts,
+                                                          const unsigned* __restrict__ keep,
+                                                          int* __restrict__ out) {
+  static_assert(SAMPLE_PARTS == MK_WAVE, "one part per lane of the first wavefront");
+  __shared__ float running[SAMPLE_PARTS + 1];   // mass before each part, at the row's maximum
+  __shared__ float chunk_sum[256];
+  __shared__ int where[2];                      // the part that holds the draw; greedy answer
+  __shared__ float row_max;
+  const int row = blockIdx.x, tid = threadIdx.x;
+  const float t = temperatures[row];
+  if (tid < MK_WAVE) {
+    const SamplePart mine = parts[row * SAMPLE_PARTS + tid];
+    MaxIdx best = {mine.best_v, mine.best_i};
+    float m = mine.m;
+#pragma unroll
+    for (int k = MK_WAVE / 2; k > 0; k >>= 1) {
+      MaxIdx o = {__shfl_xor(best.v, k, MK_WAVE), __shfl_xor(best.i, k, MK_WAVE)};
+      best = better(best, o);
+      m = fmaxf(m, __shfl_xor(m, k, MK_WAVE));
+    }
+    // inclusive running total of the rescaled sums, in part order
+    float mass = mine.z > 0.f ? mine.z * expf(mine.m - m) : 0.f;
+    float incl = mass;
+#pragma unroll
+    for (int k = 1; k < MK_WAVE; k <<= 1) {
+      const float up = __shfl_up(incl, k, MK_WAVE);
+      if (tid >= k) incl += up;
+    }
+    running[tid + 1] = incl;
+    if (tid == 0) {
+      running[0] = 0.f;
+      where[1] = best.i == 0x7fffffff ? 0 : best.i;
+      row_max = m;
+    }
+  }
+  __syncthreads();
+  if (t <= 0.f) {
+    if (tid == 0) out[row] = where[1];
     return;
   }
-  const float inv_t = 1.f / fmaxf(temperature, 1e-5f);
-
-  // softmax of the scaled logits; the maximum of the scaled row is at the argmax.
-  const float top = best.v * inv_t;
-  float z = 0.f;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) {
-    const float e = expf(row[i] * inv_t - top);
-    probs[i] = e;
-    z += e;
-  }
-  z = block_sum(z, scratch);
-  const float inv_z = 1.f / z;
-  for (int i = threadIdx.x; i < vocab; i += blockDim.x) probs[i] *= inv_z;
-  __syncthreads();
-
-  // The smallest kept probability: the least v with mass_above(v) <= top_p, found by
-  // bisection over the bit patterns of non-negative floats (monotone in value).
-  float keep_from = 0.f;
-  const float top_p = top_ps[r];
-  if (top_p < 1.f) {
-    unsigned lo = 0u, hi = __float_as_uint(inv_z);  // exp(0) / z is the largest probability
-    while (lo < hi) {
-      const unsigned mid = lo + (hi - lo) / 2u;
-      if (mass_above(probs, vocab, __uint_as_float(mid), scratch) <= top_p)
-        hi = mid;
-      else
-        lo = mid + 1u;
-    }
-    keep_from = __uint_as_float(lo);
-  }
-
-  // Inverse CDF in index order: each thread owns one contiguous chunk.
-  const int per = (vocab + blockDim.x - 1) / blockDim.x;
-  const int begin = min(vocab, (int)threadIdx.x * per), end = min(vocab, begin + per);
-  float mine = 0.f;
-  for (int i = begin; i < end; ++i) {
-    const float p = probs[i];
-    if (p >= keep_from) mine += p;
-  }
-  chunk_sum[threadIdx.x] = mine;
-  if (threadIdx.x == 0) chosen = -1;
-  __syncthreads();
-  if (threadIdx.x == 0) {
-    float total = 0.f;
-    for (int c = 0; c < (int)blockDim.x; ++c) total += chunk_sum[c];
-    const float target = uniforms[r] * total;
-    float running = 0.f;
+  const float total = running[SAMPLE_PARTS];
+  const float target = uniforms[row] * total;
+  if (tid == 0) {
+    // the first part whose running total passes the target; if u * total rounded up to the
+    // total, the last part that holds any mass
     int c = 0;
-    for (; c < (int)blockDim.x; ++c) {
-      if (running + chunk_sum[c] > target) break;
-      running += chunk_sum[c];
+    while (c < SAMPLE_PARTS && !(running[c + 1] > target)) ++c;
+    if (c == SAMPLE_PARTS)
+      for (c = SAMPLE_PARTS - 1; c > 0 && running[c + 1] == running[c]; --c) {}
+    where[0] = c;
+  }
+  __syncthreads();
+  const int c = where[0];
+  const int per = (vocab + SAMPLE_PARTS - 1) / SAMPLE_PARTS;
+  const int begin = min(vocab, c * per), count = min(vocab, begin + per) - begin;
+  const float* x = logits + (size_t)row * row_stride + begin;
+  const float inv_t = 1.f / fmaxf(t, 1e-5f), m = row_max;
+  const unsigned keep_from = keep ? keep[row] : 0u;
+  // every thread a contiguous chunk of the stretch, then the chunks in order
+  const int each = (count + 255) / 256;
+  const int lo = min(count, tid * each), hi = min(count, lo + each);
+  float mine = 0.f;
+  for (int i = lo; i < hi; ++i) mine += draw_weight(x[i], inv_t, m, keep_from);
+  chunk_sum[tid] = mine;
+  __syncthreads();
+  if (tid == 0) {
+    float before = running[c];
+    int k = 0;
+    for (; k < 256; ++k) {
+      if (before + chunk_sum[k] > target) break;
+      before += chunk_sum[k];
     }
-    if (c == (int)blockDim.x) {
-      // u * total rounded up to the total: take the last kept token.
-      for (c = blockDim.x - 1; c > 0 && chunk_sum[c] == 0.f; --c) {}
-      running = -1.f;
-    }
-    const int cb = min(vocab, c * per), ce = min(vocab, cb + per);
+    // the token that crosses the target, or, where rounding lets none cross (u * total
+    // rounded up to the total; the two sums of a chunk differing), the last kept one
+    if (k == 256) k = 255;
     int pick = -1, last_kept = -1;
-    for (int i = cb; i < ce; ++i) {
-      const float p = probs[i];
-      if (p < keep_from) continue;
-      last_kept = i;
-      if (running >= 0.f) {
-        running += p;
-        if (running > target) {
-          pick = i;
+    for (; k >= 0 && pick < 0 && last_kept < 0; --k) {
+      const int klo = min(count, k * each), khi = min(count, klo + each);
+      for (int i = klo; i < khi; ++i) {
+        const float e = draw_weight(x[i], inv_t, m, keep_from);
+        if (e <= 0.f) continue;
+        last_kept = begin + i;
+        before += e;
+        if (before > target) {
+          pick = begin + i;
           break;
         }
       }
+      before = INFINITY;                      // earlier chunks only lend their last kept token
     }
-    chosen = pick >= 0 ? pick : (last_kept >= 0 ? last_kept : best.i);
+    if (pick < 0) pick = last_kept >= 0 ? last_kept : where[1];
+    out[row] = max(0, min(vocab - 1, pick));
+  }
+}
+
+// ------------------------------------------------------------------- the nucleus, found
+//
+// A token is kept iff the mass of the tokens weightier than it is at most top_p of the row's
+// (so the token that crosses top_p stays, and tokens of equal weight stay or go together).
+// With weights e = exp(x / t - max) in (0, 1], whose float bit patterns order as the values
+// do, that is: kept are the patterns >= the least pattern b with mass(patterns > b) <=
+// top_p * total.  The search takes three histograms of the mass by pattern: over the upper 11
+// bits, then, inside the bin found, over the next 11, then over the last 10.  Every
+// workgroup gathers its stretch's histogram in LDS and adds the bins it touched to the
+// row's; mass is added up as 40-bit fixed point integers, so no sum depends on the order of
+// the atomic additions.
+#define NUCLEUS_LEVELS 3
+__device__ __host__ constexpr int nucleus_shift(int level) { return level == 0 ? 21 : (level == 1 ? 10 : 0); }
+__device__ __host__ constexpr int nucleus_bins(int level) { return level == 0 ? 512 : (level == 1 ? 2048 : 1024); }
+#define NUCLEUS_ROW_BINS (512 + 2048 + 1024)
+
+struct NucleusRow {
+  unsigned long long above;  // mass of the patterns above the prefix's range
+  unsigned long long limit;  // top_p of the total
+  unsigned prefix;           // the threshold's upper bits found so far, in place
+  unsigned pad;
+};
+
+__device__ __forceinline__ unsigned long long fixed_mass(float e) {
+  return (unsigned long long)((double)e * 1099511627776.0);   // 2^40
+}
+
+__global__ void zero_u64_kernel(unsigned long long* p, size_t n) {
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n;
+       i += (size_t)gridDim.x * blockDim.x)
+    p[i] = 0ull;
+}
+
+// The row's largest scaled logit, out of the parts' (every thread of the workgroup gets it).
+__device__ float row_maximum(const SamplePart* parts, int row, float* shared) {
+  if (threadIdx.x < MK_WAVE) {
+    const float m = wave_max(parts[row * SAMPLE_PARTS + threadIdx.x].m);
+    if (threadIdx.x == 0) *shared = m;
   }
   __syncthreads();
-  if (threadIdx.x == 0) out[r] = chosen;
+  return *shared;
+}
+
+// Mass by the LEVEL's bits of the pattern, of the tokens whose bits above them equal the
+// prefix found so far.  hist: the row's bins of this level.
+template <int LEVEL>
+__global__ __launch_bounds__(256) void nucleus_histogram_kernel(
+    const float* __restrict__ logits, int vocab, long long row_stride,
+    const float* __restrict__ temperatures, const float* __restrict__ top_ps,
+    const SamplePart* __restrict__ parts, const NucleusRow* __restrict__ rows,
+    unsigned long long* __restrict__ hist) {
+  constexpr int SHIFT = nucleus_shift(LEVEL), BINS = nucleus_bins(LEVEL);
+  constexpr int ABOVE = LEVEL == 0 ? 32 : nucleus_shift(LEVEL - 1);   // bits from here up are the prefix
+  __shared__ unsigned long long local[BINS];
+  __shared__ float row_max;
+  const int row = blockIdx.y, part = blockIdx.x;
+  const float t = temperatures[row];
+  if (t <= 0.f || top_ps[row] >= 1.f) return;     // greedy, or nothing to restrict
+  for (int i = threadIdx.x; i < BINS; i += blockDim.x) local[i] = 0ull;
+  const int per = (vocab + SAMPLE_PARTS - 1) / SAMPLE_PARTS;
+  const int begin = min(vocab, part * per), count = min(vocab, begin + per) - begin;
+  const float* x = logits + (size_t)row * row_stride + begin;
+  const float inv_t = 1.f / fmaxf(t, 1e-5f), m = row_maximum(parts, row, &row_max);   // syncs
+  const unsigned prefix = LEVEL == 0 ? 0u : rows[row].prefix;
+  for (int i = threadIdx.x; i < count; i += blockDim.x) {
+    const float e = expf(x[i] * inv_t - m);
+    const unsigned b = __float_as_uint(e);
+    if (LEVEL == 0 || (b >> ABOVE) == (prefix >> ABOVE))
+      atomicAdd(&local[(b >> SHIFT) & (BINS - 1)], fixed_mass(e));
+  }
+  __syncthreads();
+  unsigned long long* mine = hist + (size_t)row * BINS;
+  for (int i = threadIdx.x; i < BINS; i += blockDim.x)
+    if (local[i] != 0ull) atomicAdd(mine + i, local[i]);
+}
+
+// Walk a level's histogram from its top: the least bin with mass(bins above it) + what lies
+// above the prefix's range <= limit.  One workgroup per row; thread k sums bins
+// [k * EACH, (k + 1) * EACH), the first thread then walks the sums and the bins of one.
+template <int LEVEL>
+__global__ __launch_bounds__(256) void nucleus_pick_kernel(
+    const float* __restrict__ temperatures, const float* __restrict__ top_ps,
+    const unsigned long long* __restrict__ hist, NucleusRow* __restrict__ rows,
+    unsigned* __restrict__ keep) {
+  constexpr int BINS = nucleus_bins(LEVEL), EACH = BINS / 256, SHIFT = nucleus_shift(LEVEL);
+  __shared__ unsigned long long chunk[256];
+  const int row = blockIdx.x, tid = threadIdx.x;
+  if (temperatures[row] <= 0.f || top_ps[row] >= 1.f) {
+    if (LEVEL == NUCLEUS_LEVELS - 1 && tid == 0) keep[row] = 0u;   // everything is kept
+    return;
+  }
+  const unsigned long long* bins = hist + (size_t)row * BINS;
+  unsigned long long sum = 0ull;
+  for (int i = 0; i < EACH; ++i) sum += bins[tid * EACH + i];
+  chunk[tid] = sum;
+  __syncthreads();
+  if (tid != 0) return;
+  unsigned long long above, limit;
+  if (LEVEL == 0) {
+    unsigned long long total = 0ull;
+    for (int k = 0; k < 256; ++k) total += chunk[k];
+    above = 0ull;
+    limit = (unsigned long long)((double)top_ps[row] * (double)total);
+  } else {
+    above = rows[row].above;
+    limit = rows[row].limit;
+  }
+  // `above` never passes the limit: the bin it belongs to is a valid threshold.  Down the
+  // chunks while a whole chunk still fits, then down the bins of the chunk that does not.
+  int k = 255;
+  while (k > 0 && above + chunk[k] <= limit) above += chunk[k--];
+  int i = EACH - 1;
+  while (i > 0 && above + bins[k * EACH + i] <= limit) above += bins[k * EACH + i--];
+  const unsigned found = (unsigned)(k * EACH + i);
+  const unsigned prefix = (LEVEL == 0 ? 0u : rows[row].prefix) | (found << SHIFT);
+  rows[row].above = above;
+  rows[row].limit = limit;
+  rows[row].prefix = prefix;
+  if (LEVEL == NUCLEUS_LEVELS - 1) keep[row] = prefix;
+}
+
+// The parts again, for the draw, into a second array: the row's maximum for every part, and
+// the kept mass only.
+__global__ __launch_bounds__(256) void nucleus_parts_kernel(const float* __restrict__ logits,
+                                                            int vocab, long long row_stride,
+                                                            const float* __restrict__ temperatures,
+                                                            const unsigned* __restrict__ keep,
+                                                            const SamplePart* __restrict__ parts,
+                                                            SamplePart* __restrict__ kept) {
+  __shared__ float scratch[16];
+  __shared__ float row_max;
+  const int row = blockIdx.y, part = blockIdx.x;
+  SamplePart out = parts[row * SAMPLE_PARTS + part];
+  out.z = 0.f;
+  const float t = temperatures[row];
+  if (t > 0.f) {   // the same for every thread of the workgroup
+    const float m = row_maximum(parts, row, &row_max);
+    const int per = (vocab + SAMPLE_PARTS - 1) / SAMPLE_PARTS;
+    const int begin = min(vocab, part * per), count = min(vocab, begin + per) - begin;
+    const float* x = logits + (size_t)row * row_stride + begin;
+    const float inv_t = 1.f / fmaxf(t, 1e-5f);
+    const unsigned keep_from = keep[row];
+    float z = 0.f;
+    for (int i = threadIdx.x; i < count; i += blockDim.x) z += draw_weight(x[i], inv_t, m, keep_from);
+    out.z = block_sum(z, scratch);
+    out.m = m;
+  }
+  if (threadIdx.x == 0) kept[row * SAMPLE_PARTS + part] = out;
+}
+
+static size_t align_up(size_t n) { return (n + 255) / 256 * 256; }
+
+// Bytes of scratch mk_sample needs for `rows` rows: the parts alone without a nucleus, else
+// the parts twice, the rows' search records and thresholds, and the two histograms.
+extern "C" long long mk_sample_scratch_bytes(int rows, int nucleus) {
+  const size_t parts = align_up((size_t)rows * SAMPLE_PARTS * sizeof(SamplePart));
+  if (!nucleus) return (long long)parts;
+  return (long long)(2 * parts + align_up((size_t)rows * sizeof(NucleusRow)) +
+                     align_up((size_t)rows * sizeof(unsigned)) +
+                     (size_t)rows * NUCLEUS_ROW_BINS * 8);
 }
 
 extern "C" int mk_sample(const float* logits, int rows, int vocab, long long row_stride,
                          const float* temperatures, const float* top_ps, const float* uniforms,
-                         float* probs_scratch, int* out, hipStream_t stream) {
+                         void* scratch, int* out, hipStream_t stream) {
   MK_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "sample: bad sizes");
-  MK_REQUIRE(probs_scratch != nullptr, "sample: needs a [rows, V] float32 scratch buffer");
   if (rows == 0) return 0;
-  sample_kernel<<<rows, SP_THREADS, 0, stream>>>(logits, vocab, row_stride, temperatures, top_ps,
-                                                 uniforms, probs_scratch, out);
+  MK_REQUIRE(scratch != nullptr && rows <= 65535,
+             "sample: needs its scratch buffer (mk_sample_scratch_bytes) and at most 65535 rows");
+  char* at = (char*)scratch;
+  SamplePart* parts = (SamplePart*)at;
+  const dim3 grid(SAMPLE_PARTS, rows);
+  sample_parts_kernel<<<grid, 256, 0, stream>>>(logits, vocab, row_stride, temperatures, parts);
+  if (top_ps == nullptr) {   // no row restricts the nucleus
+    sample_pick_kernel<<<rows, 256, 0, stream>>>(logits, vocab, row_stride, temperatures, uniforms,
+                                                 parts, nullptr, out);
+    MK_LAUNCH_CHECK("sample");
+    return 0;
+  }
+  const size_t parts_bytes = align_up((size_t)rows * SAMPLE_PARTS * sizeof(SamplePart));
+  at += parts_bytes;
+  SamplePart* kept = (SamplePart*)at;
+  at += parts_bytes;
+  NucleusRow* search = (NucleusRow*)at;
+  at += align_up((size_t)rows * sizeof(NucleusRow));
+  unsigned* keep = (unsigned*)at;
+  at += align_up((size_t)rows * sizeof(unsigned));
+  unsigned long long* hist0 = (unsigned long long*)at;
+  unsigned long long* hist1 = hist0 + (size_t)rows * nucleus_bins(0);
+  unsigned long long* hist2 = hist1 + (size_t)rows * nucleus_bins(1);
+  const size_t bins = (size_t)rows * NUCLEUS_ROW_BINS;
+  zero_u64_kernel<<<(int)((bins + 1023) / 1024 < 1024 ? (bins + 1023) / 1024 : 1024), 256, 0,
+                    stream>>>(hist0, bins);
+  nucleus_histogram_kernel<0><<<grid, 256, 0, stream>>>(logits, vocab, row_stride, temperatures,
+                                                         top_ps, parts, search, hist0);
+  nucleus_pick_kernel<0><<<rows, 256, 0, stream>>>(temperatures, top_ps, hist0, search, keep);
+  nucleus_histogram_kernel<1><<<grid, 256, 0, stream>>>(logits, vocab, row_stride, temperatures,
+                                                         top_ps, parts, search, hist1);
+  nucleus_pick_kernel<1><<<rows, 256, 0, stream>>>(temperatures, top_ps, hist1, search, keep);
+  nucleus_histogram_kernel<2><<<grid, 256, 0, stream>>>(logits, vocab, row_stride, temperatures,
+                                                         top_ps, parts, search, hist2);
+  nucleus_pick_kernel<2><<<rows, 256, 0, stream>>>(temperatures, top_ps, hist2, search, keep);
+  nucleus_parts_kernel<<<grid, 256, 0, stream>>>(logits, vocab, row_stride, temperatures, keep,
+                                                 parts, kept);
+  sample_pick_kernel<<<rows, 256, 0, stream>>>(logits, vocab, row_stride, temperatures, uniforms,
+                                               kept, keep, out);
   MK_LAUNCH_CHECK("sample");
   return 0;
 }

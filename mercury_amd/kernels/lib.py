@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 
 from . import build
 
-ABI_VERSION = 3
+ABI_VERSION = 4
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -27,6 +27,7 @@ _SIGNATURES = {
         "mk_silu_mul_partials": [P, I, L, P, I, I, I, P],
         "mk_qkv_finish": [P, I, L, P, I, P, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_argmax": [P, I, I, L, P, P, P],
+        "mk_sample_scratch_bytes": [I, I],
         "mk_sample": [P, I, I, L, P, P, P, P, P, P],
     },
     "mfma": {
@@ -45,6 +46,8 @@ _SIGNATURES = {
         "mk_attention_mfma": [P, I, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, P, P, P],
     },
 }
+
+_RETURNS_SIZE = {"mk_sample_scratch_bytes"}    # byte counts; everything else returns int
 
 _loaded: dict = {}
 
@@ -78,7 +81,7 @@ def load(name: str = "core") -> ctypes.CDLL:
     for fn_name, argtypes in _SIGNATURES[name].items():
         fn = getattr(lib, fn_name)
         fn.argtypes = argtypes
-        fn.restype = c_int
+        fn.restype = c_longlong if fn_name in _RETURNS_SIZE else c_int
     _loaded[name] = lib
     return lib
 

@@ -544,20 +544,23 @@ def argmax(logits: torch.Tensor) -> torch.Tensor:
     return out
 
 
-def sample(logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor,
+def sample(logits: torch.Tensor, temperatures: torch.Tensor, top_ps: torch.Tensor | None,
            uniforms: torch.Tensor) -> torch.Tensor:
     """One token per row: argmax where temperature <= 0, else an inverse-CDF draw from the
-    temperature softmax restricted to the nucleus, using the row's uniform number."""
+    temperature softmax restricted to the nucleus, using the row's uniform number.
+    `top_ps` None says that no row restricts its nucleus, which takes a faster path (the
+    vocabulary shared out over many workgroups, no threshold search)."""
     _dev(logits, temperatures, top_ps, uniforms)
     if logits.dtype != torch.float32 or logits.dim() != 2:
         raise KernelArgumentError("sample: logits must be float32 [n, V]")
     rows, vocab = logits.shape
     for name, t in (("temperatures", temperatures), ("top_ps", top_ps), ("uniforms", uniforms)):
-        if t.dtype != torch.float32 or t.shape != (rows,):
+        if t is not None and (t.dtype != torch.float32 or t.shape != (rows,)):
             raise KernelArgumentError(f"sample: {name} must be float32 [{rows}]")
-    scratch = torch.empty((rows, vocab), dtype=torch.float32, device=logits.device)
-    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     lib = _lib.load("core")
+    scratch = torch.empty((lib.mk_sample_scratch_bytes(rows, int(top_ps is not None)),),
+                          dtype=torch.uint8, device=logits.device)
+    out = torch.empty((rows,), dtype=torch.int32, device=logits.device)
     _lib.check(lib, lib.mk_sample(_ptr(logits), rows, vocab, vocab, _ptr(temperatures),
                                   _ptr(top_ps), _ptr(uniforms), _ptr(scratch), _ptr(out),
                                   _stream()), "sample")

@@ -50,4 +50,5 @@ class Sampler:
         us = [uniform_for(self.seed if r.params.seed is None else r.params.seed, r.rid,
                           len(r.out) + ahead) for r in requests]
         packed = torch.tensor([temps, top_ps, us], dtype=torch.float32).to(logits.device)
-        return ops.sample(logits, packed[0], packed[1], packed[2])
+        nucleus = packed[1] if any(p < 1.0 for p in top_ps) else None
+        return ops.sample(logits, packed[0], nucleus, packed[2])

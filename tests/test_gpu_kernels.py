@@ -780,6 +780,62 @@ def test_sampling_rules():
             assert abs(float(cum[hi - 1] - float(us[r]))) < 1e-5 or float(cum[hi] - cum[lo]) < 1e-5
 
 
+@pytest.mark.parametrize("vocab", [50, 1003, 151936])
+def test_sampling_without_a_nucleus_over_many_workgroups(vocab):
+    """With no row restricting its nucleus the vocabulary is shared out over 64 workgroups per
+    row: the same draws as the one-workgroup kernel told that every top_p is 1, greedy rows
+    and tiny temperatures included."""
+    rows = 9
+    logits = rnd(rows, vocab, seed=103, scale=2.5)
+    logits[3, vocab - 1] = 40.0                  # all the mass in the last stretch
+    logits[4, 0] = 40.0                          # ... or in the first
+    temps = torch.tensor([0.8, 0.0, 1.3, 0.7, 0.7, 1e-7, 0.8, 0.8, 2.0])
+    us = torch.tensor([0.5, 0.3, 0.999999, 0.2, 0.9, 0.4, 0.0, 0.25, 0.75])
+    ones = torch.ones(rows)
+    fast = ops().sample(logits.to(DEV), temps.to(DEV), None, us.to(DEV)).cpu().tolist()
+    slow = ops().sample(logits.to(DEV), temps.to(DEV), ones.to(DEV), us.to(DEV)).cpu().tolist()
+    assert fast[1] == int(logits[1].argmax()) and fast[5] == int(logits[5].argmax())
+    assert fast[3] == vocab - 1 and fast[4] == 0
+    for r in range(rows):
+        if fast[r] == slow[r] or temps[r] <= 0:
+            continue
+        # only a rounding of the cumulative sum may move the draw: both tokens are where the
+        # running mass crosses u
+        probs = plain.sampling_distribution(logits[r], float(temps[r]), 1.0)
+        cum = probs.double().cumsum(-1)
+        lo, hi = sorted((fast[r], slow[r]))
+        assert float(cum[hi] - cum[lo]) < 1e-5 or abs(float(cum[hi - 1]) - float(us[r])) < 1e-5
+
+
+@pytest.mark.parametrize("vocab", [1003, 151936])
+def test_nucleus_over_a_large_vocabulary(vocab):
+    """The nucleus is found by histograms of the probability mass over the bits of the
+    probabilities: for several top_p, temperatures and uniforms per row the draw is the plain
+    implementation's (or its neighbour where a rounding of the running sum decides), and never
+    a token outside the plain nucleus."""
+    top_ps = [0.05, 0.5, 0.9, 0.999, 0.5, 1e-6, 0.9, 0.9]
+    temps = [0.8, 0.8, 1.3, 0.6, 2.0, 0.8, 0.8, 0.8]
+    us = [0.0, 0.37, 0.81, 0.999, 0.5, 0.9, 0.25, 0.75]
+    rows = len(us)
+    logits = rnd(rows, vocab, seed=104, scale=2.0)
+    logits[6, :] = 0.0
+    logits[6, 100:700] = 12.0                      # a plateau with nearly all the mass, across the edge: kept together
+    logits[7, :] = 1.25                            # all equal: everything is kept
+    got = ops().sample(logits.to(DEV), torch.tensor(temps).to(DEV), torch.tensor(top_ps).to(DEV),
+                       torch.tensor(us).to(DEV)).cpu().tolist()
+    assert got[5] == int(logits[5].argmax())       # a nucleus of one token
+    assert 100 <= got[6] < 700
+    assert got[7] == min(vocab - 1, int(0.75 * vocab))
+    for r in range(6):      # rows 6 and 7 are ties, which a sort cuts anywhere and we keep whole
+        probs = plain.sampling_distribution(logits[r], temps[r], top_ps[r])
+        want = plain.inverse_cdf_draw(probs, us[r])
+        assert probs[got[r]] > 0, f"row {r} drew a token outside the nucleus"
+        if got[r] != want:
+            cum = probs.double().cumsum(-1)
+            lo, hi = sorted((got[r], want))
+            assert float(cum[hi] - cum[lo]) < 1e-4 or abs(float(cum[hi - 1]) - us[r]) < 1e-4, r
+
+
 def test_sampling_frequencies_follow_the_distribution():
     vocab = 50
     logits = rnd(1, vocab, seed=102, scale=1.5).repeat(4000, 1)
