@@ -27,6 +27,25 @@ def uniform_for(seed: int, rid: str, index: int) -> float:
 class Sampler:
     def __init__(self, seed: int = 0):
         self.seed = int(seed)
+        self._staging: list = []     # pinned [3, n] float32 buffers, used in turn
+        self._next = 0
+
+    def _to_device(self, rows: list, device) -> torch.Tensor:
+        """[len(rows), n] float32 on the device without making the host wait for the GPU: a
+        copy out of pageable memory would, and a step may be running ahead.  A staging buffer
+        comes round again after four uses, long after its copy has run (at most two steps'
+        sampling is ever in flight)."""
+        n = len(rows[0])
+        if device.type != "cuda":
+            return torch.tensor(rows, dtype=torch.float32, device=device)
+        if not self._staging or self._staging[0].numel() < len(rows) * n:
+            size = len(rows) * max(256, 2 * n)
+            self._staging = [torch.empty(size, dtype=torch.float32, pin_memory=True)
+                             for _ in range(4)]
+        host = self._staging[self._next][: len(rows) * n].view(len(rows), n)
+        self._next = (self._next + 1) % len(self._staging)
+        host.copy_(torch.tensor(rows, dtype=torch.float32))
+        return host.to(device, non_blocking=True)
 
     def sample(self, logits: torch.Tensor, requests: list) -> list:
         """One token per row of float32 logits [n, V]; row i belongs to requests[i], whose
@@ -49,6 +68,6 @@ class Sampler:
         top_ps = [float(r.params.top_p) for r in requests]
         us = [uniform_for(self.seed if r.params.seed is None else r.params.seed, r.rid,
                           len(r.out) + ahead) for r in requests]
-        packed = torch.tensor([temps, top_ps, us], dtype=torch.float32).to(logits.device)
+        packed = self._to_device([temps, top_ps, us], logits.device)
         nucleus = packed[1] if any(p < 1.0 for p in top_ps) else None
         return ops.sample(logits, packed[0], nucleus, packed[2])
