@@ -372,46 +372,6 @@ extern "C" int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const floa
 
 // ------------------------------------------ consumers of split-K partial sums (decode path)
 
-// SiLU gating of a projection that arrives as `num_partials` float32 slices [p, T, 2I].
-template <typename T>
-__global__ void silu_mul_partials_kernel(const float* __restrict__ partials, int num_partials,
-                                         size_t partial_stride, T* __restrict__ out, int inter,
-                                         size_t total) {
-  for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < total;
-       idx += (size_t)gridDim.x * blockDim.x) {
-    const size_t t = idx / inter;
-    const int i = (int)(idx - t * inter);
-    const float* row = partials + t * 2 * (size_t)inter;
-    float g = sum_partials(row + i, num_partials, partial_stride);
-    float u = sum_partials(row + inter + i, num_partials, partial_stride);
-    // The reference rounds both projections to the storage type before gating.
-    g = Elem<T>::round(g);
-    u = Elem<T>::round(u);
-    const float s = Elem<T>::round(g / (1.f + expf(-g)));
-    Elem<T>::store(out + idx, s * u);
-  }
-}
-
-extern "C" int mk_silu_mul_partials(const float* partials, int num_partials,
-                                    long long partial_stride, void* out, int out_dtype,
-                                    int tokens, int inter, hipStream_t stream) {
-  MK_REQUIRE(tokens >= 0 && inter > 0 && num_partials >= 1, "silu_mul: bad sizes");
-  if (tokens == 0) return 0;
-  const size_t total = (size_t)tokens * inter;
-  size_t blocks = (total + 255) / 256;
-  if (blocks > 65536) blocks = 65536;
-  if (out_dtype == MK_BF16)
-    silu_mul_partials_kernel<bf16_t><<<(int)blocks, 256, 0, stream>>>(
-        partials, num_partials, (size_t)partial_stride, (bf16_t*)out, inter, total);
-  else if (out_dtype == MK_F32)
-    silu_mul_partials_kernel<float><<<(int)blocks, 256, 0, stream>>>(
-        partials, num_partials, (size_t)partial_stride, (float*)out, inter, total);
-  else
-    MK_REQUIRE(false, "silu_mul: unknown dtype %d", out_dtype);
-  MK_LAUNCH_CHECK("silu_mul_partials");
-  return 0;
-}
-
 // The q/k/v projection arrives as float32 slices [p, T, (n_q + 2 n_kv) d]; this adds them up,
 // adds the bias, rotates q and k, writes q [T, n_q d] and the cache.  Sums and rotation are
 // float32; q, k and v are rounded to the storage type first, as a stored projection would be.

@@ -712,8 +712,8 @@ static void launch_tiled_cfg(const void* x, const void* w, const void* bias, int
         (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo);
 }
 
-// Tile configurations, by index: 0 = 128x128 (k 64), 1 = 64x128, 2 = 64x64, 3 = 128x128 (k 32).
-#define TILED_CONFIGS 4
+// Tile configurations, by index: 0 = 128x128, 1 = 64x128, 2 = 64x64 (k in stages of 64).
+#define TILED_CONFIGS 3
 
 template <int EPI>
 static void launch_tiled(int config, const void* x, const void* w, const void* bias,
@@ -722,8 +722,7 @@ static void launch_tiled(int config, const void* x, const void* w, const void* b
   switch (config) {
     case 0: launch_tiled_cfg<128, 128, 64, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
     case 1: launch_tiled_cfg<64, 128, 64, 1, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 2: launch_tiled_cfg<64, 64, 64, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    default: launch_tiled_cfg<128, 128, 32, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    default: launch_tiled_cfg<64, 64, 64, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
   }
 }
 

@@ -52,10 +52,9 @@ int mk_attention_generic(const void* q, int q_stride, void* out, int out_stride,
                          int table_stride, int page_size, int n_q, int n_kv, int d, float scale,
                          int window, int tokens, hipStream_t stream);
 
-// The same two for a projection that arrives as float32 partial sums [p, T, width] of a
-// K-split product: the slices are added in order (with the bias) before the op proper.
-int mk_silu_mul_partials(const float* partials, int num_partials, long long partial_stride,
-                         void* out, int out_dtype, int tokens, int inter, hipStream_t stream);
+// mk_rope_kv_write for a projection that arrives as float32 partial sums [p, T, width] of a
+// K-split product: the slices are added in order (with the bias) before the rotation; q goes
+// to q_out [T, n_q d].
 int mk_qkv_finish(const float* partials, int num_partials, long long partial_stride,
                   const void* bias, int bias_dtype, void* q_out, int dtype,
                   const float* cos_table, const float* sin_table, int table_positions,

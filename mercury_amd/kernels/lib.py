@@ -24,7 +24,6 @@ _SIGNATURES = {
         "mk_rope_kv_write": [P, I, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_linear_generic": [P, P, I, P, I, P, I, I, I, I, I, I, I, P],
         "mk_attention_generic": [P, I, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
-        "mk_silu_mul_partials": [P, I, L, P, I, I, I, P],
         "mk_qkv_finish": [P, I, L, P, I, P, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_argmax": [P, I, I, L, P, P, P],
         "mk_sample_scratch_bytes": [I, I],

@@ -103,23 +103,9 @@ def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.
     return out
 
 
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None,
-             out_dtype: torch.dtype | None = None) -> torch.Tensor:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up [T, 2I], or for
-    float32 partial sums [P, T, 2I] of it (summed first; the result is `out_dtype`)."""
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up [T, 2I]."""
     _dev(gate_up, out)
-    if gate_up.dim() == 3:
-        if gate_up.dtype != torch.float32 or out_dtype is None:
-            raise KernelArgumentError("silu_mul: partial sums are float32 and need an out_dtype")
-        slices, tokens, two_i = gate_up.shape
-        inter = two_i // 2
-        if out is None:
-            out = torch.empty((tokens, inter), dtype=out_dtype, device=gate_up.device)
-        lib = _lib.load("core")
-        _lib.check(lib, lib.mk_silu_mul_partials(_ptr(gate_up), slices, tokens * two_i, _ptr(out),
-                                                 dtype_code(out_dtype), tokens, inter, _stream()),
-                   "silu_mul")
-        return out
     tokens, two_i = gate_up.shape
     if two_i % 2:
         raise KernelArgumentError("silu_mul: the last dimension must be even")
@@ -159,7 +145,7 @@ def _skinny_eligible(x, w: torch.Tensor) -> bool:
 
 def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """Float32 partial sums [P, M, N] of x W^T over P slices of K; the consumer (rmsnorm,
-    rope_kv_write, silu_mul: their `partials` forms) adds them up in slice order."""
+    rope_kv_write: their `partials` forms) adds them up in slice order."""
     _dev(x, w)
     if not _skinny_eligible(x, w) or x.shape[1] != w.shape[1]:
         raise KernelArgumentError(f"linear_partials: x {tuple(x.shape)} / W {tuple(w.shape)} not eligible")
@@ -500,11 +486,6 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
         # decoding: every sequence's own range in equal parts
         splits = max(1, min(blocks // ATTENTION_MIN_BLOCKS_PER_SPLIT or 1,
                             -(-ATTENTION_TARGET_WAVES // waves), 1024))
-    elif blocks > ATTENTION_PROMPT_SPLIT_BLOCKS:
-        # prompts: no wavefront walks more than a fixed stretch of keys, so the tiles at the
-        # end of a long causal prompt do not outlast all the others
-        split_blocks = ATTENTION_PROMPT_SPLIT_BLOCKS
-        splits = -(-blocks // split_blocks)
     if split_override is not None:
         splits, split_blocks = split_override
     part_o = part_ml = None
@@ -523,7 +504,6 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
 ATTENTION_TARGET_WAVES = 1024
 ATTENTION_STAGED_WORKGROUPS = 128
 ATTENTION_WIDE_TILE_WAVES = 400
-ATTENTION_PROMPT_SPLIT_BLOCKS = 1 << 30   # prompts are not split: the merge costs what the split gains
 ATTENTION_MIN_BLOCKS_PER_SPLIT = 2
 
 

@@ -329,14 +329,8 @@ def test_matrix_core_projection_refuses_what_it_cannot_do():
 
 
 def test_consumers_of_partial_sums():
-    """SiLU gating and rotary + cache write over K-split slices equal the stored-projection
-    forms applied to the rounded sum."""
-    parts = rnd(3, 9, 2 * 200, seed=27)
-    whole = parts.sum(0).to(torch.bfloat16)
-    want = ops().silu_mul(whole.to(DEV))
-    got = ops().silu_mul(parts.to(DEV), out_dtype=torch.bfloat16)
-    assert torch.equal(got.cpu(), want.cpu())
-
+    """Rotary + cache write over K-split slices equals the stored-projection form applied to
+    the rounded sum."""
     n_q, n_kv, d, page = 6, 2, 32, 16
     width = (n_q + 2 * n_kv) * d
     parts = rnd(4, 5, width, seed=28)
