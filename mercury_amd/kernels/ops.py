@@ -26,8 +26,30 @@ def dtype_code(dtype: torch.dtype) -> int:
         raise KernelArgumentError(f"kernels take float32 or bfloat16 tensors, not {dtype}") from None
 
 
+_pinned_stream: int | None = None
+
+
 def _stream() -> int:
+    if _pinned_stream is not None:
+        return _pinned_stream
     return torch.cuda.current_stream().cuda_stream
+
+
+class on_current_stream:
+    """Within this context every kernel here goes to the stream that was current at its entry,
+    looked up once instead of at every launch (the lookup costs as much as a launch).  Not to
+    be held across a change of the current stream, such as entering a graph capture."""
+
+    def __enter__(self):
+        global _pinned_stream
+        self.before = _pinned_stream
+        _pinned_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _pinned_stream
+        _pinned_stream = self.before
+        return False
 
 
 def _dev(*tensors) -> None:

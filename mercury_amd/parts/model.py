@@ -129,12 +129,13 @@ class DecoderModel(Part):
 
         caches: execution-list index -> LayerCache; states: layer index -> state tensor.
         """
-        h = ops.embed(step.token_ids, self.embedding)
-        pending = None
-        for n, call in enumerate(self.calls):
-            pending = self.layers[call.layer].forward(h, step, caches.get(n),
-                                                      states.get(call.layer), self.dtype, pending)
-        if step.num_logit_rows == 0:
-            return torch.empty((0, self.vocab_size), dtype=torch.float32, device=h.device)
-        x = self.final_norm.forward(h, self.dtype, rows=step.logit_rows, partials=pending)
-        return ops.linear(x, self.head, out_dtype=torch.float32)
+        with ops.on_current_stream():
+            h = ops.embed(step.token_ids, self.embedding)
+            pending = None
+            for n, call in enumerate(self.calls):
+                pending = self.layers[call.layer].forward(
+                    h, step, caches.get(n), states.get(call.layer), self.dtype, pending)
+            if step.num_logit_rows == 0:
+                return torch.empty((0, self.vocab_size), dtype=torch.float32, device=h.device)
+            x = self.final_norm.forward(h, self.dtype, rows=step.logit_rows, partials=pending)
+            return ops.linear(x, self.head, out_dtype=torch.float32)
