@@ -14,11 +14,11 @@
 //    consumes the projection (RMSNorm, rotary + cache write) adds the slices up in slice
 //    order, so results are reproducible.
 //
-//  * tiled (M > 64, prompts): tiles of y per workgroup of four wavefronts (128 x 128, or
-//    smaller when the matrix would otherwise leave compute units idle), K in stages through
-//    two LDS buffers with the next stage's global loads in flight during the current stage's
-//    products.  Epilogues: bfloat16 store with bias, float32 store, or float32 accumulate
-//    into the residual stream.
+//  * tiled (M > 64, prompts): tiles of y per workgroup (256 x 256 down to 64 x 64, whichever
+//    is estimated fastest for the problem), K in stages through a ring of LDS buffers that
+//    global memory is loaded into directly, several stages ahead of the products.
+//    Epilogues: bfloat16 store with bias, float32 store, float32 accumulate into the
+//    residual stream, or SiLU gating.
 //
 // In both, lane l of a wavefront holds row (l % 16) and k-slots (l / 16) * 8 .. + 8 of an
 // operand, so the four lanes of a row read 64 contiguous bytes per load instruction.
@@ -478,39 +478,63 @@ extern "C" int mk_qkv_skinny(const void* x, const void* w, const void* bias, int
 
 enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3 };
 
-// One workgroup of 4 wavefronts (WM x WN) computes a BM x BN tile of y; K advances TK per
-// stage through two LDS buffers, the next stage's global loads in flight during the current
-// stage's products.  The 16-byte chunks of a tile row are permuted in LDS (or the row padded)
-// so that operand reads of 16 rows and staging writes of 2 rows hit distinct banks.
-// EPI_GATED: W is [gate rows | up rows] of N each; a tile holds BN / 2 gate rows and the BN / 2
-// matching up rows, every wavefront spans the tile's whole width (WN = 1), and the epilogue
-// writes act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
-template <int BM, int BN, int TK, int WM, int WN, int EPI, typename TBIAS>
-__global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
-                                                         const bf16_t* __restrict__ w,
-                                                         const TBIAS* __restrict__ bias,
-                                                         void* __restrict__ out_, int M, int N,
-                                                         int K, int ldo) {
-  static_assert(WM * WN == 4, "four wavefronts");
-  static_assert(EPI != EPI_GATED || WN == 1, "gating needs both halves in one wavefront");
-  constexpr bool SWIZZLED = TK == 64;
-  constexpr int LD = SWIZZLED ? TK : TK + 8;
-  // Where the 8 elements from k (a multiple of 8) of a tile row lie in LDS.  Rows of 64
-  // elements are 128 bytes, half the banks; the 16-byte chunks of a row are permuted by the
-  // row pair's index, so that the 16 rows one operand read touches hit 16 different bank
-  // groups, as do the two rows a staging write fills.  Other widths pad the row instead.
-  auto lds_at = [](int row, int k) {
-    return SWIZZLED ? row * LD + ((((k >> 3) ^ (row >> 1)) & 7) << 3) : row * LD + k;
-  };
+#define TILE_K 64  // k per stage: a tile row is 128 bytes in LDS, one cache line of the operand
+
+// Sixteen zero bytes: what a lane fetches for k past K, so that a last, partial stage
+// multiplies zeros.
+__device__ __attribute__((aligned(16))) const unsigned int tiled_zero_chunk[4] = {0u, 0u, 0u, 0u};
+
+// The LDS buffer of stage S of the ring: x rows first, then W rows.  Static buffers, one per
+// stage and instantiation.
+template <int S, int ELEMS>
+__device__ __forceinline__ bf16_t* tiled_stage_buffer() {
+  __shared__ __attribute__((aligned(1024))) bf16_t buffer[ELEMS];
+  return buffer;
+}
+
+// s_waitcnt immediate: at most `loads` vector-memory loads outstanding, every LDS operation
+// complete (vmcnt is split over bits 3:0 and 15:14, lgkmcnt is bits 11:8, expcnt 6:4 unused).
+#define TILED_WAIT(loads) (((loads) & 15) | (((loads) >> 4) << 14) | (7 << 4) | (0 << 8))
+
+// One workgroup of WM x WN wavefronts computes a BM x BN tile of y.  K advances 64 per stage
+// through a ring of STAGES LDS buffers.  The tiles travel from global memory straight into
+// LDS (global_load_lds_dwordx4: each lane's 16 bytes land at M0 + 16 * lane, no register in
+// between), so a stage's loads can be asked for STAGES - 1 stages before they are used at no
+// cost in registers: the latency of a load under full traffic is more than a stage's worth
+// of products.  One wavefront instruction fills 8 tile rows; which 16 bytes of its row a
+// lane fetches is permuted by the row pair's index, so that the operand reads of 16 rows hit
+// 16 different bank groups.  Per stage: wait until this wavefront's loads of the stage have
+// landed, barrier (now everybody's have, and everybody is done with the previous stage's
+// buffer), ask for the stage STAGES - 1 ahead into that buffer, multiply.
+//
+// The loads are inline assembly: the compiler counts its own vector-memory operations only
+// (there are none inside the loop), and the waits for these are written out by hand.
+//
+// EPI_GATED: W is [gate rows | up rows] of N each.  A wavefront's BN / WN tile rows are half
+// gate rows and half the matching up rows, so its accumulators hold both; the epilogue writes
+// act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
+template <int BM, int BN, int STAGES, int WM, int WN, int EPI, typename TBIAS>
+__global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
+                                                                  const bf16_t* __restrict__ w,
+                                                                  const TBIAS* __restrict__ bias,
+                                                                  void* __restrict__ out_, int M,
+                                                                  int N, int K, int ldo) {
+  constexpr int WAVES = WM * WN, TK = TILE_K;
+  constexpr int NI = (BM + BN) / 8 / WAVES;                 // load instructions per wavefront and stage
+  static_assert((BM + BN) % (8 * WAVES) == 0 && WAVES % 2 == 0, "tile rows divide over the wavefronts");
+  static_assert(BM % 16 == 0 && (STAGES - 2) * NI < 64, "tile shape");
+  constexpr int ELEMS = (BM + BN) * TK;
   constexpr int TM = BM / WM / 16, TN = BN / WN / 16;       // MFMA tiles per wavefront
-  constexpr int CHUNKS_ROW = TK / 8;                        // 16-byte chunks per tile row
-  constexpr int XCH = BM * CHUNKS_ROW / 256, WCH = BN * CHUNKS_ROW / 256;  // per thread
-  static_assert(XCH >= 1 && WCH >= 1, "tile too small for 256 threads");
-  __shared__ __attribute__((aligned(16))) bf16_t xs[2][BM * LD];
-  __shared__ __attribute__((aligned(16))) bf16_t ws[2][BN * LD];
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  static_assert(EPI != EPI_GATED || TN % 2 == 0, "gating needs gate and up tiles in one wavefront");
+  constexpr int WIDTH = BN / WN;                            // W rows per wavefront
+  constexpr int COLS = EPI == EPI_GATED ? BN / 2 : BN;      // output columns per tile
+  // Where the 8 elements from k-chunk `chunk` of tile row `row` lie in a stage buffer.
+  auto lds_at = [](int row, int chunk) { return row * TK + (((chunk ^ (row >> 1)) & 7) << 3); };
+
+  const int tid = threadIdx.x, lane = tid & 63;
+  const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int r = lane & 15, g4 = lane >> 4;
-  const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * (BN / WN);
+  const int wm = (wave / WN) * (BM / WM), wn = (wave % WN) * WIDTH;
   // Which tile: workgroups go to the 8 XCDs in turn, each with an L2 of its own, so the
   // launch index is first renumbered to give every XCD a contiguous stretch of tiles, and the
   // stretch is walked in bands of 8 tile rows, column by column, so that the tiles in flight
@@ -528,28 +552,33 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     tile_m = first + in_band % height;
     tile_n = in_band / height;
   }
-  const int m0 = tile_m * BM, n0 = tile_n * (EPI == EPI_GATED ? BN / 2 : BN);
+  const int m0 = tile_m * BM, n0 = tile_n * COLS;
 
-  // Staging: thread t moves chunk t, t + 256, ... of each operand's tile.
-  const bf16_t* xg[XCH];
-  const bf16_t* wg[WCH];
-  int xo[XCH], wo[WCH];
-  const int sk = (tid % CHUNKS_ROW) * 8;
+  // Load instruction i of this wavefront fills buffer rows [8 j, 8 j + 8), j = wave + WAVES i;
+  // lane l lands on chunk l % 8 of row 8 j + l / 8, and fetches the k-chunk that belongs
+  // there.  (row >> 1) & 7 = (4 j + l / 16) & 7 has the same value for every i, WAVES being
+  // even, and so has the k-chunk.
+  const int chunk = ((lane & 7) ^ (4 * wave + (lane >> 4))) & 7;
+  const bf16_t* src[NI];
 #pragma unroll
-  for (int i = 0; i < XCH; ++i) {
-    const int row = (tid + i * 256) / CHUNKS_ROW;
-    xg[i] = x + (size_t)min(m0 + row, M - 1) * K + sk;
-    xo[i] = lds_at(row, sk);
+  for (int i = 0; i < NI; ++i) {
+    const int row = (wave + WAVES * i) * 8 + (lane >> 3);
+    if (row < BM) {
+      src[i] = x + (size_t)min(m0 + row, M - 1) * K + chunk * 8;
+    } else {
+      int wrow = row - BM;
+      if (EPI == EPI_GATED) {  // per wavefront: WIDTH / 2 gate rows, then the matching up rows
+        const int col = min(n0 + wrow / WIDTH * (WIDTH / 2) + wrow % (WIDTH / 2), N - 1);
+        wrow = (wrow % WIDTH < WIDTH / 2 ? 0 : N) + col;
+      } else {
+        wrow = min(n0 + wrow, N - 1);
+      }
+      src[i] = w + (size_t)wrow * K + chunk * 8;
+    }
   }
-#pragma unroll
-  for (int i = 0; i < WCH; ++i) {
-    const int row = (tid + i * 256) / CHUNKS_ROW;
-    int wrow = min(n0 + row, N - 1);
-    if (EPI == EPI_GATED)  // tile rows [0, BN/2) are gate rows, [BN/2, BN) the matching up rows
-      wrow = row < BN / 2 ? min(n0 + row, N - 1) : N + min(n0 + row - BN / 2, N - 1);
-    wg[i] = w + (size_t)wrow * K + sk;
-    wo[i] = lds_at(row, sk);
-  }
+  const int steps = (K + TK - 1) / TK;
+  const bool ragged = K % TK != 0;
+  const bool past_k = (steps - 1) * TK + chunk * 8 >= K;    // this lane's part of a partial last stage
 
   f32x4 acc[TM][TN];
 #pragma unroll
@@ -557,37 +586,35 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
 #pragma unroll
     for (int b = 0; b < TN; ++b) acc[a][b] = (f32x4){0.f, 0.f, 0.f, 0.f};
 
-  // A stage's loads are asked for one or two stages before it is needed, into registers (the
-  // latency of a load is several stages' worth of products), and parked in LDS one stage
-  // before.
-  struct Staged {
-    uint4 x[XCH], w[WCH];
+  // Stages past the last are asked for as the last one again: they land in buffers nobody
+  // reads any more, and every iteration has the same number of loads to count.
+  auto fetch = [&](int s, bf16_t* buffer) __attribute__((always_inline)) {
+    const int stage = min(s, steps - 1);
+    const bool partial = ragged && stage == steps - 1;      // the same for the whole workgroup
+#pragma unroll
+    for (int i = 0; i < NI; ++i) {
+      const unsigned int dst = (unsigned int)(uintptr_t)(
+          __attribute__((address_space(3))) void*)(buffer + (wave + WAVES * i) * 512);
+      const bf16_t* from = src[i] + stage * TK;
+      if (partial) from = past_k ? (const bf16_t*)tiled_zero_chunk : from;
+      asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
+                   :
+                   : "s"(dst), "v"(from)
+                   : "memory");
+    }
   };
-  auto fetch = [&](int k0) __attribute__((always_inline)) {
-    Staged r;
-    const bool ok = k0 + sk < K;
-#pragma unroll
-    for (int i = 0; i < XCH; ++i) r.x[i] = ok ? ld16(xg[i] + k0) : make_uint4(0, 0, 0, 0);
-#pragma unroll
-    for (int i = 0; i < WCH; ++i) r.w[i] = ok ? ld16(wg[i] + k0) : make_uint4(0, 0, 0, 0);
-    return r;
-  };
-  auto stash = [&](const Staged& r, int buf) __attribute__((always_inline)) {
-#pragma unroll
-    for (int i = 0; i < XCH; ++i) *(uint4*)(&xs[buf][xo[i]]) = r.x[i];
-#pragma unroll
-    for (int i = 0; i < WCH; ++i) *(uint4*)(&ws[buf][wo[i]]) = r.w[i];
-  };
-  auto products = [&](int buf) __attribute__((always_inline)) {
+  auto products = [&](const bf16_t* buffer) __attribute__((always_inline)) {
+    const bf16_t* xs = buffer;
+    const bf16_t* ws = buffer + BM * TK;
 #pragma unroll
     for (int kk = 0; kk < TK; kk += 32) {
       Frag a[TM], b[TN];
 #pragma unroll
       for (int t = 0; t < TM; ++t)
-        a[t].u = *(const uint4*)(&xs[buf][lds_at(wm + t * 16 + r, kk + g4 * 8)]);
+        a[t].u = *(const uint4*)(&xs[lds_at(wm + t * 16 + r, kk / 8 + g4)]);
 #pragma unroll
       for (int t = 0; t < TN; ++t)
-        b[t].u = *(const uint4*)(&ws[buf][lds_at(wn + t * 16 + r, kk + g4 * 8)]);
+        b[t].u = *(const uint4*)(&ws[lds_at(wn + t * 16 + r, kk / 8 + g4)]);
 #pragma unroll
       for (int ta = 0; ta < TM; ++ta)
 #pragma unroll
@@ -598,41 +625,30 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     }
   };
 
-  const int steps = (K + TK - 1) / TK;
-  // Small tiles have the registers for a second set in flight (the loop is unrolled by two so
-  // that no set is ever copied: a copy would wait for its loads); the 128 x 128 tile would
-  // lose its second workgroup per compute unit to it, and asks one stage ahead only.
-  constexpr bool TWO_AHEAD = BM * BN <= 64 * 128;
-  Staged even = fetch(0);
-  stash(even, 0);
-  if constexpr (TWO_AHEAD) {
-    Staged odd = fetch(TK);          // past K: zeros, never parked
-    even = fetch(2 * TK);
-    __syncthreads();
-    for (int s = 0; s < steps; s += 2) {
-      products(0);
-      if (s + 1 < steps) stash(odd, 1);
-      odd = fetch((s + 3) * TK);
-      __syncthreads();
-      if (s + 1 < steps) {
-        products(1);
-        if (s + 2 < steps) stash(even, 0);
-        even = fetch((s + 4) * TK);
-        __syncthreads();
+  bf16_t* ring[STAGES];
+  ring[0] = tiled_stage_buffer<0, ELEMS>();
+  ring[1] = tiled_stage_buffer<1, ELEMS>();
+  if constexpr (STAGES > 2) ring[2] = tiled_stage_buffer<2, ELEMS>();
+  if constexpr (STAGES > 3) ring[3] = tiled_stage_buffer<3, ELEMS>();
+  static_assert(STAGES >= 2 && STAGES <= 4, "two to four stages");
+
+#pragma unroll
+  for (int s = 0; s < STAGES - 1; ++s) fetch(s, ring[s]);
+  for (int s0 = 0; s0 < steps; s0 += STAGES) {
+#pragma unroll
+    for (int u = 0; u < STAGES; ++u) {   // unrolled: every buffer of the ring is a constant
+      if (s0 + u < steps) {
+        asm volatile("" ::: "memory");
+        __builtin_amdgcn_s_waitcnt(TILED_WAIT((STAGES - 2) * NI));
+        __builtin_amdgcn_s_barrier();
+        asm volatile("" ::: "memory");
+        fetch(s0 + u + STAGES - 1, ring[(u + STAGES - 1) % STAGES]);
+        products(ring[u]);
       }
-    }
-  } else {
-    __syncthreads();
-    for (int s = 0; s < steps; ++s) {   // not unrolled: the loop body's registers are the limit
-      const int buf = s & 1;
-      if (s + 1 < steps) even = fetch((s + 1) * TK);
-      products(buf);
-      if (s + 1 < steps) stash(even, buf ^ 1);
-      __syncthreads();
     }
   }
 
-  // acc[ta][tb][i] = y[m = m0 + wm + ta*16 + r][n = n0 + wn + tb*16 + g4*4 + i]
+  // acc[ta][tb][i] = y[m = m0 + wm + ta*16 + r][tile column wn + tb*16 + g4*4 + i]
 #pragma unroll
   for (int ta = 0; ta < TM; ++ta) {
     const int m = m0 + wm + ta * 16 + r;
@@ -640,7 +656,7 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
     if (EPI == EPI_GATED) {
 #pragma unroll
       for (int tb = 0; tb < TN / 2; ++tb) {
-        const int n = n0 + tb * 16 + g4 * 4;
+        const int n = n0 + wn / 2 + tb * 16 + g4 * 4;
         bf16_t* dst = (bf16_t*)out_ + (size_t)m * ldo + n;
         float o[4];
 #pragma unroll
@@ -700,51 +716,97 @@ __global__ __launch_bounds__(256) void gemm_tiled_kernel(const bf16_t* __restric
   }
 }
 
-template <int BM, int BN, int TK, int WM, int WN, int EPI>
+// Tile configurations, by index.  `rate` is what one workgroup sustains on a busy chip in
+// TFLOP/s, `alone` what it sustains with a compute unit to itself, `resident` how many
+// workgroups a compute unit holds (LDS decides); measured on problems of many tiles.
+struct TiledConfig {
+  int bm, bn, resident;
+  float rate, alone;
+};
+#define TILED_CONFIGS 6
+static const TiledConfig tiled_configs[TILED_CONFIGS] = {
+    {256, 256, 1, 5.3f, 5.3f},   // 0: 2 stages (128 KB), 8 wavefronts
+    {128, 256, 1, 5.0f, 5.0f},   // 1: 3 stages (144 KB), 8 wavefronts
+    {128, 128, 1, 4.2f, 4.2f},   // 2: 3 stages (96 KB), 8 wavefronts
+    {128, 128, 2, 2.18f, 3.7f},  // 3: 2 stages (64 KB), 4 wavefronts
+    {64, 64, 2, 1.3f, 2.2f},     // 4: 4 stages (64 KB), 4 wavefronts
+    {64, 128, 1, 2.15f, 2.15f},  // 5: 4 stages (96 KB), 4 wavefronts
+};
+
+template <int BM, int BN, int STAGES, int WM, int WN, int EPI>
 static void launch_tiled_cfg(const void* x, const void* w, const void* bias, int bias_dtype,
                              void* out, int M, int N, int K, int ldo, hipStream_t stream) {
-  dim3 grid((N + BN - 1) / BN, (M + BM - 1) / BM);
+  constexpr int COLS = EPI == EPI_GATED ? BN / 2 : BN;
+  dim3 grid((N + COLS - 1) / COLS, (M + BM - 1) / BM);
   if (bias && bias_dtype == MK_BF16)
-    gemm_tiled_kernel<BM, BN, TK, WM, WN, EPI, bf16_t><<<grid, 256, 0, stream>>>(
+    gemm_tiled_kernel<BM, BN, STAGES, WM, WN, EPI, bf16_t><<<grid, 64 * WM * WN, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, out, M, N, K, ldo);
   else
-    gemm_tiled_kernel<BM, BN, TK, WM, WN, EPI, float><<<grid, 256, 0, stream>>>(
+    gemm_tiled_kernel<BM, BN, STAGES, WM, WN, EPI, float><<<grid, 64 * WM * WN, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo);
 }
-
-// Tile configurations, by index: 0 = 128x128, 1 = 64x128, 2 = 64x64 (k in stages of 64).
-#define TILED_CONFIGS 3
 
 template <int EPI>
 static void launch_tiled(int config, const void* x, const void* w, const void* bias,
                          int bias_dtype, void* out, int M, int N, int K, int ldo,
                          hipStream_t stream) {
   switch (config) {
-    case 0: launch_tiled_cfg<128, 128, 64, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 1: launch_tiled_cfg<64, 128, 64, 1, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    default: launch_tiled_cfg<64, 64, 64, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 0: launch_tiled_cfg<256, 256, 2, 2, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 1: launch_tiled_cfg<128, 256, 3, 2, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 2: launch_tiled_cfg<128, 128, 3, 2, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 3: launch_tiled_cfg<128, 128, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 4: launch_tiled_cfg<64, 64, 4, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    default: launch_tiled_cfg<64, 128, 4, 1, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
   }
 }
 
-// 128 x 128 tiles when they give every compute unit a workgroup, else 64 x 64 (measured:
-// 2048 x 3584 x 18944 runs a quarter faster in 448 large tiles than in 1792 small ones,
-// 2048 x 896 x 4864 a quarter slower in 112 large tiles than in 448 small ones).
-// At most 64 rows: 64 x 128 tiles, no half of a tile idle.
-extern "C" int mk_linear_tiled_config(int M, int N, int K) {
-  if (M <= 64) return 1;
-  const long groups = (long)((M + 127) / 128) * ((N + 127) / 128);
-  return groups >= 256 ? 0 : 2;
+// The configuration with the least estimated time for y[M, cols] over K.  A tile covers
+// `bn / halves` columns (halves = 2 when gate and up rows share a tile) and moves `out_bytes`
+// per element in its epilogue.  Tiles are dealt to the 256 compute units; a tile costs its
+// products at the configuration's rate plus a start (the first loads' latency) and a finish
+// (the epilogue, at what one workgroup streams: about 35 GB/s); of two resident workgroups
+// one's start and finish hide behind the other's products, and an odd last one runs alone.
+static int tiled_config_for(int M, int cols, int K, int halves, int out_bytes) {
+  int best = -1;
+  double best_time = 0.0;
+  for (int c = 0; c < TILED_CONFIGS; ++c) {
+    const TiledConfig& t = tiled_configs[c];
+    if (M <= 64 && t.bm > 64) continue;
+    const int width = t.bn / halves;
+    const long tiles = (long)((M + t.bm - 1) / t.bm) * ((cols + width - 1) / width);
+    const bool few = tiles <= 4 * 256;
+    const double per_unit = few ? (double)((tiles + 255) / 256) : tiles / 256.0 + 0.5;
+    const double products = 2.0 * t.bm * t.bn * K * 1e-6;            // MFLOP
+    const double edges = 1.5 + (double)t.bm * width * out_bytes / 35e3;  // microseconds
+    double time;
+    if (t.resident == 1) {
+      time = per_unit * (products / t.rate + edges);
+    } else if (few) {
+      const long n = (long)per_unit;
+      time = (n / 2) * (products / t.rate + edges / 2) + (n % 2) * (products / t.alone + edges);
+    } else {
+      time = per_unit / 2 * (products / t.rate + edges / 2);
+    }
+    if (best < 0 || time < best_time) best = c, best_time = time;
+  }
+  return best;
+}
+
+extern "C" int mk_linear_tiled_configs(void) { return TILED_CONFIGS; }
+
+extern "C" int mk_linear_tiled_config(int M, int N, int K, int out_bytes) {
+  return tiled_config_for(M, N, K, 1, out_bytes);
 }
 
 // act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K].
 extern "C" int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K,
-                              hipStream_t stream) {
+                              int config, hipStream_t stream) {
   MK_REQUIRE(M > 0 && inter > 0 && K > 0 && K % 8 == 0,
              "gated projection: K=%d must be a multiple of 8 (M=%d I=%d)", K, M, inter);
-  MK_REQUIRE((M + 127) / 128 <= 65535, "gated projection: M=%d too large for one launch", M);
-  dim3 grid((inter + 63) / 64, (M + 127) / 128);
-  gemm_tiled_kernel<128, 128, 64, 4, 1, EPI_GATED, float><<<grid, 256, 0, stream>>>(
-      (const bf16_t*)x, (const bf16_t*)w, (const float*)nullptr, act, M, inter, K, inter);
+  MK_REQUIRE((M + 63) / 64 <= 65535, "gated projection: M=%d too large for one launch", M);
+  if (config < 0) config = tiled_config_for(M, inter, K, 2, 2);
+  MK_REQUIRE(config < TILED_CONFIGS, "gated projection: no configuration %d", config);
+  launch_tiled<EPI_GATED>(config, x, w, nullptr, MK_F32, act, M, inter, K, inter, stream);
   MK_LAUNCH_CHECK("gated_tiled");
   return 0;
 }
@@ -758,7 +820,8 @@ extern "C" int mk_linear_tiled(const void* x, const void* w, const void* bias, i
   MK_REQUIRE(!accumulate || out_dtype == MK_F32,
              "tiled projection: accumulation needs a float32 destination");
   MK_REQUIRE((M + 63) / 64 <= 65535, "tiled projection: M=%d too large for one launch", M);
-  if (config < 0) config = mk_linear_tiled_config(M, N, K);
+  if (config < 0)
+    config = mk_linear_tiled_config(M, N, K, accumulate ? 8 : (out_dtype == MK_F32 ? 4 : 2));
   MK_REQUIRE(config < TILED_CONFIGS, "tiled projection: no configuration %d", config);
   if (accumulate)
     launch_tiled<EPI_ACC>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, stream);

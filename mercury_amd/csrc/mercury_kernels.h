@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 4
+#define MK_ABI_VERSION 5
 
 #ifdef __cplusplus
 extern "C" {
@@ -90,14 +90,17 @@ int mk_qkv_skinny(const void* x, const void* w, const void* bias, int bias_dtype
                   int table_stride, void* k_cache, void* v_cache, int page_size, int n_q,
                   int n_kv, int d, int rotate, int M, int K, hipStream_t stream);
 
-// The same for any M, tiled through LDS.
-int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K,
+// The same for any M, tiled through LDS; config: a tile configuration, -1 for the one
+// estimated fastest.
+int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K, int config,
                    hipStream_t stream);
 
 // y = x W^T (+ bias) for any M, tiled through LDS; output bfloat16 or float32, or float32
-// accumulated into `out`.  config: a tile configuration (mk_linear_tiled_config picks one for
-// the shape; -1 does the same).
-int mk_linear_tiled_config(int M, int N, int K);
+// accumulated into `out`.  config: a tile configuration, 0 .. mk_linear_tiled_configs() - 1
+// (mk_linear_tiled_config picks the one estimated fastest for the shape and the bytes the
+// epilogue moves per element of y; -1 does the same).
+int mk_linear_tiled_configs(void);
+int mk_linear_tiled_config(int M, int N, int K, int out_bytes);
 int mk_linear_tiled(const void* x, const void* w, const void* bias, int bias_dtype, void* out,
                     int out_dtype, int accumulate, int M, int N, int K, int ldo, int config,
                     hipStream_t stream);

@@ -187,10 +187,12 @@ def fuses_gating(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
             and x.shape[0] > 0 and x.shape[1] % 8 == 0 and w_gate_up.shape[0] % 2 == 0)
 
 
-def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
+def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor,
+                     tile_config: int | None = None) -> torch.Tensor:
     """act = silu(x Wg^T) * (x Wu^T) for bfloat16 x and W = [Wg | Wu] stacked [2 I, K]: one
     kernel on the matrix cores, the gating in the projection's epilogue (the skinny kernel for
-    few rows, the tiled one for many)."""
+    few rows, the tiled one for many; `tile_config` forces the tiled one with that tile
+    configuration, -1 for its own choice)."""
     _dev(x, w_gate_up)
     if not fuses_gating(x, w_gate_up) or x.shape[1] != w_gate_up.shape[1]:
         raise KernelArgumentError("gated_projection: operands not eligible")
@@ -202,9 +204,12 @@ def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor) -> torch.Tensor:
     # re-reads (measured at 18944 x 3584: 75 against 85 to 112 us)
     skinny = m <= SKINNY_MAX_ROWS and not (m >= GATED_TILED_MIN_ROWS
                                            and inter * k >= GATED_TILED_MIN_WEIGHTS)
-    fn = lib.mk_gated_skinny if skinny else lib.mk_gated_tiled
-    _lib.check(lib, fn(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream()),
-               "gated_projection")
+    if skinny and tile_config is None:
+        code = lib.mk_gated_skinny(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream())
+    else:
+        code = lib.mk_gated_tiled(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k,
+                                  -1 if tile_config is None else tile_config, _stream())
+    _lib.check(lib, code, "gated_projection")
     return act
 
 

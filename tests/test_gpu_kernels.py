@@ -192,6 +192,43 @@ def test_gated_projection(m, inter, k):
     torch.testing.assert_close(got.float().cpu(), plain_want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("m,n,k", [(300, 520, 200), (257, 130, 64), (70, 1004, 1096), (513, 264, 8)])
+def test_every_tile_configuration(m, n, k):
+    """Each tile shape of the tiled projection, forced, at sizes that leave partial tiles in
+    both directions and a partial last stage of K: every epilogue, and the gated form with
+    gate and up rows interleaved per wavefront."""
+    lib = ops()._lib.load("mfma")
+    x_h, x_d = as_dtype(rnd(m, k, seed=27), torch.bfloat16)
+    w_h, w_d = as_dtype(rnd(n, k, seed=28, scale=0.1), torch.bfloat16)
+    b_h, b_d = as_dtype(rnd(n, seed=29), torch.bfloat16)
+    want = (x_h.double() @ w_h.double().T).float()
+    inter = n // 2
+    stored = want.to(torch.bfloat16)
+    gated_want = ops().silu_mul(stored.to(DEV)).float().cpu()
+    acc = rnd(m, n, seed=30)
+    for config in range(lib.mk_linear_tiled_configs()):
+        got = ops().linear(x_d, w_d, b_d, kernel="mfma", tile_config=config)
+        torch.testing.assert_close(got.float().cpu(), want + b_h, **tol(torch.bfloat16))
+        got32 = ops().linear(x_d, w_d, out_dtype=torch.float32, kernel="mfma", tile_config=config)
+        torch.testing.assert_close(got32.cpu(), want, atol=5e-4, rtol=1e-4)
+        acc_d = acc.clone().to(DEV)
+        ops().linear(x_d, w_d, out=acc_d, accumulate=True, kernel="mfma", tile_config=config)
+        torch.testing.assert_close(acc_d.cpu(), acc + want, atol=5e-4, rtol=1e-4)
+        gated = ops().gated_projection(x_d, w_d, tile_config=config)
+        assert gated.shape == (m, inter)
+        torch.testing.assert_close(gated.float().cpu(), gated_want, atol=2e-3, rtol=1.6e-2)
+
+
+def test_the_tile_configuration_follows_the_problem():
+    """Large tiles where they fill the chip, small ones where large ones would leave compute
+    units idle, and at most 64 tile rows for at most 64 rows of x."""
+    lib = ops()._lib.load("mfma")
+    assert lib.mk_linear_tiled_config(8192, 8192, 8192, 2) == 0        # 256 x 256
+    assert lib.mk_linear_tiled_config(2048, 896, 4864, 8) == 4         # 64 x 64: 448 tiles
+    assert lib.mk_linear_tiled_config(2048, 3584, 18944, 8) == 1       # 128 x 256: 224 tiles
+    assert lib.mk_linear_tiled_config(40, 151936, 896, 4) in (4, 5)
+
+
 def test_which_skinny_projections_are_split():
     """K is split into partial sums only where the matrix is large and has too few rows to
     occupy the chip with 16-row workgroups."""
