@@ -718,19 +718,20 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
 
 // Tile configurations, by index.  `rate` is what one workgroup sustains on a busy chip in
 // TFLOP/s, `alone` what it sustains with a compute unit to itself, `resident` how many
-// workgroups a compute unit holds (LDS decides); measured on problems of many tiles.
+// workgroups a compute unit holds (LDS decides); measured on problems of many tiles with
+// weights that no cache holds, as a model's are.
 struct TiledConfig {
   int bm, bn, resident;
   float rate, alone;
 };
 #define TILED_CONFIGS 6
 static const TiledConfig tiled_configs[TILED_CONFIGS] = {
-    {256, 256, 1, 5.3f, 5.3f},   // 0: 2 stages (128 KB), 8 wavefronts
-    {128, 256, 1, 5.0f, 5.0f},   // 1: 3 stages (144 KB), 8 wavefronts
-    {128, 128, 1, 4.2f, 4.2f},   // 2: 3 stages (96 KB), 8 wavefronts
-    {128, 128, 2, 2.18f, 3.7f},  // 3: 2 stages (64 KB), 4 wavefronts
-    {64, 64, 2, 1.3f, 2.2f},     // 4: 4 stages (64 KB), 4 wavefronts
-    {64, 128, 1, 2.15f, 2.15f},  // 5: 4 stages (96 KB), 4 wavefronts
+    {256, 256, 1, 4.9f, 4.9f},    // 0: 2 stages (128 KB), 8 wavefronts
+    {128, 256, 1, 4.27f, 4.27f},  // 1: 3 stages (144 KB), 8 wavefronts
+    {128, 128, 1, 3.6f, 3.6f},    // 2: 3 stages (96 KB), 8 wavefronts
+    {128, 128, 2, 2.02f, 2.8f},   // 3: 2 stages (64 KB), 4 wavefronts
+    {64, 64, 2, 1.15f, 1.95f},    // 4: 4 stages (64 KB), 4 wavefronts
+    {64, 128, 1, 2.14f, 2.14f},   // 5: 4 stages (96 KB), 4 wavefronts
 };
 
 template <int BM, int BN, int STAGES, int WM, int WN, int EPI>
