@@ -505,15 +505,17 @@ __device__ __forceinline__ bf16_t* tiled_stage_buffer() {
 // lane fetches is permuted by the row pair's index, so that the operand reads of 16 rows hit
 // 16 different bank groups.  Per stage: wait until this wavefront's loads of the stage have
 // landed, barrier (now everybody's have, and everybody is done with the previous stage's
-// buffer), ask for the stage STAGES - 1 ahead into that buffer, multiply.
+// buffer), ask for the stage STAGES - 1 ahead into that buffer while multiplying.
 //
 // The loads are inline assembly: the compiler counts its own vector-memory operations only
-// (there are none inside the loop), and the waits for these are written out by hand.
+// (there are none inside the loop), and the waits for these are written out by hand.  The
+// compiler may move LDS reads past a load but not past the barrier, which is fenced: a load
+// writes the buffer whose reads ended before the barrier.
 //
 // EPI_GATED: W is [gate rows | up rows] of N each.  A wavefront's BN / WN tile rows are half
 // gate rows and half the matching up rows, so its accumulators hold both; the epilogue writes
 // act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
-template <int BM, int BN, int STAGES, int WM, int WN, int EPI, typename TBIAS>
+template <int BM, int BN, int STAGES, int WM, int WN, int SPREAD, int EPI, typename TBIAS>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
                                                                   const bf16_t* __restrict__ w,
                                                                   const TBIAS* __restrict__ bias,
@@ -588,26 +590,32 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
 
   // Stages past the last are asked for as the last one again: they land in buffers nobody
   // reads any more, and every iteration has the same number of loads to count.
-  auto fetch = [&](int s, bf16_t* buffer) __attribute__((always_inline)) {
+  // Load instructions [first, last) of stage s.
+  auto fetch = [&](int s, bf16_t* buffer, int first, int last) __attribute__((always_inline)) {
     const int stage = min(s, steps - 1);
     const bool partial = ragged && stage == steps - 1;      // the same for the whole workgroup
 #pragma unroll
-    for (int i = 0; i < NI; ++i) {
+    for (int i = first; i < last; ++i) {
       const unsigned int dst = (unsigned int)(uintptr_t)(
           __attribute__((address_space(3))) void*)(buffer + (wave + WAVES * i) * 512);
       const bf16_t* from = src[i] + stage * TK;
       if (partial) from = past_k ? (const bf16_t*)tiled_zero_chunk : from;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                    :
-                   : "s"(dst), "v"(from)
-                   : "memory");
+                   : "s"(dst), "v"(from));
     }
   };
-  auto products = [&](const bf16_t* buffer) __attribute__((always_inline)) {
+  // The products of a stage, with the loads of stage `ahead` handed out between them: all up
+  // front (SPREAD 0), half before each half of k (1), or a few before every row of MFMA
+  // tiles (2).  Requests that arrive in one burst per stage take longer to be served.
+  auto products = [&](const bf16_t* buffer, int ahead, bf16_t* into) __attribute__((always_inline)) {
     const bf16_t* xs = buffer;
     const bf16_t* ws = buffer + BM * TK;
+    constexpr int HALVES = TK / 32, SLOTS = HALVES * TM;
+    if (SPREAD == 0) fetch(ahead, into, 0, NI);
 #pragma unroll
     for (int kk = 0; kk < TK; kk += 32) {
+      if (SPREAD == 1) fetch(ahead, into, kk / 32 * NI / HALVES, (kk / 32 + 1) * NI / HALVES);
       Frag a[TM], b[TN];
 #pragma unroll
       for (int t = 0; t < TM; ++t)
@@ -616,12 +624,15 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
       for (int t = 0; t < TN; ++t)
         b[t].u = *(const uint4*)(&ws[lds_at(wn + t * 16 + r, kk / 8 + g4)]);
 #pragma unroll
-      for (int ta = 0; ta < TM; ++ta)
+      for (int ta = 0; ta < TM; ++ta) {
+        const int slot = kk / 32 * TM + ta;
+        if (SPREAD == 2) fetch(ahead, into, slot * NI / SLOTS, (slot + 1) * NI / SLOTS);
 #pragma unroll
         for (int tb = 0; tb < TN; ++tb)
           // A = W rows (n), B = x rows (m): the result holds 4 consecutive n per lane.
           acc[ta][tb] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(b[tb].v, a[ta].v, acc[ta][tb],
                                                                 0, 0, 0);
+      }
     }
   };
 
@@ -633,7 +644,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
   static_assert(STAGES >= 2 && STAGES <= 4, "two to four stages");
 
 #pragma unroll
-  for (int s = 0; s < STAGES - 1; ++s) fetch(s, ring[s]);
+  for (int s = 0; s < STAGES - 1; ++s) fetch(s, ring[s], 0, NI);
   for (int s0 = 0; s0 < steps; s0 += STAGES) {
 #pragma unroll
     for (int u = 0; u < STAGES; ++u) {   // unrolled: every buffer of the ring is a constant
@@ -642,8 +653,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
         __builtin_amdgcn_s_waitcnt(TILED_WAIT((STAGES - 2) * NI));
         __builtin_amdgcn_s_barrier();
         asm volatile("" ::: "memory");
-        fetch(s0 + u + STAGES - 1, ring[(u + STAGES - 1) % STAGES]);
-        products(ring[u]);
+        products(ring[u], s0 + u + STAGES - 1, ring[(u + STAGES - 1) % STAGES]);
       }
     }
   }
@@ -726,24 +736,24 @@ struct TiledConfig {
 };
 #define TILED_CONFIGS 6
 static const TiledConfig tiled_configs[TILED_CONFIGS] = {
-    {256, 256, 1, 4.9f, 4.9f},    // 0: 2 stages (128 KB), 8 wavefronts
-    {128, 256, 1, 4.27f, 4.27f},  // 1: 3 stages (144 KB), 8 wavefronts
-    {128, 128, 1, 3.6f, 3.6f},    // 2: 3 stages (96 KB), 8 wavefronts
-    {128, 128, 2, 2.02f, 2.8f},   // 3: 2 stages (64 KB), 4 wavefronts
-    {64, 64, 2, 1.15f, 1.95f},    // 4: 4 stages (64 KB), 4 wavefronts
+    {256, 256, 1, 5.03f, 5.03f},  // 0: 2 stages (128 KB), 16 wavefronts
+    {128, 256, 1, 4.7f, 4.7f},    // 1: 3 stages (144 KB), 8 wavefronts
+    {128, 128, 1, 3.75f, 3.75f},  // 2: 3 stages (96 KB), 8 wavefronts
+    {128, 128, 2, 2.03f, 2.8f},   // 3: 2 stages (64 KB), 4 wavefronts
+    {64, 64, 2, 1.2f, 2.0f},      // 4: 4 stages (64 KB), 4 wavefronts
     {64, 128, 1, 2.14f, 2.14f},   // 5: 4 stages (96 KB), 4 wavefronts
 };
 
-template <int BM, int BN, int STAGES, int WM, int WN, int EPI>
+template <int BM, int BN, int STAGES, int WM, int WN, int SPREAD, int EPI>
 static void launch_tiled_cfg(const void* x, const void* w, const void* bias, int bias_dtype,
                              void* out, int M, int N, int K, int ldo, hipStream_t stream) {
   constexpr int COLS = EPI == EPI_GATED ? BN / 2 : BN;
   dim3 grid((N + COLS - 1) / COLS, (M + BM - 1) / BM);
   if (bias && bias_dtype == MK_BF16)
-    gemm_tiled_kernel<BM, BN, STAGES, WM, WN, EPI, bf16_t><<<grid, 64 * WM * WN, 0, stream>>>(
+    gemm_tiled_kernel<BM, BN, STAGES, WM, WN, SPREAD, EPI, bf16_t><<<grid, 64 * WM * WN, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, out, M, N, K, ldo);
   else
-    gemm_tiled_kernel<BM, BN, STAGES, WM, WN, EPI, float><<<grid, 64 * WM * WN, 0, stream>>>(
+    gemm_tiled_kernel<BM, BN, STAGES, WM, WN, SPREAD, EPI, float><<<grid, 64 * WM * WN, 0, stream>>>(
         (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo);
 }
 
@@ -752,12 +762,12 @@ static void launch_tiled(int config, const void* x, const void* w, const void* b
                          int bias_dtype, void* out, int M, int N, int K, int ldo,
                          hipStream_t stream) {
   switch (config) {
-    case 0: launch_tiled_cfg<256, 256, 2, 2, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 1: launch_tiled_cfg<128, 256, 3, 2, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 2: launch_tiled_cfg<128, 128, 3, 2, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 3: launch_tiled_cfg<128, 128, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 4: launch_tiled_cfg<64, 64, 4, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    default: launch_tiled_cfg<64, 128, 4, 1, 4, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 0: launch_tiled_cfg<256, 256, 2, 4, 4, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 1: launch_tiled_cfg<128, 256, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 2: launch_tiled_cfg<128, 128, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 3: launch_tiled_cfg<128, 128, 2, 2, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 4: launch_tiled_cfg<64, 64, 4, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    default: launch_tiled_cfg<64, 128, 4, 1, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
   }
 }
 
