@@ -368,7 +368,7 @@ __device__ __forceinline__ StagedRegs<D> staged_fetch(const AttnParams& p, Table
                                                       int lane) {
   StagedRegs<D> regs;
   const int ps = 1 << p.page_shift;
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & 255;   // within the four wavefronts that share the block
   int page[2], off[2];
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
@@ -398,7 +398,7 @@ __device__ __forceinline__ StagedRegs<D> staged_fetch(const AttnParams& p, Table
 
 template <int D>
 __device__ __forceinline__ void staged_store(const StagedRegs<D>& regs, uint4* lds_k, uint4* lds_v) {
-  const int tid = threadIdx.x;
+  const int tid = threadIdx.x & 255;
 #pragma unroll
   for (int i = 0; i < D / 64; ++i) {
     const int idx = tid + i * 256;
@@ -432,12 +432,22 @@ __device__ __forceinline__ void staged_operands(KeyBlock<D>& blk, const uint4* l
     }
 }
 
-template <int D, int RT>
-__global__ __launch_bounds__(64 * ATTN_WAVES) void attn_staged_kernel(AttnParams p) {
+// KG groups of four wavefronts share a workgroup's 64 * RT rows: group g takes the key blocks
+// b0 + g, b0 + g + KG, ... with LDS buffers of its own, and at the end the groups' running
+// maxima, sums and weighted values are combined through LDS in group order.  A long prompt's
+// last rows see thousands of keys; the groups cut that chain of dependent blocks into KG
+// shorter ones that run side by side on the same compute unit.
+template <int D, int RT, int KG>
+__global__ __launch_bounds__(64 * ATTN_WAVES * KG) void attn_staged_kernel(AttnParams p) {
   static_assert(D % 64 == 0, "256 threads bring whole 16-byte chunks of 32 keys");
-  __shared__ uint4 lds_k[2][32 * D / 8];
-  __shared__ uint4 lds_v[2][32 * D / 8];
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  constexpr int BLOCK = 32 * D / 8;                       // 16-byte units of a block's keys (or values)
+  constexpr int MERGE = RT * (D / 4 + 2);                 // floats a thread hands over
+  static_assert(KG == 1 || (KG - 1) * MERGE * 4 <= KG * 4 * BLOCK * 4, "merge space fits the buffers");
+  __shared__ uint4 lds[KG * 4 * BLOCK];                   // per group: keys[2], values[2]
+  const int lane = threadIdx.x & 63;
+  const int kgroup = (threadIdx.x >> 6) / ATTN_WAVES, wave = (threadIdx.x >> 6) % ATTN_WAVES;
+  uint4* const lds_k = lds + kgroup * 4 * BLOCK;
+  uint4* const lds_v = lds_k + 2 * BLOCK;
   const int tile = p.num_tiles - 1 - (int)blockIdx.x;   // the longest work first
   const int kvh = blockIdx.y;
   const int seq = p.tile_seq[tile];
@@ -484,27 +494,75 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_staged_kernel(AttnParams
   const float c = p.scale * 1.44269504088896340736f;
 
   TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
-  StagedRegs<D> ra = staged_fetch<D>(p, tw, b0, b1, wg_kmin, wg_kmax, kvh, lane);
-  StagedRegs<D> rb = staged_fetch<D>(p, tw, b0 + 1, b1, wg_kmin, wg_kmax, kvh, lane);
+  const int first = b0 + kgroup;                        // this group's blocks: first, first + KG, ...
+  StagedRegs<D> ra = staged_fetch<D>(p, tw, first, b1, wg_kmin, wg_kmax, kvh, lane);
+  StagedRegs<D> rb = staged_fetch<D>(p, tw, first + KG, b1, wg_kmin, wg_kmax, kvh, lane);
   KeyBlock<D> blk;
   // One block: park what was fetched two iterations ago in LDS, ask for the block two ahead,
   // and, once every wavefront's share is in place, use the block.  Blocks past this
-  // wavefront's last key or before its first are the others' business.
+  // wavefront's last key or before its first are the others' business; blocks past the
+  // workgroup's last (a group may have one fewer than another) fetch a page that exists and
+  // are not used.
 #define STAGED_ITERATION(regs, b, buf)                                                  \
   do {                                                                                  \
-    staged_store<D>(regs, lds_k[buf], lds_v[buf]);                                      \
-    regs = staged_fetch<D>(p, tw, (b) + 2, b1, wg_kmin, wg_kmax, kvh, lane);            \
+    staged_store<D>(regs, lds_k + (buf) * BLOCK, lds_v + (buf) * BLOCK);                \
+    regs = staged_fetch<D>(p, tw, (b) + 2 * KG, b1, wg_kmin, wg_kmax, kvh, lane);       \
     __syncthreads();                                                                    \
     if (((b) << 5) <= kmax && ((b) << 5) + 31 >= kmin) {                                \
-      staged_operands<D>(blk, lds_k[buf], lds_v[buf], (b), kmin, kmax, lane);           \
+      staged_operands<D>(blk, lds_k + (buf) * BLOCK, lds_v + (buf) * BLOCK, (b), kmin,  \
+                         kmax, lane);                                                   \
       attend<D, RT>(st, blk, (b) << 5, c, g4, see_upto, see_from);                      \
     }                                                                                   \
   } while (0)
-  for (int b = b0; b < b1; b += 2) {
+  const int iterations = (b1 - b0 + KG - 1) / KG;       // the same for every group
+  for (int i = 0; i < iterations; i += 2) {
+    const int b = first + i * KG;
     STAGED_ITERATION(ra, b, 0);
-    if (b + 1 < b1) STAGED_ITERATION(rb, b + 1, 1);
+    if (i + 1 < iterations) STAGED_ITERATION(rb, b + KG, 1);
   }
 #undef STAGED_ITERATION
+
+  if constexpr (KG > 1) {
+    // Groups 1.. hand their state to group 0, element by element: the same lane of the same
+    // wavefront-in-group holds the same rows and dims in every group.
+    __syncthreads();                                    // the key and value buffers are free now
+    float* const merge = (float*)lds;
+    const int slot = threadIdx.x & 255;
+    if (kgroup > 0) {
+      float* mine = merge + (size_t)(kgroup - 1) * MERGE * 256 + slot;
+      int e = 0;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        mine[256 * e++] = st.m[t];
+        mine[256 * e++] = st.lsum[t];
+#pragma unroll
+        for (int dt = 0; dt < D / 16; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i) mine[256 * e++] = st.acc[t][dt][i];
+      }
+    }
+    __syncthreads();
+    if (kgroup > 0) return;
+#pragma unroll
+    for (int g = 1; g < KG; ++g) {
+      const float* theirs = merge + (size_t)(g - 1) * MERGE * 256 + slot;
+      int e = 0;
+#pragma unroll
+      for (int t = 0; t < RT; ++t) {
+        const float m_g = theirs[256 * e++], l_g = theirs[256 * e++];
+        const float m_new = fmaxf(st.m[t], m_g);
+        const float c_own = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(st.m[t] - m_new);
+        const float c_g = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_g - m_new);
+        st.m[t] = m_new;
+        st.lsum[t] = st.lsum[t] * c_own + l_g * c_g;
+#pragma unroll
+        for (int dt = 0; dt < D / 16; ++dt)
+#pragma unroll
+          for (int i = 0; i < 4; ++i)
+            st.acc[t][dt][i] = st.acc[t][dt][i] * c_own + theirs[256 * e++] * c_g;
+      }
+    }
+  }
 
 #pragma unroll
   for (int t = 0; t < RT; ++t) {
@@ -577,13 +635,17 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
 }
 
 template <int D>
-static void launch_staged(const AttnParams& p, int rows_per_tile, hipStream_t stream) {
+static void launch_staged(const AttnParams& p, int rows_per_tile, int key_groups, hipStream_t stream) {
   if constexpr (D == 64 || D == 128) {   // wider heads do not fit the register file
     dim3 grid(p.num_tiles, p.n_kv);
-    if (rows_per_tile == 16)
-      attn_staged_kernel<D, 1><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
-    else
-      attn_staged_kernel<D, 2><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
+    if (rows_per_tile == 32)
+      attn_staged_kernel<D, 2, 1><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
+    else if (key_groups == 1)
+      attn_staged_kernel<D, 1, 1><<<grid, 64 * ATTN_WAVES, 0, stream>>>(p);
+    else if (key_groups == 2)
+      attn_staged_kernel<D, 1, 2><<<grid, 64 * ATTN_WAVES * 2, 0, stream>>>(p);
+    else if constexpr (D == 64)   // 16 wavefronts of a wider head do not fit the register file
+      attn_staged_kernel<D, 1, 4><<<grid, 64 * ATTN_WAVES * 4, 0, stream>>>(p);
   }
 }
 
@@ -610,10 +672,12 @@ extern "C" int mk_attention_mfma_max_rows(int head_dim) {
   return head_dim <= 64 ? 64 : (head_dim <= 128 ? 32 : 16);
 }
 
-// Whether the kernel that stages keys and values in LDS (workgroups of 4 * rows_per_tile rows
-// of one sequence) takes this head size and tile height.
+// Into how many groups (1, 2 or 4) the kernel that stages keys and values in LDS (workgroups
+// of 4 * rows_per_tile rows of one sequence) can split a workgroup's keys at this head size
+// and tile height; 0 if it does not take them at all.
 extern "C" int mk_attention_mfma_staged(int head_dim, int rows_per_tile) {
-  return (head_dim == 64 || head_dim == 128) && (rows_per_tile == 16 || rows_per_tile == 32);
+  if (head_dim != 64 && head_dim != 128) return 0;
+  return rows_per_tile == 16 ? (head_dim == 64 ? 4 : 2) : (rows_per_tile == 32 ? 1 : 0);
 }
 
 extern "C" int mk_attention_mfma_supported(int head_dim, int page_size) {
@@ -646,9 +710,11 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   MK_REQUIRE(rows_per_tile <= mk_attention_mfma_max_rows(d),
              "attention: %d rows per tile are too many for head size %d", rows_per_tile, d);
   MK_REQUIRE(split_blocks >= 0, "attention: negative split size");
-  MK_REQUIRE(!staged || (num_splits == 1 && mk_attention_mfma_staged(d, rows_per_tile)),
+  MK_REQUIRE(staged == 0 || staged == 1 || staged == 2 || staged == 4,
+             "attention: %d key groups (0, 1, 2 or 4)", staged);
+  MK_REQUIRE(!staged || (num_splits == 1 && staged <= mk_attention_mfma_staged(d, rows_per_tile)),
              "attention: staging in LDS takes unsplit keys, head sizes 64 and 128 and 16 or 32 "
-             "rows per wavefront");
+             "rows per wavefront (one key group with 32)");
   if (num_tiles == 0) return 0;
   AttnParams p;
   p.q = (const bf16_t*)q;
@@ -675,12 +741,12 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   p.split_blocks = split_blocks;
   p.tile_rows = rows_per_tile;
   switch (d) {
-    case 32: staged ? launch_staged<32>(p, rows_per_tile, stream) : launch_attn<32>(p, rows_per_tile, stream); break;
-    case 64: staged ? launch_staged<64>(p, rows_per_tile, stream) : launch_attn<64>(p, rows_per_tile, stream); break;
-    case 96: staged ? launch_staged<96>(p, rows_per_tile, stream) : launch_attn<96>(p, rows_per_tile, stream); break;
-    case 128: staged ? launch_staged<128>(p, rows_per_tile, stream) : launch_attn<128>(p, rows_per_tile, stream); break;
-    case 192: staged ? launch_staged<192>(p, rows_per_tile, stream) : launch_attn<192>(p, rows_per_tile, stream); break;
-    case 256: staged ? launch_staged<256>(p, rows_per_tile, stream) : launch_attn<256>(p, rows_per_tile, stream); break;
+    case 32: staged ? launch_staged<32>(p, rows_per_tile, staged, stream) : launch_attn<32>(p, rows_per_tile, stream); break;
+    case 64: staged ? launch_staged<64>(p, rows_per_tile, staged, stream) : launch_attn<64>(p, rows_per_tile, stream); break;
+    case 96: staged ? launch_staged<96>(p, rows_per_tile, staged, stream) : launch_attn<96>(p, rows_per_tile, stream); break;
+    case 128: staged ? launch_staged<128>(p, rows_per_tile, staged, stream) : launch_attn<128>(p, rows_per_tile, stream); break;
+    case 192: staged ? launch_staged<192>(p, rows_per_tile, staged, stream) : launch_attn<192>(p, rows_per_tile, stream); break;
+    case 256: staged ? launch_staged<256>(p, rows_per_tile, staged, stream) : launch_attn<256>(p, rows_per_tile, stream); break;
   }
   MK_LAUNCH_CHECK("attention_mfma");
   return 0;

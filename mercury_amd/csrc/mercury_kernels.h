@@ -117,9 +117,10 @@ int mk_attention_mfma_max_rows(int head_dim);
 // counts, kv_len [S] their lengths once this step's tokens are written.  With num_splits > 1
 // the keys are split, split_blocks blocks of 32 keys per split (0: each tile's own range in
 // num_splits equal parts), and part_o [tiles, n_kv, splits, rows_per_tile, d] /
-// part_ml [.., rows_per_tile, 2] hold the partial results.  staged != 0 (see
-// mk_attention_mfma_staged): the tiles are of 4 * rows_per_tile rows, one per workgroup, whose
-// wavefronts share the keys and values through LDS; for many rows per sequence, keys unsplit.
+// part_ml [.., rows_per_tile, 2] hold the partial results.  staged != 0: the tiles are of
+// 4 * rows_per_tile rows, one per workgroup, whose wavefronts share the keys and values
+// through LDS, `staged` (1, 2 or 4, at most what mk_attention_mfma_staged returns) groups of
+// four wavefronts taking the key blocks in turn; for many rows per sequence, keys unsplit.
 int mk_attention_mfma_staged(int head_dim, int rows_per_tile);
 int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       const void* k_cache, const void* v_cache, const int* tile_seq,

@@ -454,6 +454,7 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     size and the float32-arithmetic kernel otherwise; "generic" and "mfma" force one.
     tile_rows (16, 32 or 64) overrides how many rows a wavefront of the matrix-core kernel
     takes, split_override = (splits, key blocks per split) how the keys are split, staged
+    (False, or 1, 2 or 4 groups of wavefronts that split a workgroup's keys among them)
     whether workgroups of four wavefronts share the keys and values of one sequence's rows
     through LDS; by default the step's size decides all three.
     """
@@ -504,7 +505,16 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
                   and bool(lib.mk_attention_mfma_staged(head_dim, 16)))
         if staged:
             rows = 16
+            staged = -1       # as many key groups as pay, once the tiles are counted
     tile_seq, tile_row0, num_tiles = step.tiles(group, rows * 4 if staged else rows)
+    if staged == -1:
+        # A workgroup's chain of key blocks is cut into 2 or 4 chains side by side while that
+        # leaves the chip short of wavefronts and every chain a few blocks (measured at 2,048
+        # tokens, 14 heads of 64: 62, 50, 36 us with 1, 2, 4 groups; at 8,192: 372, 323, 385).
+        staged = lib.mk_attention_mfma_staged(head_dim, 16)
+        while staged > 1 and (num_tiles * n_kv * 4 * staged > ATTENTION_STAGED_MAX_WAVES
+                              or blocks < 4 * staged):
+            staged //= 2
     splits, split_blocks = 1, 0
     waves = max(1, num_tiles * n_kv)
     if staged:
@@ -530,6 +540,7 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
 
 ATTENTION_TARGET_WAVES = 1024
 ATTENTION_STAGED_WORKGROUPS = 128
+ATTENTION_STAGED_MAX_WAVES = 16384
 ATTENTION_WIDE_TILE_WAVES = 400
 ATTENTION_MIN_BLOCKS_PER_SPLIT = 2
 

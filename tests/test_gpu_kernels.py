@@ -680,14 +680,17 @@ def test_attention_wide_tiles_for_prompts(tile_rows, d, n_q, n_kv, window, split
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
-@pytest.mark.parametrize("tile_rows,d,n_q,n_kv,page", [(16, 64, 14, 2, 16), (32, 64, 14, 2, 16),
-                                                       (16, 128, 8, 2, 32), (32, 128, 4, 4, 16),
-                                                       (32, 64, 3, 1, 64)])
+@pytest.mark.parametrize("tile_rows,d,n_q,n_kv,page,groups", [
+    (16, 64, 14, 2, 16, 1), (32, 64, 14, 2, 16, 1), (16, 128, 8, 2, 32, 1), (32, 128, 4, 4, 16, 1),
+    (32, 64, 3, 1, 64, 1), (16, 64, 14, 2, 16, 2), (16, 64, 14, 2, 16, 4), (16, 128, 8, 2, 32, 2),
+    (16, 64, 3, 1, 64, 4)])
 @pytest.mark.parametrize("window", [None, 40])
-def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, window):
-    """Workgroups whose four wavefronts share the keys and values of one sequence through LDS:
-    prompt portions of different length, one over a cached prefix, one ending inside a
-    workgroup's rows, beside a decoded token; pages scattered and poisoned outside."""
+def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, groups, window):
+    """Workgroups whose wavefronts share the keys and values of one sequence through LDS, in
+    one, two or four groups that take the key blocks in turn (with a window of 40 some groups
+    get no block at all): prompt portions of different length, one over a cached prefix, one
+    ending inside a workgroup's rows, beside a decoded token; pages scattered and poisoned
+    outside."""
     lens, q_lens = [333, 150, 77, 90], [333, 150, 33, 1]
     qs, ks, vs = [], [], []
     for i, s in enumerate(lens):
@@ -702,7 +705,7 @@ def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, window
         at += n
     got = run_attention([q[-ql:] for q, ql in zip(qs, q_lens)], ks, vs, torch.bfloat16, pages, page,
                         sum(per) + 5, lens, q_lens, d ** -0.5, window=window, poison=1e4,
-                        kernel="mfma", tile_rows=tile_rows, staged=True)
+                        kernel="mfma", tile_rows=tile_rows, staged=groups)
     want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-ql:]
                       for q, k, v, ql in zip(qs, ks, vs, q_lens)])
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
