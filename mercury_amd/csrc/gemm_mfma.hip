@@ -331,31 +331,53 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   }
 }
 
-// Slices of K for the plain skinny projection: enough workgroups to fill the chip (about
-// 512), every wavefront of a workgroup with at least one k-step, and no more partial results
-// than the weights are worth (slices * M * 4 bytes per output column against K * 2).
+// What a skinny projection over `slices` slices of K costs, relative to one workgroup
+// streaming 32 whole rows of W: the chip serves every compute unit about the same share of
+// HBM bandwidth, so the time is that of the unit with the most bytes, workgroups being dealt
+// out over the 256 units in turn; every further slice adds a little (partial results, x read
+// again, a workgroup's start and finish).  Measured at 5120 x 27648, 8 rows: 71, 77, 57, 62, 65, 59, 60, 56 us for 1..8
+// slices, which is this function's shape.
+static double skinny_split_cost(int tiles, int slices, int M, int K) {
+  const long groups = (long)tiles * slices;
+  const double extra = 0.02 * (slices - 1) + 2.0 * slices * M / K;   // the second: partial results
+  return (double)((groups + 255) / 256) / slices * (1.0 + extra);
+}
+
+// Slices of K for the plain skinny projection: the count with the least cost above, every
+// wavefront of a workgroup with at least one k-step, and no more partial results than the
+// weights are worth (slices * M * 4 bytes per output column against K * 2).
 extern "C" int mk_linear_skinny_slices(int M, int N, int K) {
   const int tiles = (N + 31) / 32;
   const int steps = (K + 127) / 128;
-  int slices = (512 + tiles - 1) / tiles;
-  const int by_steps = (steps + SK_WAVES - 1) / SK_WAVES;
-  if (slices > by_steps) slices = by_steps;
+  int limit = (steps + SK_WAVES - 1) / SK_WAVES;
   const int cap = K / (8 * (M > 0 ? M : 1));
-  if (slices > cap) slices = cap;
-  if (slices < 1) slices = 1;
-  const int per = (steps + slices - 1) / slices;
-  return (steps + per - 1) / per;
+  if (limit > cap) limit = cap;
+  if (limit > 16) limit = 16;
+  int best = 1;
+  double best_cost = skinny_split_cost(tiles, 1, M, K);
+  for (int slices = 2; slices <= limit; ++slices) {
+    const int per = (steps + slices - 1) / slices;
+    if ((steps + per - 1) / per != slices) continue;   // not a count the steps divide into
+    const double cost = skinny_split_cost(tiles, slices, M, K);
+    if (cost < best_cost - 1e-9) best = slices, best_cost = cost;
+  }
+  return best;
 }
 
 // Whether a projection added straight into the residual stream should keep all of K in one
-// workgroup (no partial results, one kernel less to wait for): for at most 16 rows of x,
-// when 16-row workgroups alone occupy most of the chip, or when the matrix is so small that
-// latency, not bandwidth, is what its kernel costs.  One workgroup alone pulls about 35 GB/s;
-// with more rows of x every workgroup re-reads so much of x from the L2 that fewer, larger
-// workgroups over slices of K are faster.
+// workgroup of 16 rows (no partial results): for at most 16 rows of x, when the matrix is so
+// small that latency, not bandwidth, is what its kernel costs, or when 16-row workgroups
+// spread over the compute units clearly more evenly than the best split does (they stream a
+// little slower than 32-row workgroups over half of K: 32.7 against 29.6 us at
+// 3584 x 18944).  With more rows of x every workgroup re-reads so much of x from the L2 that
+// fewer, larger workgroups over slices of K are faster.
 extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
+  if (M > 16) return 0;
+  if ((double)N * K * 2.0 <= 4.0e6) return 1;
   const int tiles16 = (N + 15) / 16;
-  return M <= 16 && (tiles16 >= 192 || (double)N * K * 2.0 <= 4.0e6);
+  const double whole = 0.5 * ((tiles16 + 255) / 256);
+  const double split = skinny_split_cost((N + 31) / 32, mk_linear_skinny_slices(M, N, K), M, K);
+  return whole < 0.9 * split;
 }
 
 template <int NT, int EPI>

@@ -230,16 +230,21 @@ def test_the_tile_configuration_follows_the_problem():
 
 
 def test_which_skinny_projections_are_split():
-    """K is split into partial sums only where the matrix is large and has too few rows to
-    occupy the chip with 16-row workgroups."""
+    """K is split into partial sums wherever the matrix is large enough for bandwidth to
+    matter; how often follows how evenly the workgroups then spread over the compute units."""
+    lib = ops()._lib.load("mfma")
+
     def wants(m, n, k):
         return ops().wants_partials(torch.zeros(m, k, dtype=torch.bfloat16, device=DEV),
                                     torch.zeros(n, k, dtype=torch.bfloat16, device=DEV))
-    assert wants(8, 896, 4864)             # 8.7 MB behind 56 tiles of rows
+    assert wants(8, 896, 4864)             # 8.7 MB behind 28 tiles of rows
     assert not wants(8, 896, 896)          # small: latency is the cost, not bandwidth
-    assert not wants(8, 3584, 4096)        # 224 tiles of rows are workgroups enough
-    assert wants(64, 3584, 4096)           # many rows of x: re-reading them costs more than slices
+    assert wants(8, 3584, 4096) and wants(64, 3584, 4096)
     assert not wants(8, 896, 4868)         # K % 8 != 0: not for the matrix cores at all
+    assert lib.mk_linear_skinny_slices(8, 896, 4864) == 8      # 224 workgroups: one a unit
+    assert lib.mk_linear_skinny_slices(8, 3584, 18944) == 2    # 224 again
+    assert lib.mk_linear_skinny_slices(8, 5120, 27648) == 3    # 480: two a unit, few idle
+    assert lib.mk_linear_skinny_slices(8, 8192, 8192) == 1     # 256 as it is
 
 
 @pytest.mark.parametrize("m,n,k", [(1, 896, 896), (8, 1003, 168), (17, 130, 264), (64, 3584, 1024),
