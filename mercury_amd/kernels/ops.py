@@ -153,8 +153,8 @@ GATED_TILED_MIN_ROWS, GATED_TILED_MIN_WEIGHTS = 33, 16 << 20
 
 def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether x W^T is best computed as K-split float32 partial sums (`linear_partials`):
-    few rows of bfloat16 x, where the weights are the traffic and the chip needs the split to
-    have enough wavefronts in flight."""
+    few rows of bfloat16 x and a matrix large enough for bandwidth to matter, where slices
+    of K spread the workgroups evenly over the compute units."""
     if not _skinny_eligible(x, w):
         return False
     return not _lib.load("mfma").mk_linear_skinny_unsplit(x.shape[0], w.shape[0], w.shape[1])
@@ -254,7 +254,7 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
         lib = _lib.load("mfma")
         # Few rows straight from HBM into the matrix cores; from 17 rows on, a wide matrix
         # (the head over the vocabulary) is faster through LDS tiles, which read x once per
-        # 128 columns instead of once per 32.
+        # 64 or 128 columns instead of once per 32.
         if (m <= SKINNY_MAX_ROWS and out_dtype == torch.float32 and bias is None and not accumulate
                 and (m <= 16 or n < WIDE_MATRIX_COLUMNS)):
             _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, 1, _stream()),
