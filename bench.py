@@ -9,6 +9,12 @@ One JSON line is printed: `value` is decoded tokens per second; `prefill` times 
 prompt as one step; `roofline` divides the bytes a decode step has to read (every weight it
 uses once, and the cache of the live requests) by its time and by the HBM peak; `points`
 holds decode throughput at batch 1 and 64.
+
+    python bench.py --shape 32b --serve
+
+runs a whole workload through the scheduler instead (64 requests with prompts of 2,048 tokens,
+admitted in portions of 512 beside the decoding of the others, each decoded to 4,096) and
+prints the generated tokens per second of the whole run.
 """
 
 from __future__ import annotations
@@ -63,6 +69,13 @@ def parse_args(argv=None):
     p.add_argument("--no-lookahead", action="store_true",
                    help="never start a decode step before the previous one's tokens are read")
     p.add_argument("--seed", type=int, default=0)
+    p.add_argument("--serve", action="store_true",
+                   help="instead of the decode steps: --serve-requests requests with prompts of "
+                        "half the context through the scheduler, prompts in portions of "
+                        "--serve-chunk tokens beside the others' decoding, each decoded to the "
+                        "context; one line with the generated tokens a second")
+    p.add_argument("--serve-requests", type=int, default=64)
+    p.add_argument("--serve-chunk", type=int, default=512)
     return p.parse_args(argv)
 
 
@@ -79,7 +92,7 @@ def prefill_flops(cfg: dict, tokens: int) -> float:
 
 class Bench:
     def __init__(self, cfg: dict, dtype: str, max_batch: int, context: int, seed: int,
-                 lookahead: bool = True):
+                 lookahead: bool = True, prefill_budget: int = 8192):
         import torch
 
         from mercury_amd.cache import CacheManager, PageHasher
@@ -100,7 +113,7 @@ class Bench:
         pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + PREFILL_TOKENS // BLOCK_SIZE + 8
         self.engine_cfg = EngineConfig(
             model="random", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
-            max_running=max_batch + 1, prefill_budget=8192, max_model_len=context + 128, seed=seed,
+            max_running=max_batch + 1, prefill_budget=prefill_budget, max_model_len=context + 128, seed=seed,
             lookahead=lookahead)
         manager = CacheManager(model.cache_slots, pages, BLOCK_SIZE, max_batch + 1, False)
         runner = ModelRunner(model, manager, torch_dtype, device, context + 128)
@@ -185,6 +198,79 @@ class Bench:
         return {"tok_s": tokens / seconds, "ms": 1e3 * seconds}
 
 
+    def serve(self, requests: int, prompt_len: int, new_tokens: int) -> dict:
+        """All requests submitted at once and run to their last token by the engine's own
+        loop: prompts enter in portions under the token budget beside the decoding of the
+        requests already in."""
+        from mercury_amd import SamplingParams
+
+        generated = [0]
+
+        def sink(event):
+            if event.kind == "token":
+                generated[0] += 1
+
+        for _ in range(requests):
+            rid = f"bench-{self.counter}"
+            self.counter += 1
+            self.engine.submit(rid, self.tokens(prompt_len), new_tokens, sink,
+                               params=SamplingParams(ignore_eos=True))
+        self.engine._drain_commands()
+        self.sync()
+        start = time.perf_counter()
+        steps = mixed = 0
+        split = {"sched": 0.0, "prepare": 0.0, "forward": 0.0}
+        first_all_decoding = None
+        while self.engine.sched.has_work():
+            record = self.engine.step()
+            steps += 1
+            mixed += bool(record.num_prefill and record.num_decode)
+            split["sched"] += record.sched_s
+            split["prepare"] += record.prepare_s
+            split["forward"] += record.forward_s
+            if first_all_decoding is None and not record.num_prefill and not self.engine.sched.waiting:
+                self.sync()
+                first_all_decoding = time.perf_counter() - start
+            if steps % 256 == 0:
+                print(f"[bench] serve: step {steps}, {generated[0]} tokens", file=sys.stderr, flush=True)
+        self.sync()
+        elapsed = time.perf_counter() - start
+        assert self.engine.leaked_blocks() == 0
+        assert generated[0] == requests * new_tokens, (generated[0], requests * new_tokens)
+        return {"tok_s": generated[0] / elapsed, "seconds": elapsed, "steps": steps, "mixed": mixed,
+                "generated": generated[0], "prompt_seconds": first_all_decoding or 0.0,
+                "preemptions": self.engine.metrics.summary().get("preemptions", 0),
+                "split": {k: round(v, 3) for k, v in split.items()}}
+
+
+def serve_main(args, model_name: str, cfg: dict, full_layers: int) -> int:
+    prompt_len = args.context // 2
+    new_tokens = args.context - prompt_len
+    bench = Bench(cfg, args.dtype, args.serve_requests, args.context, args.seed,
+                  not args.no_lookahead, prefill_budget=args.serve_chunk)
+    run = bench.serve(args.serve_requests, prompt_len, new_tokens)
+    short = "bf16" if args.dtype == "bfloat16" else "fp32"
+    print(json.dumps({
+        "metric": f"generated tok/s, {args.serve_requests} requests of {prompt_len} prompt tokens "
+                  f"in portions of {args.serve_chunk} beside decoding, to a context of "
+                  f"{args.context} ({model_name} shapes)",
+        "value": round(run["tok_s"], 1), "unit": "tok/s", "n_gpus": 1, "steps": run["steps"],
+        "warmup": 0, "ms_per_step": round(1e3 * run["seconds"] / run["steps"], 4),
+        "higher_is_better": True, "scaling": "weak", "vs_baseline": None, "dtype": short,
+        "data": "synthetic: seeded uniform-random token ids, random weights N(0, 0.02) drawn on the GPU",
+        "config": {"model": f"{model_name} shapes", "layers": cfg["num_hidden_layers"],
+                   "layers_full": full_layers, "requests": args.serve_requests,
+                   "prompt_len": prompt_len, "new_tokens": new_tokens,
+                   "prefill_budget": args.serve_chunk, "seq_len": args.context,
+                   "block_size": BLOCK_SIZE, "parallelism": "single GPU"},
+        "seconds": round(run["seconds"], 3), "generated": run["generated"],
+        "steps_with_prompt_and_decode": run["mixed"],
+        "seconds_until_all_decode": round(run["prompt_seconds"], 3),
+        "preemptions": run["preemptions"], "host_seconds": run["split"],
+    }), flush=True)
+    return 0
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     if args.gpus != 1:
@@ -196,6 +282,8 @@ def main(argv=None) -> int:
     full_layers = cfg["num_hidden_layers"]
     if args.layers:
         cfg["num_hidden_layers"] = args.layers
+    if args.serve:
+        return serve_main(args, model_name, cfg, full_layers)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
     bench = Bench(cfg, args.dtype, max_batch, args.context, args.seed, not args.no_lookahead)
 
