@@ -542,7 +542,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
                                                                   const bf16_t* __restrict__ w,
                                                                   const TBIAS* __restrict__ bias,
                                                                   void* __restrict__ out_, int M,
-                                                                  int N, int K, int ldo) {
+                                                                  int N, int K, int ldo,
+                                                                  int slice_stages) {
   constexpr int WAVES = WM * WN, TK = TILE_K;
   constexpr int NI = (BM + BN) / 8 / WAVES;                 // load instructions per wavefront and stage
   static_assert((BM + BN) % (8 * WAVES) == 0 && WAVES % 2 == 0, "tile rows divide over the wavefronts");
@@ -600,9 +601,16 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
       src[i] = w + (size_t)wrow * K + chunk * 8;
     }
   }
-  const int steps = (K + TK - 1) / TK;
-  const bool ragged = K % TK != 0;
-  const bool past_k = (steps - 1) * TK + chunk * 8 >= K;    // this lane's part of a partial last stage
+  // gridDim.z slices of K, slice_stages stages each, every slice with a result of its own
+  // (EPI_F32 only): out[slice][M][ldo].
+  const int all_steps = (K + TK - 1) / TK;
+  const int first_step = blockIdx.z * slice_stages;
+  const int steps = min(slice_stages, all_steps - first_step);
+  const bool ragged = K % TK != 0 && first_step + steps == all_steps;
+  const bool past_k = (all_steps - 1) * TK + chunk * 8 >= K;  // this lane's part of a partial last stage
+#pragma unroll
+  for (int i = 0; i < NI; ++i) src[i] += (size_t)first_step * TK;
+  if (EPI == EPI_F32) out_ = (float*)out_ + (size_t)blockIdx.z * M * ldo;
 
   f32x4 acc[TM][TN];
 #pragma unroll
@@ -768,67 +776,117 @@ static const TiledConfig tiled_configs[TILED_CONFIGS] = {
 
 template <int BM, int BN, int STAGES, int WM, int WN, int SPREAD, int EPI>
 static void launch_tiled_cfg(const void* x, const void* w, const void* bias, int bias_dtype,
-                             void* out, int M, int N, int K, int ldo, hipStream_t stream) {
+                             void* out, int M, int N, int K, int ldo, int slices,
+                             hipStream_t stream) {
   constexpr int COLS = EPI == EPI_GATED ? BN / 2 : BN;
-  dim3 grid((N + COLS - 1) / COLS, (M + BM - 1) / BM);
+  const int all_steps = (K + TILE_K - 1) / TILE_K;
+  const int slice_stages = (all_steps + slices - 1) / slices;
+  dim3 grid((N + COLS - 1) / COLS, (M + BM - 1) / BM, (all_steps + slice_stages - 1) / slice_stages);
   if (bias && bias_dtype == MK_BF16)
     gemm_tiled_kernel<BM, BN, STAGES, WM, WN, SPREAD, EPI, bf16_t><<<grid, 64 * WM * WN, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, out, M, N, K, ldo);
+        (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, out, M, N, K, ldo, slice_stages);
   else
     gemm_tiled_kernel<BM, BN, STAGES, WM, WN, SPREAD, EPI, float><<<grid, 64 * WM * WN, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo);
+        (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo, slice_stages);
 }
 
 template <int EPI>
 static void launch_tiled(int config, const void* x, const void* w, const void* bias,
-                         int bias_dtype, void* out, int M, int N, int K, int ldo,
+                         int bias_dtype, void* out, int M, int N, int K, int ldo, int slices,
                          hipStream_t stream) {
   switch (config) {
-    case 0: launch_tiled_cfg<256, 256, 2, 4, 4, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 1: launch_tiled_cfg<128, 256, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 2: launch_tiled_cfg<128, 128, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 3: launch_tiled_cfg<128, 128, 2, 2, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    case 4: launch_tiled_cfg<64, 64, 4, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
-    default: launch_tiled_cfg<64, 128, 4, 1, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, stream); break;
+    case 0: launch_tiled_cfg<256, 256, 2, 4, 4, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
+    case 1: launch_tiled_cfg<128, 256, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
+    case 2: launch_tiled_cfg<128, 128, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
+    case 3: launch_tiled_cfg<128, 128, 2, 2, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
+    case 4: launch_tiled_cfg<64, 64, 4, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
+    default: launch_tiled_cfg<64, 128, 4, 1, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
   }
 }
 
-// The configuration with the least estimated time for y[M, cols] over K.  A tile covers
-// `bn / halves` columns (halves = 2 when gate and up rows share a tile) and moves `out_bytes`
-// per element in its epilogue.  Tiles are dealt to the 256 compute units; a tile costs its
-// products at the configuration's rate plus a start (the first loads' latency) and a finish
-// (the epilogue, at what one workgroup streams: about 35 GB/s); of two resident workgroups
-// one's start and finish hide behind the other's products, and an odd last one runs alone.
+// The estimated time, in microseconds, of y[M, cols] over K in configuration t with K cut
+// into `slices`.  A tile covers `bn / halves` columns (halves = 2 when gate and up rows share
+// a tile) and moves `out_bytes` per element in its epilogue.  Tiles are dealt to the 256
+// compute units; a tile costs its products at the configuration's rate plus a start (the
+// first loads' latency) and a finish (the epilogue, at what one workgroup streams: about
+// 35 GB/s); of two resident workgroups one's start and finish hide behind the other's
+// products, and an odd last one runs alone.
+static double tiled_time(const TiledConfig& t, int M, int cols, int K, int halves, int out_bytes,
+                         int slices) {
+  const int width = t.bn / halves;
+  const long tiles = (long)((M + t.bm - 1) / t.bm) * ((cols + width - 1) / width) * slices;
+  const bool few = tiles <= 4 * 256;
+  const double per_unit = few ? (double)((tiles + 255) / 256) : tiles / 256.0 + 0.5;
+  const double products = 2.0 * t.bm * t.bn * K * 1e-6 / slices;        // MFLOP
+  const double edges = 1.5 + (double)t.bm * width * out_bytes / 35e3;  // microseconds
+  if (t.resident == 1) return per_unit * (products / t.rate + edges);
+  if (few) {
+    const long n = (long)per_unit;
+    return (n / 2) * (products / t.rate + edges / 2) + (n % 2) * (products / t.alone + edges);
+  }
+  return per_unit / 2 * (products / t.rate + edges / 2);
+}
+
+// The configuration with the least estimated time, K whole.
 static int tiled_config_for(int M, int cols, int K, int halves, int out_bytes) {
   int best = -1;
   double best_time = 0.0;
   for (int c = 0; c < TILED_CONFIGS; ++c) {
-    const TiledConfig& t = tiled_configs[c];
-    if (M <= 64 && t.bm > 64) continue;
-    const int width = t.bn / halves;
-    const long tiles = (long)((M + t.bm - 1) / t.bm) * ((cols + width - 1) / width);
-    const bool few = tiles <= 4 * 256;
-    const double per_unit = few ? (double)((tiles + 255) / 256) : tiles / 256.0 + 0.5;
-    const double products = 2.0 * t.bm * t.bn * K * 1e-6;            // MFLOP
-    const double edges = 1.5 + (double)t.bm * width * out_bytes / 35e3;  // microseconds
-    double time;
-    if (t.resident == 1) {
-      time = per_unit * (products / t.rate + edges);
-    } else if (few) {
-      const long n = (long)per_unit;
-      time = (n / 2) * (products / t.rate + edges / 2) + (n % 2) * (products / t.alone + edges);
-    } else {
-      time = per_unit / 2 * (products / t.rate + edges / 2);
-    }
+    if (M <= 64 && tiled_configs[c].bm > 64) continue;
+    const double time = tiled_time(tiled_configs[c], M, cols, K, halves, out_bytes, 1);
     if (best < 0 || time < best_time) best = c, best_time = time;
   }
   return best;
+}
+
+// Configuration and number of slices of K (each with a float32 result of its own, for a
+// consumer that adds them up) with the least estimated time: for few rows of x over a long K,
+// where whole-K tiles are too few to occupy the chip.  Every slice keeps at least 8 stages.
+static void tiled_plan_sliced(int M, int N, int K, int* config, int* slices) {
+  const int all_steps = (K + TILE_K - 1) / TILE_K;
+  double best_time = 0.0;
+  *config = -1, *slices = 1;
+  for (int c = 0; c < TILED_CONFIGS; ++c) {
+    if (M <= 64 && tiled_configs[c].bm > 64) continue;
+    for (int s = 1; s <= 16 && (s == 1 || all_steps / s >= 8); ++s) {
+      const int per = (all_steps + s - 1) / s;
+      if ((all_steps + per - 1) / per != s) continue;
+      // a slice more costs its share of writing and re-reading the partial results
+      const double time = tiled_time(tiled_configs[c], M, N, K, 1, 4, s) * (1.0 + 0.02 * (s - 1));
+      if (*config < 0 || time < best_time) *config = c, *slices = s, best_time = time;
+    }
+  }
 }
 
 extern "C" int mk_linear_tiled_configs(void) { return TILED_CONFIGS; }
 
 extern "C" int mk_linear_tiled_config(int M, int N, int K, int out_bytes) {
   return tiled_config_for(M, N, K, 1, out_bytes);
+}
+
+extern "C" int mk_linear_tiled_slices(int M, int N, int K) {
+  int config, slices;
+  tiled_plan_sliced(M, N, K, &config, &slices);
+  return slices;
+}
+
+// out[slices, M, N] (float32): partial sums of x W^T over `slices` slices of K
+// (mk_linear_tiled_slices says how many pay), for a consumer that adds them in slice order.
+extern "C" int mk_linear_tiled_partials(const void* x, const void* w, float* out, int M, int N,
+                                        int K, int slices, hipStream_t stream) {
+  MK_REQUIRE(M > 0 && N > 0 && K > 0 && K % 8 == 0,
+             "tiled projection: K=%d must be a multiple of 8 (M=%d N=%d)", K, M, N);
+  MK_REQUIRE((M + 63) / 64 <= 65535, "tiled projection: M=%d too large for one launch", M);
+  int config, planned;
+  tiled_plan_sliced(M, N, K, &config, &planned);
+  const int all_steps = (K + TILE_K - 1) / TILE_K;
+  const int per = (all_steps + (slices > 0 ? slices : 1) - 1) / (slices > 0 ? slices : 1);
+  MK_REQUIRE(slices >= 1 && slices <= 1024 && (all_steps + per - 1) / per == slices,
+             "tiled projection: %d stages of K do not divide into %d slices", all_steps, slices);
+  if (slices != planned) config = tiled_config_for(M, N, (K + slices - 1) / slices, 1, 4);
+  launch_tiled<EPI_F32>(config, x, w, nullptr, MK_F32, out, M, N, K, N, slices, stream);
+  MK_LAUNCH_CHECK("linear_tiled_partials");
+  return 0;
 }
 
 // act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K].
@@ -839,7 +897,7 @@ extern "C" int mk_gated_tiled(const void* x, const void* w, void* act, int M, in
   MK_REQUIRE((M + 63) / 64 <= 65535, "gated projection: M=%d too large for one launch", M);
   if (config < 0) config = tiled_config_for(M, inter, K, 2, 2);
   MK_REQUIRE(config < TILED_CONFIGS, "gated projection: no configuration %d", config);
-  launch_tiled<EPI_GATED>(config, x, w, nullptr, MK_F32, act, M, inter, K, inter, stream);
+  launch_tiled<EPI_GATED>(config, x, w, nullptr, MK_F32, act, M, inter, K, inter, 1, stream);
   MK_LAUNCH_CHECK("gated_tiled");
   return 0;
 }
@@ -857,11 +915,11 @@ extern "C" int mk_linear_tiled(const void* x, const void* w, const void* bias, i
     config = mk_linear_tiled_config(M, N, K, accumulate ? 8 : (out_dtype == MK_F32 ? 4 : 2));
   MK_REQUIRE(config < TILED_CONFIGS, "tiled projection: no configuration %d", config);
   if (accumulate)
-    launch_tiled<EPI_ACC>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
+    launch_tiled<EPI_ACC>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, 1, stream);
   else if (out_dtype == MK_F32)
-    launch_tiled<EPI_F32>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
+    launch_tiled<EPI_F32>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, 1, stream);
   else if (out_dtype == MK_BF16)
-    launch_tiled<EPI_BF16>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, stream);
+    launch_tiled<EPI_BF16>(config, x, w, bias, bias_dtype, out, M, N, K, ldo, 1, stream);
   else
     MK_REQUIRE(false, "tiled projection: unknown out dtype %d", out_dtype);
   MK_LAUNCH_CHECK("linear_tiled");

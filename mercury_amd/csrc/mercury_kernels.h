@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 5
+#define MK_ABI_VERSION 6
 
 #ifdef __cplusplus
 extern "C" {
@@ -99,6 +99,12 @@ int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, in
 // accumulated into `out`.  config: a tile configuration, 0 .. mk_linear_tiled_configs() - 1
 // (mk_linear_tiled_config picks the one estimated fastest for the shape and the bytes the
 // epilogue moves per element of y; -1 does the same).
+// mk_linear_tiled_partials: the same product as float32 partial sums out[slices, M, N] over
+// slices of K, for few rows of x over a long K (mk_linear_tiled_slices: how many slices pay;
+// any count that the 64-wide stages of K divide into is taken).
+int mk_linear_tiled_slices(int M, int N, int K);
+int mk_linear_tiled_partials(const void* x, const void* w, float* out, int M, int N, int K,
+                             int slices, hipStream_t stream);
 int mk_linear_tiled_configs(void);
 int mk_linear_tiled_config(int M, int N, int K, int out_bytes);
 int mk_linear_tiled(const void* x, const void* w, const void* bias, int bias_dtype, void* out,

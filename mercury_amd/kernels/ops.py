@@ -146,6 +146,8 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Te
 
 
 SKINNY_MAX_ROWS = 64
+SKINNY_SPLIT_MAX_ROWS = 16     # K-split partial sums: the skinny kernel up to here, tiles beyond
+FUSED_QKV_MAX_WEIGHTS = 48 << 20  # bytes; with more than 16 rows of x
 WIDE_MATRIX_COLUMNS = 8192
 FUSED_QKV_MIN_WORKGROUPS = 128
 GATED_TILED_MIN_ROWS, GATED_TILED_MIN_WEIGHTS = 33, 16 << 20
@@ -153,31 +155,45 @@ GATED_TILED_MIN_ROWS, GATED_TILED_MIN_WEIGHTS = 33, 16 << 20
 
 def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether x W^T is best computed as K-split float32 partial sums (`linear_partials`):
-    few rows of bfloat16 x and a matrix large enough for bandwidth to matter, where slices
-    of K spread the workgroups evenly over the compute units."""
-    if not _skinny_eligible(x, w):
+    bfloat16 x of few enough rows, and a matrix large enough for bandwidth to matter, that
+    whole-K workgroups would leave compute units idle or unevenly loaded."""
+    if not _mfma_eligible(x, w):
         return False
-    return not _lib.load("mfma").mk_linear_skinny_unsplit(x.shape[0], w.shape[0], w.shape[1])
+    lib = _lib.load("mfma")
+    m, (n, k) = x.shape[0], w.shape
+    if m <= SKINNY_SPLIT_MAX_ROWS:
+        return not lib.mk_linear_skinny_unsplit(m, n, k)
+    return lib.mk_linear_tiled_slices(m, n, k) > 1
+
+
+def _mfma_eligible(x, w: torch.Tensor) -> bool:
+    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
+            and x.shape[0] > 0 and x.shape[1] % 8 == 0)
 
 
 def _skinny_eligible(x, w: torch.Tensor) -> bool:
-    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-            and 0 < x.shape[0] <= SKINNY_MAX_ROWS and x.shape[1] % 8 == 0)
+    return _mfma_eligible(x, w) and x.shape[0] <= SKINNY_MAX_ROWS
 
 
 def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """Float32 partial sums [P, M, N] of x W^T over P slices of K; the consumer (rmsnorm,
-    rope_kv_write: their `partials` forms) adds them up in slice order."""
+    rope_kv_write: their `partials` forms) adds them up in slice order.  At most 16 rows:
+    the weights stream straight into the matrix cores; more: tiles through LDS."""
     _dev(x, w)
-    if not _skinny_eligible(x, w) or x.shape[1] != w.shape[1]:
+    if not _mfma_eligible(x, w) or x.shape[1] != w.shape[1]:
         raise KernelArgumentError(f"linear_partials: x {tuple(x.shape)} / W {tuple(w.shape)} not eligible")
     m, k = x.shape
     n = w.shape[0]
     lib = _lib.load("mfma")
-    slices = lib.mk_linear_skinny_slices(m, n, k)
-    out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
-    _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream()),
-               "linear_partials")
+    if m <= SKINNY_SPLIT_MAX_ROWS:
+        slices = lib.mk_linear_skinny_slices(m, n, k)
+        out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+        code = lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream())
+    else:
+        slices = lib.mk_linear_tiled_slices(m, n, k)
+        out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+        code = lib.mk_linear_tiled_partials(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream())
+    _lib.check(lib, code, "linear_partials")
     return out
 
 
@@ -379,9 +395,12 @@ def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int
     """Whether `qkv_project` runs as one kernel by itself: few bfloat16 rows, K a multiple of
     8, heads a multiple of 32 wide and rotated over their whole width or not at all, pages a
     power of two; and, as that kernel has one workgroup per 32 rows of W with all of K, more
-    than 16 rows of x only where those workgroups are many."""
+    than 16 rows of x only where those workgroups are many and the matrix is not so large
+    that tiles over slices of K stream it faster (7168 x 5120 at 64 rows: 43 us in one
+    kernel, 20 + 7 in two)."""
     return (_qkv_fusable(x, w, head_dim, rotary_dim, page_size)
-            and (x.shape[0] <= 16 or w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS))
+            and (x.shape[0] <= 16 or (w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS
+                                      and w.numel() * 2 <= FUSED_QKV_MAX_WEIGHTS)))
 
 
 def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor | None,

@@ -153,8 +153,32 @@ def test_skinny_projection_partial_sums(m, n, k):
     torch.testing.assert_close(parts.sum(0).cpu(), want, atol=2e-4, rtol=1e-4)
     whole = ops().linear(x_d, w_d, out_dtype=torch.float32, kernel="mfma")   # one slice: the logits path
     torch.testing.assert_close(whole.cpu(), want, atol=2e-4, rtol=1e-4)
-    assert not ops().wants_partials(torch.zeros(65, k, dtype=torch.bfloat16, device=DEV), w_d)
     assert not ops().wants_partials(x_d.float(), w_d.float())
+
+
+@pytest.mark.parametrize("m,n,k", [(17, 130, 264), (64, 3584, 1024), (300, 72, 2048), (129, 1152, 896),
+                                   (512, 896, 4864), (40, 1003, 4104)])
+def test_tiled_projection_partial_sums(m, n, k):
+    """More than 16 rows over a long K: tiles through LDS over slices of K, every slice with a
+    float32 result of its own; their sum is the product, for the planner's own number of
+    slices and for any other that the stages of K divide into."""
+    lib = ops()._lib.load("mfma")
+    x_h, x_d = as_dtype(rnd(m, k, seed=51), torch.bfloat16)
+    w_h, w_d = as_dtype(rnd(n, k, seed=52, scale=0.1), torch.bfloat16)
+    want = (x_h.double() @ w_h.double().T).float()
+    parts = ops().linear_partials(x_d, w_d)
+    assert parts.shape == (lib.mk_linear_tiled_slices(m, n, k), m, n)
+    torch.testing.assert_close(parts.sum(0).cpu(), want, atol=5e-4, rtol=1e-4)
+    stages = -(-k // 64)
+    for slices in (1, 2, 3, 5):
+        per = -(-stages // slices)
+        if -(-stages // per) != slices:
+            continue
+        out = torch.full((slices, m, n), 7.0, device=DEV)
+        ops()._lib.check(lib, lib.mk_linear_tiled_partials(
+            x_d.data_ptr(), w_d.data_ptr(), out.data_ptr(), m, n, k, slices,
+            torch.cuda.current_stream().cuda_stream), "partials")
+        torch.testing.assert_close(out.sum(0).cpu(), want, atol=5e-4, rtol=1e-4)
 
 
 @pytest.mark.parametrize("m,n,k", [(70, 130, 56), (129, 1152, 896), (300, 64, 264), (2048, 896, 4864),
