@@ -147,10 +147,10 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Te
 
 SKINNY_MAX_ROWS = 64
 SKINNY_SPLIT_MAX_ROWS = 16     # K-split partial sums: the skinny kernel up to here, tiles beyond
+SKINNY_SPLIT_MAX_WEIGHTS = 20 << 20   # bytes; larger matrices stream faster through the tiles' LDS ring
+TILED_MIN_ROWS = 8             # head and gated projection: the skinny kernel below, tiles from here
 FUSED_QKV_MAX_WEIGHTS = 48 << 20  # bytes; with more than 16 rows of x
-WIDE_MATRIX_COLUMNS = 8192
 FUSED_QKV_MIN_WORKGROUPS = 128
-GATED_TILED_MIN_ROWS, GATED_TILED_MIN_WEIGHTS = 33, 16 << 20
 
 
 def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -161,9 +161,17 @@ def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
         return False
     lib = _lib.load("mfma")
     m, (n, k) = x.shape[0], w.shape
-    if m <= SKINNY_SPLIT_MAX_ROWS:
+    if _partials_by_skinny(m, n, k):
         return not lib.mk_linear_skinny_unsplit(m, n, k)
     return lib.mk_linear_tiled_slices(m, n, k) > 1
+
+
+def _partials_by_skinny(m: int, n: int, k: int) -> bool:
+    """Few rows over a matrix of modest size: weights straight from HBM into the matrix cores.
+    More rows re-read x too often that way, and a large matrix streams faster through the
+    tiled kernel's ring of LDS buffers (5120 x 27648 at 8 rows: 57 against 50 us; 896 x 4864:
+    4.8 against 5.4)."""
+    return m <= SKINNY_SPLIT_MAX_ROWS and n * k * 2 < SKINNY_SPLIT_MAX_WEIGHTS
 
 
 def _mfma_eligible(x, w: torch.Tensor) -> bool:
@@ -177,15 +185,16 @@ def _skinny_eligible(x, w: torch.Tensor) -> bool:
 
 def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """Float32 partial sums [P, M, N] of x W^T over P slices of K; the consumer (rmsnorm,
-    rope_kv_write: their `partials` forms) adds them up in slice order.  At most 16 rows:
-    the weights stream straight into the matrix cores; more: tiles through LDS."""
+    rope_kv_write: their `partials` forms) adds them up in slice order.  At most 16 rows of
+    a matrix of modest size: the weights stream straight into the matrix cores; otherwise
+    tiles through LDS."""
     _dev(x, w)
     if not _mfma_eligible(x, w) or x.shape[1] != w.shape[1]:
         raise KernelArgumentError(f"linear_partials: x {tuple(x.shape)} / W {tuple(w.shape)} not eligible")
     m, k = x.shape
     n = w.shape[0]
     lib = _lib.load("mfma")
-    if m <= SKINNY_SPLIT_MAX_ROWS:
+    if _partials_by_skinny(m, n, k):
         slices = lib.mk_linear_skinny_slices(m, n, k)
         out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
         code = lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream())
@@ -216,10 +225,9 @@ def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor,
     inter = w_gate_up.shape[0] // 2
     act = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
     lib = _lib.load("mfma")
-    # 33 to 64 rows of a large matrix: the tiled kernel's shared x beats the skinny one's
-    # re-reads (measured at 18944 x 3584: 75 against 85 to 112 us)
-    skinny = m <= SKINNY_MAX_ROWS and not (m >= GATED_TILED_MIN_ROWS
-                                           and inter * k >= GATED_TILED_MIN_WEIGHTS)
+    # From 8 rows on the tiled kernel streams the weights faster than the skinny one
+    # (18944 x 3584 at 1, 8, 16, 32 rows: skinny 50, 57, 63, 80 us; tiles 55, 55, 55, 58).
+    skinny = m < TILED_MIN_ROWS
     if skinny and tile_config is None:
         code = lib.mk_gated_skinny(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream())
     else:
@@ -268,15 +276,15 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
         if x.dtype != torch.bfloat16 or k % 8:
             raise KernelArgumentError("linear: the matrix-core kernels take bfloat16 with K % 8 == 0")
         lib = _lib.load("mfma")
-        # Few rows straight from HBM into the matrix cores; from 17 rows on, a wide matrix
-        # (the head over the vocabulary) is faster through LDS tiles, which read x once per
-        # 64 or 128 columns instead of once per 32.
-        if (m <= SKINNY_MAX_ROWS and out_dtype == torch.float32 and bias is None and not accumulate
-                and (m <= 16 or n < WIDE_MATRIX_COLUMNS)):
+        # A few rows straight from HBM into the matrix cores; from 8 rows on the tiles' ring of
+        # LDS buffers streams the weights faster (the head, 152064 x 3584, at 1, 8, 16, 64
+        # rows: skinny 188, 204, 238, 429 us; tiles 187, 191, 198, 221).
+        if (m < TILED_MIN_ROWS and out_dtype == torch.float32 and bias is None
+                and not accumulate):
             _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, 1, _stream()),
                        "linear")
             return out
-        if m <= SKINNY_MAX_ROWS and accumulate:
+        if m <= SKINNY_SPLIT_MAX_ROWS and accumulate:
             _lib.check(lib, lib.mk_linear_skinny_acc(
                 _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
                 _ptr(out), m, n, k, _stream()), "linear")
