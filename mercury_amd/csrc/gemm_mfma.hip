@@ -1,24 +1,24 @@
 // bfloat16 projections on the matrix cores: y[M,N] = x[M,K] W[N,K]^T, float32 accumulate.
 //
-// Two kernels for the two regimes of an inference step:
+// Two kernels:
 //
-//  * skinny (M <= 64, decoding): the weights are read once, straight from HBM into the A
-//    operand of v_mfma_f32_16x16x32_bf16 (16 rows of W by 32 k per instruction); the few rows
-//    of x are the B operand and come out of the L2.  A workgroup owns 16 or 32 rows of W, its
-//    wavefronts taking the k-steps in turn.  Where those workgroups occupy the chip, or the
-//    matrix is too small for bandwidth to matter, a workgroup keeps all of K and finishes the
-//    job in its epilogue: adds into the float32 residual stream, gates (gate/up projection),
-//    or adds the bias, rotates and writes q and the paged cache (q/k/v projection).
-//    Otherwise K is split:
-//    every slice writes its own float32 partial result [slice, M, N], and whichever kernel
-//    consumes the projection (RMSNorm, rotary + cache write) adds the slices up in slice
-//    order, so results are reproducible.
+//  * skinny (at most 16 rows of x; the q/k/v projection up to 64): the weights are read once,
+//    straight from HBM into the A operand of v_mfma_f32_16x16x32_bf16 (16 rows of W by 32 k
+//    per instruction); the few rows of x are the B operand and come out of the L2.  A
+//    workgroup owns 16 or 32 rows of W, its wavefronts taking the k-steps in turn.  A
+//    workgroup that keeps all of K finishes the job in its epilogue: adds into the float32
+//    residual stream, gates (gate/up projection), or adds the bias, rotates and writes q and
+//    the paged cache (q/k/v projection).  Otherwise K is split: every slice writes its own
+//    float32 partial result [slice, M, N], and whichever kernel consumes the projection
+//    (RMSNorm, rotary + cache write) adds the slices up in slice order, so results are
+//    reproducible.  It is the kernel of choice for a handful of rows and matrices of modest
+//    size; from 8 rows on, and for large matrices, the tiled kernel streams weights faster.
 //
-//  * tiled (M > 64, prompts): tiles of y per workgroup (256 x 256 down to 64 x 64, whichever
-//    is estimated fastest for the problem), K in stages through a ring of LDS buffers that
-//    global memory is loaded into directly, several stages ahead of the products.
-//    Epilogues: bfloat16 store with bias, float32 store, float32 accumulate into the
-//    residual stream, or SiLU gating.
+//  * tiled: tiles of y per workgroup (256 x 256 down to 64 x 64, whichever is estimated
+//    fastest for the problem), K in stages through a ring of LDS buffers that global memory
+//    is loaded into directly, several stages ahead of the products.  Epilogues: bfloat16
+//    store with bias, float32 store, float32 accumulate into the residual stream, SiLU
+//    gating, or float32 partial sums over slices of K.
 //
 // In both, lane l of a wavefront holds row (l % 16) and k-slots (l / 16) * 8 .. + 8 of an
 // operand, so the four lanes of a row read 64 contiguous bytes per load instruction.
@@ -383,13 +383,16 @@ extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
 template <int NT, int EPI>
 static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream) {
   // 8 wavefronts where the grid is small; with 3 or 4 tiles of x rows they would not fit
-  // the register file.
+  // the register file.  More than 16 rows of x only for the q/k/v projection: the others
+  // take the tiled kernel there.
   constexpr int W = (EPI == SK_ACC || EPI == SK_QKV) ? 8 : SK_WAVES;
-  switch ((a.M + 15) / 16) {
-    case 1: gemm_skinny_kernel<1, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a); break;
-    case 2: gemm_skinny_kernel<2, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a); break;
-    case 3: gemm_skinny_kernel<3, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
-    default: gemm_skinny_kernel<4, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a); break;
+  const int tiles = (a.M + 15) / 16;
+  if (tiles == 1) {
+    gemm_skinny_kernel<1, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a);
+  } else if constexpr (EPI == SK_QKV) {
+    if (tiles == 2) gemm_skinny_kernel<2, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a);
+    else if (tiles == 3) gemm_skinny_kernel<3, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a);
+    else gemm_skinny_kernel<4, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a);
   }
 }
 
@@ -408,7 +411,7 @@ static SkinnyArgs skinny_args(const void* x, const void* w, void* out, int M, in
 
 extern "C" int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int K,
                                 int slices, hipStream_t stream) {
-  MK_REQUIRE(M >= 1 && M <= 64, "skinny projection: M=%d outside 1..64", M);
+  MK_REQUIRE(M >= 1 && M <= 16, "skinny projection: M=%d outside 1..16", M);
   MK_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny projection: K=%d must be a multiple of 8", K);
   const int steps = (K + 127) / 128;
   MK_REQUIRE(slices >= 1 && slices <= steps, "skinny projection: %d slices for %d steps", slices,
@@ -422,11 +425,11 @@ extern "C" int mk_linear_skinny(const void* x, const void* w, float* out, int M,
   return 0;
 }
 
-// out[M, N] (float32) += x W^T (+ bias), 1 <= M <= 64, all of K in each workgroup.
+// out[M, N] (float32) += x W^T (+ bias), 1 <= M <= 16, all of K in each workgroup.
 extern "C" int mk_linear_skinny_acc(const void* x, const void* w, const void* bias,
                                     int bias_dtype, float* out, int M, int N, int K,
                                     hipStream_t stream) {
-  MK_REQUIRE(M >= 1 && M <= 64, "skinny projection: M=%d outside 1..64", M);
+  MK_REQUIRE(M >= 1 && M <= 16, "skinny projection: M=%d outside 1..16", M);
   MK_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny projection: K=%d must be a multiple of 8", K);
   MK_REQUIRE(bias_dtype == MK_F32 || bias_dtype == MK_BF16, "skinny projection: bias dtype");
   SkinnyArgs a = skinny_args(x, w, out, M, N, K, (K + 127) / 128);
@@ -441,10 +444,10 @@ extern "C" int mk_linear_skinny_acc(const void* x, const void* w, const void* bi
   return 0;
 }
 
-// act[M, I] = silu(x Wg^T) * (x Wu^T) for W = [Wg | Wu] stacked as [2 I, K], 1 <= M <= 64.
+// act[M, I] = silu(x Wg^T) * (x Wu^T) for W = [Wg | Wu] stacked as [2 I, K], 1 <= M <= 16.
 extern "C" int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
                                hipStream_t stream) {
-  MK_REQUIRE(M >= 1 && M <= 64, "gated projection: M=%d outside 1..64", M);
+  MK_REQUIRE(M >= 1 && M <= 16, "gated projection: M=%d outside 1..16", M);
   MK_REQUIRE(inter > 0 && K > 0 && K % 8 == 0, "gated projection: K=%d must be a multiple of 8",
              K);
   launch_skinny<2, SK_GATED>(skinny_args(x, w, act, M, inter, K, (K + 127) / 128),

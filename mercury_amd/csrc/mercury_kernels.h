@@ -64,20 +64,20 @@ int mk_qkv_finish(const float* partials, int num_partials, long long partial_str
 
 // ---- library "mfma": bfloat16 kernels on the matrix cores
 
-// y = x W^T for 1 <= M <= 64 rows of x, K split into `slices` (ask mk_linear_skinny_slices
+// y = x W^T for 1 <= M <= 16 rows of x, K split into `slices` (ask mk_linear_skinny_slices
 // for a good count): out is float32 [slices, M, N], to be summed over the slices.
 int mk_linear_skinny_slices(int M, int N, int K);
 int mk_linear_skinny(const void* x, const void* w, float* out, int M, int N, int K, int slices,
                      hipStream_t stream);
 
-// out[M, N] (float32) += x W^T (+ bias) for 1 <= M <= 64, all of K in each workgroup;
-// mk_linear_skinny_unsplit says whether that keeps the chip busy for the shape.
+// out[M, N] (float32) += x W^T (+ bias) for 1 <= M <= 16, all of K in each workgroup;
+// mk_linear_skinny_unsplit says whether that is the faster form for the shape.
 int mk_linear_skinny_unsplit(int M, int N, int K);
 int mk_linear_skinny_acc(const void* x, const void* w, const void* bias, int bias_dtype,
                          float* out, int M, int N, int K, hipStream_t stream);
 
 // act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K],
-// 1 <= M <= 64.
+// 1 <= M <= 16.
 int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
                     hipStream_t stream);
 
