@@ -54,28 +54,87 @@ __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *(const uint4*)p
 //               position, q to `q_out`, k and v into the paged cache.  All of K.
 enum { SK_PARTIAL = 0, SK_GATED = 1, SK_ACC = 2, SK_QKV = 3 };
 
-struct SkinnyArgs {
+// Where the q/k/v projection's results go, and how they are rotated on the way.
+struct QkvTarget {
+  bf16_t* q_out;           // [M, n_q d]
+  const float* cos_table;  // [positions, d / 2]
+  const float* sin_table;
+  const int* positions;    // [M]
+  const int* token_seq;    // [M]
+  const int* block_table;
+  int table_stride;
+  bf16_t* k_cache;         // [pages, n_kv, page, d]
+  bf16_t* v_cache;         // [pages, n_kv, d, page]
+  int page_shift, n_q, n_kv, d, rotate;
+};
+
+struct SkinnyArgs : QkvTarget {
   const bf16_t* x;  // [M, K]
   const bf16_t* w;
   void* out;
   int M, N, K, steps_per_slice;
   const void* bias;  // SK_ACC, SK_QKV: [N] or null
   int bias_bf16;
-  // SK_QKV
-  bf16_t* q_out;
-  const float* cos_table;
-  const float* sin_table;
-  const int* positions;
-  const int* token_seq;
-  const int* block_table;
-  int table_stride;
-  bf16_t* k_cache;
-  bf16_t* v_cache;
-  int page_shift, n_q, n_kv, d, rotate;
 };
 
 __device__ __forceinline__ float load_scalar(const void* p, int is_bf16, int i) {
   return is_bf16 ? bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
+}
+
+// Token m's values (bias added) at dims dd .. dd + 4 (`lo`) and dd + d/2 .. (`hi`) of head
+// `head` of [q heads | k heads | v heads]: rounded to bfloat16 as a stored projection would
+// be, q and k rotated by the token's position (the four lanes' dims are 4 rotation pairs), q
+// written to q_out, k and v into the paged cache.
+// Formulas: reference mercury/model/qwen2.py:57-64, mercury/model/rope.py:19-29.
+__device__ __forceinline__ void qkv_store(const QkvTarget& p, int m, int head, int dd, float* lo,
+                                          float* hi) {
+  const int d = p.d, half = d / 2;
+  const int pos = p.positions[m];
+#pragma unroll
+  for (int i = 0; i < 4; ++i) {
+    lo[i] = Elem<bf16_t>::round(lo[i]);
+    hi[i] = Elem<bf16_t>::round(hi[i]);
+  }
+  const bool is_v = head >= p.n_q + p.n_kv;
+  if (p.rotate && !is_v) {
+    const float4 c = *(const float4*)(p.cos_table + (size_t)pos * half + dd);
+    const float4 s = *(const float4*)(p.sin_table + (size_t)pos * half + dd);
+    const float cs[4] = {c.x, c.y, c.z, c.w}, sn[4] = {s.x, s.y, s.z, s.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      const float u = lo[i], v = hi[i];
+      lo[i] = u * cs[i] - v * sn[i];
+      hi[i] = v * cs[i] + u * sn[i];
+    }
+  }
+  const ushort4 lo4 = make_ushort4(f32_to_bf16(lo[0]), f32_to_bf16(lo[1]), f32_to_bf16(lo[2]),
+                                   f32_to_bf16(lo[3]));
+  const ushort4 hi4 = make_ushort4(f32_to_bf16(hi[0]), f32_to_bf16(hi[1]), f32_to_bf16(hi[2]),
+                                   f32_to_bf16(hi[3]));
+  if (head < p.n_q) {
+    bf16_t* dst = p.q_out + (size_t)m * p.n_q * d + head * d + dd;
+    *(ushort4*)dst = lo4;
+    *(ushort4*)(dst + half) = hi4;
+    return;
+  }
+  const int page = p.block_table[(size_t)p.token_seq[m] * p.table_stride + (pos >> p.page_shift)];
+  if (page < 0) return;
+  const int ps = 1 << p.page_shift, off = pos & (ps - 1);
+  if (!is_v) {
+    const int kh = head - p.n_q;
+    bf16_t* dst = p.k_cache + (((size_t)page * p.n_kv + kh) * ps + off) * d + dd;
+    *(ushort4*)dst = lo4;
+    *(ushort4*)(dst + half) = hi4;
+  } else {
+    const int vh = head - p.n_q - p.n_kv;
+    bf16_t* dst = p.v_cache + (((size_t)page * p.n_kv + vh) * d + dd) * ps + off;
+    const bf16_t l[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, h4[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+      dst[(size_t)i * ps] = l[i];
+      dst[(size_t)(half + i) * ps] = h4[i];
+    }
+  }
 }
 
 // One workgroup: NT tiles of 16 rows of W, its four wavefronts taking the slice's 128-wide
@@ -249,59 +308,18 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
       }
     } else if constexpr (EPI == SK_QKV) {
       // Both halves of 4 rotation pairs of one head: dims dd.. and dd + d/2..
-      const int d = p.d, half = d / 2, dd = dd0 + g4 * 4;
-      const int pos = p.positions[m];
+      const int half = p.d / 2, dd = dd0 + g4 * 4;
       float lo[4], hi[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float u = acc[0][tb][i], v = acc[1][tb][i];
+        lo[i] = acc[0][tb][i];
+        hi[i] = acc[1][tb][i];
         if (p.bias) {
-          u += load_scalar(p.bias, p.bias_bf16, n0 + g4 * 4 + i);
-          v += load_scalar(p.bias, p.bias_bf16, n0 + half + g4 * 4 + i);
-        }
-        lo[i] = Elem<bf16_t>::round(u);
-        hi[i] = Elem<bf16_t>::round(v);
-      }
-      const bool is_v = head >= p.n_q + p.n_kv;
-      if (p.rotate && !is_v) {
-        const float4 c = *(const float4*)(p.cos_table + (size_t)pos * half + dd);
-        const float4 s = *(const float4*)(p.sin_table + (size_t)pos * half + dd);
-        const float cs[4] = {c.x, c.y, c.z, c.w}, sn[4] = {s.x, s.y, s.z, s.w};
-#pragma unroll
-        for (int i = 0; i < 4; ++i) {
-          const float u = lo[i], v = hi[i];
-          lo[i] = u * cs[i] - v * sn[i];
-          hi[i] = v * cs[i] + u * sn[i];
+          lo[i] += load_scalar(p.bias, p.bias_bf16, n0 + g4 * 4 + i);
+          hi[i] += load_scalar(p.bias, p.bias_bf16, n0 + half + g4 * 4 + i);
         }
       }
-      const ushort4 lo4 = make_ushort4(f32_to_bf16(lo[0]), f32_to_bf16(lo[1]), f32_to_bf16(lo[2]),
-                                       f32_to_bf16(lo[3]));
-      const ushort4 hi4 = make_ushort4(f32_to_bf16(hi[0]), f32_to_bf16(hi[1]), f32_to_bf16(hi[2]),
-                                       f32_to_bf16(hi[3]));
-      if (head < p.n_q) {
-        bf16_t* dst = p.q_out + (size_t)m * p.n_q * d + head * d + dd;
-        *(ushort4*)dst = lo4;
-        *(ushort4*)(dst + half) = hi4;
-      } else {
-        const int page = p.block_table[(size_t)p.token_seq[m] * p.table_stride + (pos >> p.page_shift)];
-        if (page < 0) continue;
-        const int ps = 1 << p.page_shift, off = pos & (ps - 1);
-        if (!is_v) {
-          const int kh = head - p.n_q;
-          bf16_t* dst = p.k_cache + (((size_t)page * p.n_kv + kh) * ps + off) * d + dd;
-          *(ushort4*)dst = lo4;
-          *(ushort4*)(dst + half) = hi4;
-        } else {
-          const int vh = head - p.n_q - p.n_kv;
-          bf16_t* dst = p.v_cache + (((size_t)page * p.n_kv + vh) * d + dd) * ps + off;
-          const bf16_t l[4] = {lo4.x, lo4.y, lo4.z, lo4.w}, h4[4] = {hi4.x, hi4.y, hi4.z, hi4.w};
-#pragma unroll
-          for (int i = 0; i < 4; ++i) {
-            dst[(size_t)i * ps] = l[i];
-            dst[(size_t)(half + i) * ps] = h4[i];
-          }
-        }
-      }
+      qkv_store(p, m, head, dd, lo, hi);
     } else {
       float* dst = (float*)p.out + ((size_t)(EPI == SK_PARTIAL ? slice : 0) * M + m) * N;
 #pragma unroll
@@ -501,7 +519,7 @@ extern "C" int mk_qkv_skinny(const void* x, const void* w, const void* bias, int
 
 // ------------------------------------------------------------------------------- tiled
 
-enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3 };
+enum { EPI_BF16 = 0, EPI_F32 = 1, EPI_ACC = 2, EPI_GATED = 3, EPI_QKV = 4 };
 
 #define TILE_K 64  // k per stage: a tile row is 128 bytes in LDS, one cache line of the operand
 
@@ -540,22 +558,29 @@ __device__ __forceinline__ bf16_t* tiled_stage_buffer() {
 // EPI_GATED: W is [gate rows | up rows] of N each.  A wavefront's BN / WN tile rows are half
 // gate rows and half the matching up rows, so its accumulators hold both; the epilogue writes
 // act[m][n] = silu(g) * u in bfloat16 (reference: mercury/model/qwen2.py:42).
+//
+// EPI_QKV: W is [q heads | k heads | v heads] of d rows each.  A wavefront's tile rows are
+// half rows from the first halves of heads and half the rows d / 2 further, so its
+// accumulators hold both members of every rotation pair; the epilogue adds the bias,
+// rotates, and writes q and the paged cache (qkv_store).  N counts the rows of W.
 template <int BM, int BN, int STAGES, int WM, int WN, int SPREAD, int EPI, typename TBIAS>
 __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* __restrict__ x,
                                                                   const bf16_t* __restrict__ w,
                                                                   const TBIAS* __restrict__ bias,
                                                                   void* __restrict__ out_, int M,
                                                                   int N, int K, int ldo,
-                                                                  int slice_stages) {
+                                                                  int slice_stages,
+                                                                  QkvTarget target) {
   constexpr int WAVES = WM * WN, TK = TILE_K;
   constexpr int NI = (BM + BN) / 8 / WAVES;                 // load instructions per wavefront and stage
   static_assert((BM + BN) % (8 * WAVES) == 0 && WAVES % 2 == 0, "tile rows divide over the wavefronts");
   static_assert(BM % 16 == 0 && (STAGES - 2) * NI < 64, "tile shape");
   constexpr int ELEMS = (BM + BN) * TK;
   constexpr int TM = BM / WM / 16, TN = BN / WN / 16;       // MFMA tiles per wavefront
-  static_assert(EPI != EPI_GATED || TN % 2 == 0, "gating needs gate and up tiles in one wavefront");
+  constexpr bool PAIRED = EPI == EPI_GATED || EPI == EPI_QKV;
+  static_assert(!PAIRED || TN % 2 == 0, "both members of a pair of rows in one wavefront");
   constexpr int WIDTH = BN / WN;                            // W rows per wavefront
-  constexpr int COLS = EPI == EPI_GATED ? BN / 2 : BN;      // output columns per tile
+  constexpr int COLS = PAIRED ? BN / 2 : BN;                // output columns (pairs) per tile
   // Where the 8 elements from k-chunk `chunk` of tile row `row` lie in a stage buffer.
   auto lds_at = [](int row, int chunk) { return row * TK + (((chunk ^ (row >> 1)) & 7) << 3); };
 
@@ -598,6 +623,10 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
       if (EPI == EPI_GATED) {  // per wavefront: WIDTH / 2 gate rows, then the matching up rows
         const int col = min(n0 + wrow / WIDTH * (WIDTH / 2) + wrow % (WIDTH / 2), N - 1);
         wrow = (wrow % WIDTH < WIDTH / 2 ? 0 : N) + col;
+      } else if (EPI == EPI_QKV) {  // WIDTH / 2 rows of heads' first halves, then their partners
+        const int half = target.d / 2;
+        const int pair = min(n0 + wrow / WIDTH * (WIDTH / 2) + wrow % (WIDTH / 2), N / 2 - 1);
+        wrow = pair / half * target.d + pair % half + (wrow % WIDTH < WIDTH / 2 ? 0 : half);
       } else {
         wrow = min(n0 + wrow, N - 1);
       }
@@ -696,6 +725,27 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
   for (int ta = 0; ta < TM; ++ta) {
     const int m = m0 + wm + ta * 16 + r;
     if (m >= M) continue;
+    if (EPI == EPI_QKV) {
+      const int half = target.d / 2;
+#pragma unroll
+      for (int tb = 0; tb < TN / 2; ++tb) {
+        const int pair = n0 + wn / 2 + tb * 16 + g4 * 4;    // 4 pairs, all of one head
+        if (pair >= N / 2) continue;
+        const int head = pair / half, dd = pair % half;
+        float lo[4], hi[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          lo[i] = acc[ta][tb][i];
+          hi[i] = acc[ta][tb + TN / 2][i];
+          if (bias != nullptr) {
+            lo[i] += Elem<TBIAS>::load(bias + head * target.d + dd + i);
+            hi[i] += Elem<TBIAS>::load(bias + head * target.d + half + dd + i);
+          }
+        }
+        qkv_store(target, m, head, dd, lo, hi);
+      }
+      continue;
+    }
     if (EPI == EPI_GATED) {
 #pragma unroll
       for (int tb = 0; tb < TN / 2; ++tb) {
@@ -780,30 +830,31 @@ static const TiledConfig tiled_configs[TILED_CONFIGS] = {
 template <int BM, int BN, int STAGES, int WM, int WN, int SPREAD, int EPI>
 static void launch_tiled_cfg(const void* x, const void* w, const void* bias, int bias_dtype,
                              void* out, int M, int N, int K, int ldo, int slices,
-                             hipStream_t stream) {
-  constexpr int COLS = EPI == EPI_GATED ? BN / 2 : BN;
+                             const QkvTarget& target, hipStream_t stream) {
+  constexpr int COLS = (EPI == EPI_GATED || EPI == EPI_QKV) ? BN / 2 : BN;
+  const int cols = EPI == EPI_QKV ? N / 2 : N;   // q/k/v: the grid counts pairs of rows
   const int all_steps = (K + TILE_K - 1) / TILE_K;
   const int slice_stages = (all_steps + slices - 1) / slices;
-  dim3 grid((N + COLS - 1) / COLS, (M + BM - 1) / BM, (all_steps + slice_stages - 1) / slice_stages);
+  dim3 grid((cols + COLS - 1) / COLS, (M + BM - 1) / BM, (all_steps + slice_stages - 1) / slice_stages);
   if (bias && bias_dtype == MK_BF16)
     gemm_tiled_kernel<BM, BN, STAGES, WM, WN, SPREAD, EPI, bf16_t><<<grid, 64 * WM * WN, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, out, M, N, K, ldo, slice_stages);
+        (const bf16_t*)x, (const bf16_t*)w, (const bf16_t*)bias, out, M, N, K, ldo, slice_stages, target);
   else
     gemm_tiled_kernel<BM, BN, STAGES, WM, WN, SPREAD, EPI, float><<<grid, 64 * WM * WN, 0, stream>>>(
-        (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo, slice_stages);
+        (const bf16_t*)x, (const bf16_t*)w, (const float*)bias, out, M, N, K, ldo, slice_stages, target);
 }
 
 template <int EPI>
 static void launch_tiled(int config, const void* x, const void* w, const void* bias,
                          int bias_dtype, void* out, int M, int N, int K, int ldo, int slices,
-                         hipStream_t stream) {
+                         hipStream_t stream, const QkvTarget& target = QkvTarget()) {
   switch (config) {
-    case 0: launch_tiled_cfg<256, 256, 2, 4, 4, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
-    case 1: launch_tiled_cfg<128, 256, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
-    case 2: launch_tiled_cfg<128, 128, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
-    case 3: launch_tiled_cfg<128, 128, 2, 2, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
-    case 4: launch_tiled_cfg<64, 64, 4, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
-    default: launch_tiled_cfg<64, 128, 4, 1, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, stream); break;
+    case 0: launch_tiled_cfg<256, 256, 2, 4, 4, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    case 1: launch_tiled_cfg<128, 256, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    case 2: launch_tiled_cfg<128, 128, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    case 3: launch_tiled_cfg<128, 128, 2, 2, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    case 4: launch_tiled_cfg<64, 64, 4, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    default: launch_tiled_cfg<64, 128, 4, 1, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
   }
 }
 
@@ -902,6 +953,47 @@ extern "C" int mk_gated_tiled(const void* x, const void* w, void* act, int M, in
   MK_REQUIRE(config < TILED_CONFIGS, "gated projection: no configuration %d", config);
   launch_tiled<EPI_GATED>(config, x, w, nullptr, MK_F32, act, M, inter, K, inter, 1, stream);
   MK_LAUNCH_CHECK("gated_tiled");
+  return 0;
+}
+
+// The q/k/v projection of any number of tokens with everything that follows it, as
+// mk_qkv_skinny: bias, rotation of q and k by the token's position (full head width, or
+// none), q [M, n_q d] out, k and v into the paged cache (n_kv = 0: queries only).
+extern "C" int mk_qkv_tiled(const void* x, const void* w, const void* bias, int bias_dtype,
+                            void* q_out, const float* cos_table, const float* sin_table,
+                            int table_positions, const int* positions, const int* token_seq,
+                            const int* block_table, int table_stride, void* k_cache,
+                            void* v_cache, int page_size, int n_q, int n_kv, int d, int rotate,
+                            int M, int K, int config, hipStream_t stream) {
+  MK_REQUIRE(M >= 1 && (M + 63) / 64 <= 65535, "qkv projection: M=%d", M);
+  MK_REQUIRE(n_q > 0 && n_kv >= 0 && d > 0 && d % 32 == 0,
+             "qkv projection: head size %d is not a multiple of 32", d);
+  MK_REQUIRE(K > 0 && K % 8 == 0, "qkv projection: K=%d must be a multiple of 8", K);
+  MK_REQUIRE(!rotate || (cos_table && sin_table && table_positions > 0),
+             "qkv projection: rotation needs the angle tables");
+  MK_REQUIRE(n_kv == 0 || (k_cache && v_cache && block_table && mk_is_pow2(page_size)),
+             "qkv projection: the cache and a power-of-two page size are required");
+  MK_REQUIRE(bias_dtype == MK_F32 || bias_dtype == MK_BF16, "qkv projection: bias dtype");
+  const int N = (n_q + 2 * n_kv) * d;
+  QkvTarget t = {};
+  t.q_out = (bf16_t*)q_out;
+  t.cos_table = cos_table;
+  t.sin_table = sin_table;
+  t.positions = positions;
+  t.token_seq = token_seq;
+  t.block_table = block_table;
+  t.table_stride = table_stride;
+  t.k_cache = (bf16_t*)k_cache;
+  t.v_cache = (bf16_t*)v_cache;
+  t.page_shift = mk_log2(page_size > 0 ? page_size : 1);
+  t.n_q = n_q;
+  t.n_kv = n_kv;
+  t.d = d;
+  t.rotate = rotate;
+  if (config < 0) config = tiled_config_for(M, N / 2, K, 2, 2);
+  MK_REQUIRE(config < TILED_CONFIGS, "qkv projection: no configuration %d", config);
+  launch_tiled<EPI_QKV>(config, x, w, bias, bias_dtype, nullptr, M, N, K, N, 1, stream, t);
+  MK_LAUNCH_CHECK("qkv_tiled");
   return 0;
 }
 

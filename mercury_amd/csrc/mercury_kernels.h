@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 6
+#define MK_ABI_VERSION 7
 
 #ifdef __cplusplus
 extern "C" {
@@ -90,8 +90,16 @@ int mk_qkv_skinny(const void* x, const void* w, const void* bias, int bias_dtype
                   int table_stride, void* k_cache, void* v_cache, int page_size, int n_q,
                   int n_kv, int d, int rotate, int M, int K, hipStream_t stream);
 
-// The same for any M, tiled through LDS; config: a tile configuration, -1 for the one
-// estimated fastest.
+// The q/k/v projection as mk_qkv_skinny, for any M, tiled through LDS; config: a tile
+// configuration, -1 for the one estimated fastest.
+int mk_qkv_tiled(const void* x, const void* w, const void* bias, int bias_dtype, void* q_out,
+                 const float* cos_table, const float* sin_table, int table_positions,
+                 const int* positions, const int* token_seq, const int* block_table,
+                 int table_stride, void* k_cache, void* v_cache, int page_size, int n_q,
+                 int n_kv, int d, int rotate, int M, int K, int config, hipStream_t stream);
+
+// The gated projection for any M, tiled through LDS; config: a tile configuration, -1 for the
+// one estimated fastest.
 int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K, int config,
                    hipStream_t stream);
 

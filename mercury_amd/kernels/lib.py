@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 
 from . import build
 
-ABI_VERSION = 6
+ABI_VERSION = 7
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -36,6 +36,7 @@ _SIGNATURES = {
         "mk_linear_skinny_acc": [P, P, P, I, P, I, I, I, P],
         "mk_gated_skinny": [P, P, P, I, I, I, P],
         "mk_qkv_skinny": [P, P, P, I, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
+        "mk_qkv_tiled": [P, P, P, I, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, P],
         "mk_gated_tiled": [P, P, P, I, I, I, I, P],
         "mk_linear_tiled_slices": [I, I, I],
         "mk_linear_tiled_partials": [P, P, P, I, I, I, I, P],

@@ -395,44 +395,61 @@ def _qkv_finish(parts, cos, sin, positions, token_seq, block_table, k_cache, v_c
 
 
 def _qkv_fusable(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
-    return (_skinny_eligible(x, w) and head_dim % 32 == 0 and rotary_dim in (0, head_dim)
+    return (_mfma_eligible(x, w) and head_dim % 32 == 0 and rotary_dim in (0, head_dim)
             and page_size > 0 and page_size & (page_size - 1) == 0)
 
 
 def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
-    """Whether `qkv_project` runs as one kernel by itself: few bfloat16 rows, K a multiple of
-    8, heads a multiple of 32 wide and rotated over their whole width or not at all, pages a
-    power of two; and, as that kernel has one workgroup per 32 rows of W with all of K, more
-    than 16 rows of x only where those workgroups are many and the matrix is not so large
-    that tiles over slices of K stream it faster (7168 x 5120 at 64 rows: 43 us in one
-    kernel, 20 + 7 in two)."""
-    return (_qkv_fusable(x, w, head_dim, rotary_dim, page_size)
-            and (x.shape[0] <= 16 or (w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS
-                                      and w.numel() * 2 <= FUSED_QKV_MAX_WEIGHTS)))
+    """Whether `qkv_project` runs as one kernel by itself: bfloat16 rows, K a multiple of 8,
+    heads a multiple of 32 wide and rotated over their whole width or not at all, pages a
+    power of two; and not 17 to a few hundred rows over a matrix so large that tiles over
+    slices of K, followed by the rotation, stream it faster (7168 x 5120 at 64 rows: 43 us in
+    one kernel, 20 + 7 in two)."""
+    return _qkv_kernel(x, w, head_dim, rotary_dim, page_size) is not None
+
+
+def _qkv_kernel(x, w, head_dim, rotary_dim, page_size):
+    """ "skinny" (up to 64 rows: weights straight into the matrix cores, one workgroup per 32
+    rows of W with all of K), "tiled" (any number of rows, through LDS), or None."""
+    if not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
+        return None
+    m = x.shape[0]
+    if m <= 16 or (m <= SKINNY_MAX_ROWS and w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS
+                   and w.numel() * 2 <= FUSED_QKV_MAX_WEIGHTS):
+        return "skinny"
+    if m > SKINNY_MAX_ROWS and not wants_partials(x, w):
+        return "tiled"
+    return None
 
 
 def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor | None,
                 sin: torch.Tensor | None, positions: torch.Tensor, token_seq: torch.Tensor,
                 block_table: torch.Tensor, k_cache: torch.Tensor | None,
                 v_cache: torch.Tensor | None, n_q: int, n_kv: int, head_dim: int,
-                rotary_dim: int, write_kv: bool = True, fused: bool | None = None) -> torch.Tensor:
+                rotary_dim: int, write_kv: bool = True, fused: bool | None = None,
+                tile_config: int = -1) -> torch.Tensor:
     """q, k, v = x W^T + bias for W = [q heads | k heads | v heads]; q and k rotated by their
     positions; k and v written to the paged cache (`write_kv`; otherwise W holds the query
     heads only).  Returns the rotated q [T, n_q d].
 
-    Few rows take one kernel (projection, bias, rotation and cache write in its epilogue);
-    otherwise the projection is followed by `rope_kv_write`.  `fused` forces one or the
-    other."""
+    Where `fuses_qkv` says so, one kernel does all of it (projection, bias, rotation and cache
+    write in its epilogue: the skinny kernel for few rows, the tiled one for many); otherwise
+    the projection (whole or as partial sums) is followed by `rope_kv_write`.  `fused` forces
+    one or the other, `tile_config` a tile configuration of the tiled kernel."""
     heads_kv = n_kv if write_kv else 0
     width = (n_q + 2 * heads_kv) * head_dim
     if w.shape[0] != width or w.shape[1] != x.shape[1]:
         raise KernelArgumentError(f"qkv_project: W {tuple(w.shape)} is not [{width}, {x.shape[1]}]")
     page_size = k_cache.shape[2] if write_kv and k_cache is not None else 1
     if fused is None:
-        fused = fuses_qkv(x, w, head_dim, rotary_dim, page_size)
-    elif fused and not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
+        kernel = _qkv_kernel(x, w, head_dim, rotary_dim, page_size)
+    elif not fused:
+        kernel = None
+    elif not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
         raise KernelArgumentError("qkv_project: these operands cannot take the fused kernel")
-    if not fused:
+    else:
+        kernel = "skinny" if x.shape[0] <= SKINNY_MAX_ROWS and tile_config < 0 else "tiled"
+    if kernel is None:
         if wants_partials(x, w):
             return rope_kv_write(linear_partials(x, w), cos, sin, positions, token_seq,
                                  block_table, k_cache, v_cache, n_q, heads_kv, head_dim,
@@ -458,12 +475,16 @@ def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor
         _check_caches("qkv_project", k_cache, v_cache, n_kv, head_dim, torch.bfloat16)
     q = torch.empty((tokens, n_q * head_dim), dtype=torch.bfloat16, device=w.device)
     lib = _lib.load("mfma")
-    _lib.check(lib, lib.mk_qkv_skinny(
-        _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32, _ptr(q),
-        _ptr(cos), _ptr(sin), table_positions, _ptr(positions), _ptr(token_seq),
-        _ptr(block_table), block_table.shape[1], _ptr(k_cache) if write_kv else 0,
-        _ptr(v_cache) if write_kv else 0, page_size, n_q, heads_kv, head_dim,
-        int(rotary_dim > 0), tokens, k, _stream()), "qkv_project")
+    args = (_ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
+            _ptr(q), _ptr(cos), _ptr(sin), table_positions, _ptr(positions), _ptr(token_seq),
+            _ptr(block_table), block_table.shape[1], _ptr(k_cache) if write_kv else 0,
+            _ptr(v_cache) if write_kv else 0, page_size, n_q, heads_kv, head_dim,
+            int(rotary_dim > 0), tokens, k)
+    if kernel == "skinny":
+        code = lib.mk_qkv_skinny(*args, _stream())
+    else:
+        code = lib.mk_qkv_tiled(*args, tile_config, _stream())
+    _lib.check(lib, code, "qkv_project")
     return q
 
 

@@ -292,15 +292,16 @@ def test_skinny_projection_into_the_stream(m, n, k, bias_dtype):
 
 QKV_CASES = [  # n_q, n_kv, d, page, K, rows
     (14, 2, 64, 16, 896, 8), (6, 1, 32, 8, 168, 1), (4, 4, 128, 32, 264, 17), (3, 1, 96, 16, 72, 64),
-    (2, 2, 64, 16, 64, 16)]
+    (2, 2, 64, 16, 64, 16), (14, 2, 64, 32, 896, 200), (4, 4, 128, 32, 264, 130)]
 
 
 @pytest.mark.parametrize("n_q,n_kv,d,page,k,m", QKV_CASES)
 @pytest.mark.parametrize("mode", ["plain", "unrotated", "queries_only"])
 def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(n_q, n_kv, d, page, k, m, mode):
-    """The fused q/k/v kernel for few rows equals projection, then rotary + cache write, and
-    the plain implementation; tokens sit on page edges, in several sequences, one of them on
-    a page that was given back."""
+    """The fused q/k/v kernels (the skinny one for few rows, the tiled one in every tile
+    configuration for any number) equal projection, then rotary + cache write, and the plain
+    implementation; tokens sit on page edges, in several sequences, one of them on a page
+    that was given back."""
     o = ops()
     write_kv = mode != "queries_only"
     rot = 0 if mode == "unrotated" else d
@@ -330,7 +331,8 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(n_q, n_kv, d
                torch.zeros(32, n_kv, d, page, dtype=torch.bfloat16, device=DEV)] for _ in range(2)]
     x_h, x_d = as_dtype(rnd(m, k, seed=55), torch.bfloat16)
     x_in = x_d
-    assert o.fuses_qkv(x_in, w_d, d, rot, page) == (m <= 16)    # few workgroups: only for few rows
+    if m <= 64:
+        assert o.fuses_qkv(x_in, w_d, d, rot, page) == (m <= 16)    # few workgroups: only for few rows
     cos_d, sin_d = (cos.to(DEV), sin.to(DEV)) if rot else (None, None)
     q_got = o.qkv_project(x_in, w_d, b_d, cos_d, sin_d, pos_d, seq_d, table.to(DEV),
                           caches[0][0] if write_kv else None, caches[0][1] if write_kv else None,
@@ -350,6 +352,16 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(n_q, n_kv, d
         assert (caches[0][0] != 0).eq(caches[1][0] != 0).all()      # the same slots, no others
         assert (caches[0][1] != 0).eq(caches[1][1] != 0).all()
         assert caches[0][0].abs().sum() > 0
+    for config in range(o._lib.load("mfma").mk_linear_tiled_configs()):
+        tiled = [torch.zeros_like(caches[0][0]), torch.zeros_like(caches[0][1])]
+        q_tiled = o.qkv_project(x_in, w_d, b_d, cos_d, sin_d, pos_d, seq_d, table.to(DEV),
+                                tiled[0] if write_kv else None, tiled[1] if write_kv else None,
+                                n_q, n_kv, d, rot, write_kv, fused=True, tile_config=config)
+        torch.testing.assert_close(q_tiled.float().cpu(), q_ref.float().cpu(), **bf)
+        if write_kv:
+            torch.testing.assert_close(tiled[0].float().cpu(), caches[1][0].float().cpu(), **bf)
+            torch.testing.assert_close(tiled[1].float().cpu(), caches[1][1].float().cpu(), **bf)
+            assert (tiled[0] != 0).eq(caches[1][0] != 0).all() and (tiled[1] != 0).eq(caches[1][1] != 0).all()
     # and the plain implementation, from the formulas
     y = ((x_h.double() @ w_h.double().T).float() + b_h).to(torch.bfloat16).float()
     q = y[:, : n_q * d].view(m, n_q, d)
@@ -364,9 +376,9 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(n_q, n_kv, d
         v_want = y[:, (n_q + n_kv) * d:].view(m, n_kv, d)
         for t in range(m):
             pg, off = int(table[token_seq[t], positions[t] // page]), positions[t] % page
-            if t == dropped:
-                assert pg < 0
+            if pg < 0:          # the page that was given back, and whoever else sits on it
                 continue
+            assert t != dropped
             torch.testing.assert_close(caches[0][0][pg, :, off].float().cpu(), k_want[t], **bf)
             torch.testing.assert_close(caches[0][1][pg, :, :, off].float().cpu(), v_want[t], **bf)
 
@@ -381,7 +393,8 @@ def test_qkv_projection_falls_back_where_the_fused_kernel_does_not_apply():
     assert not o.fuses_qkv(x, x, 48, 48, 16)          # heads not a multiple of 32 wide
     assert not o.fuses_qkv(x, x, 64, 32, 16)          # rotation over part of the head
     assert not o.fuses_qkv(x.float(), x.float(), 64, 64, 16)
-    assert not o.fuses_qkv(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), x, 64, 64, 16)
+    assert o.fuses_qkv(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), x, 64, 64, 16)  # tiles
+    assert not o.fuses_qkv(torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV), x, 48, 48, 16)
 
 
 def test_matrix_core_projection_refuses_what_it_cannot_do():
