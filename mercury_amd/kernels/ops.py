@@ -410,14 +410,15 @@ def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int
 
 def _qkv_kernel(x, w, head_dim, rotary_dim, page_size):
     """ "skinny" (up to 64 rows: weights straight into the matrix cores, one workgroup per 32
-    rows of W with all of K), "tiled" (any number of rows, through LDS), or None."""
+    rows of W with all of K), "tiled" (any number of rows, through LDS, where whole-K tiles
+    are the faster projection anyway), or None."""
     if not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
         return None
     m = x.shape[0]
     if m <= 16 or (m <= SKINNY_MAX_ROWS and w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS
                    and w.numel() * 2 <= FUSED_QKV_MAX_WEIGHTS):
         return "skinny"
-    if m > SKINNY_MAX_ROWS and not wants_partials(x, w):
+    if not wants_partials(x, w):
         return "tiled"
     return None
 

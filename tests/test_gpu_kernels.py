@@ -331,8 +331,7 @@ def test_qkv_projection_with_rotation_and_cache_write_in_one_kernel(n_q, n_kv, d
                torch.zeros(32, n_kv, d, page, dtype=torch.bfloat16, device=DEV)] for _ in range(2)]
     x_h, x_d = as_dtype(rnd(m, k, seed=55), torch.bfloat16)
     x_in = x_d
-    if m <= 64:
-        assert o.fuses_qkv(x_in, w_d, d, rot, page) == (m <= 16)    # few workgroups: only for few rows
+    assert o.fuses_qkv(x_in, w_d, d, rot, page)
     cos_d, sin_d = (cos.to(DEV), sin.to(DEV)) if rot else (None, None)
     q_got = o.qkv_project(x_in, w_d, b_d, cos_d, sin_d, pos_d, seq_d, table.to(DEV),
                           caches[0][0] if write_kv else None, caches[0][1] if write_kv else None,
@@ -388,7 +387,9 @@ def test_qkv_projection_falls_back_where_the_fused_kernel_does_not_apply():
     x = torch.zeros(4, 64, dtype=torch.bfloat16, device=DEV)
     many = torch.zeros(40, 64, dtype=torch.bfloat16, device=DEV)
     assert o.fuses_qkv(x, torch.zeros(512, 64, dtype=torch.bfloat16, device=DEV), 64, 64, 16)
-    assert not o.fuses_qkv(many, torch.zeros(512, 64, dtype=torch.bfloat16, device=DEV), 64, 64, 16)
+    assert o.fuses_qkv(many, torch.zeros(512, 64, dtype=torch.bfloat16, device=DEV), 64, 64, 16)
+    big = torch.zeros(7168, 5120, dtype=torch.bfloat16, device=DEV)
+    assert not o.fuses_qkv(torch.zeros(64, 5120, dtype=torch.bfloat16, device=DEV), big, 128, 128, 16)
     assert o.fuses_qkv(many, torch.zeros(4608, 64, dtype=torch.bfloat16, device=DEV), 128, 128, 16)
     assert not o.fuses_qkv(x, x, 48, 48, 16)          # heads not a multiple of 32 wide
     assert not o.fuses_qkv(x, x, 64, 32, 16)          # rotation over part of the head
