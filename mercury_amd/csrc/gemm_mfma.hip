@@ -905,8 +905,11 @@ static void tiled_plan_sliced(int M, int N, int K, int* config, int* slices) {
     for (int s = 1; s <= 16 && (s == 1 || all_steps / s >= 8); ++s) {
       const int per = (all_steps + s - 1) / s;
       if ((all_steps + per - 1) / per != s) continue;
-      // a slice more costs its share of writing and re-reading the partial results
-      const double time = tiled_time(tiled_configs[c], M, N, K, 1, 4, s) * (1.0 + 0.02 * (s - 1));
+      // a slice more costs a little by itself, and whoever adds the partial results up has to
+      // read them (just written, they come at about 7 TB/s)
+      const double adding = s > 1 ? (double)s * M * N * 4.0 / 7e6 : 0.0;
+      const double time =
+          tiled_time(tiled_configs[c], M, N, K, 1, 4, s) * (1.0 + 0.02 * (s - 1)) + adding;
       if (*config < 0 || time < best_time) *config = c, *slices = s, best_time = time;
     }
   }

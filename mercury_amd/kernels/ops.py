@@ -150,6 +150,7 @@ SKINNY_SPLIT_MAX_ROWS = 16     # K-split partial sums: the skinny kernel up to h
 SKINNY_SPLIT_MAX_WEIGHTS = 20 << 20   # bytes; larger matrices stream faster through the tiles' LDS ring
 TILED_MIN_ROWS = 8             # head and gated projection: the skinny kernel below, tiles from here
 FUSED_QKV_MAX_WEIGHTS = 48 << 20  # bytes; with more than 16 rows of x
+FUSED_QKV_TILED_ROWS = 256
 FUSED_QKV_MIN_WORKGROUPS = 128
 
 
@@ -418,7 +419,8 @@ def _qkv_kernel(x, w, head_dim, rotary_dim, page_size):
     if m <= 16 or (m <= SKINNY_MAX_ROWS and w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS
                    and w.numel() * 2 <= FUSED_QKV_MAX_WEIGHTS):
         return "skinny"
-    if not wants_partials(x, w):
+    # many rows: partial sums would be a second pass over [rows, width] in float32
+    if m > FUSED_QKV_TILED_ROWS or not wants_partials(x, w):
         return "tiled"
     return None
 
