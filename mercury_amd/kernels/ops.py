@@ -570,8 +570,10 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     waves = max(1, num_tiles * n_kv)
     if staged:
         pass
-    elif waves < ATTENTION_TARGET_WAVES and step.max_q_len == 1:
-        # decoding: every sequence's own range in equal parts
+    elif waves < ATTENTION_TARGET_WAVES:
+        # decoding, and short prompt portions over a long prefix (16 tokens over 2,032: 47 us
+        # as one chain of key blocks per wavefront, 23 split): every tile's own range of keys
+        # in equal parts
         splits = max(1, min(blocks // ATTENTION_MIN_BLOCKS_PER_SPLIT or 1,
                             -(-ATTENTION_TARGET_WAVES // waves), 1024))
     if split_override is not None:
@@ -590,7 +592,7 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
 
 
 ATTENTION_TARGET_WAVES = 1024
-ATTENTION_STAGED_WORKGROUPS = 128
+ATTENTION_STAGED_WORKGROUPS = 64
 ATTENTION_STAGED_MAX_WAVES = 16384
 ATTENTION_WIDE_TILE_WAVES = 400
 ATTENTION_MIN_BLOCKS_PER_SPLIT = 2
