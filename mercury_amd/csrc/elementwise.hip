@@ -186,6 +186,7 @@ static int launch_rmsnorm(float* h, const float* partials, int num_partials,
   if (hidden % 4 == 0 && (num_partials == 0 || partial_stride % 4 == 0)) {
     const int chunks = hidden / 4;
     int threads = out_rows <= 256 ? (chunks + 63) / 64 * 64 : 256;
+    while (threads < 1024 && chunks > 4 * threads) threads *= 2;   // wide rows: at most 4 chunks a thread
     if (threads > 1024) threads = 1024;
     const int ch = (chunks + threads - 1) / threads;
 #define RMS_VEC(CH)                                                                            \
@@ -201,6 +202,7 @@ static int launch_rmsnorm(float* h, const float* partials, int num_partials,
     if (ch == 1) RMS_VEC(1);
     if (ch == 2) RMS_VEC(2);
     if (ch <= 4) RMS_VEC(4);
+    if (ch <= 8) RMS_VEC(8);
 #undef RMS_VEC
   }
   int threads = hidden >= 512 ? 256 : (hidden >= 256 ? 128 : 64);

@@ -54,7 +54,8 @@ def test_embed_gathers_rows_as_float32(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("rows,cols", [(1, 896), (7, 1000), (129, 168), (3, 4100)])
+@pytest.mark.parametrize("rows,cols", [(1, 896), (7, 1000), (129, 168), (3, 4100), (300, 5120),
+                                       (2, 20000), (260, 8200), (3, 40004), (2, 1003)])
 def test_rmsnorm_matches_plain(dtype, rows, cols):
     h = rnd(rows, cols, seed=1, scale=3.0)
     w_h, w_d = as_dtype(1 + rnd(cols, seed=2, scale=0.1), dtype)
@@ -80,12 +81,13 @@ def test_rmsnorm_constant_and_zero_rows():
     assert torch.allclose(got[1], torch.full((300,), 2.5 / math.sqrt(2.5**2 + eps)), atol=1e-6)
 
 
-def test_rmsnorm_adds_partial_sums_into_the_stream_first():
+@pytest.mark.parametrize("rows,cols,slices", [(9, 200, 3), (300, 5120, 3), (2, 1003, 5), (70, 8200, 2)])
+def test_rmsnorm_adds_partial_sums_into_the_stream_first(rows, cols, slices):
     """The residual sum is part of the norm: h <- h + sum(partials), then normalise
     (reference: the sum is the norm's second result, mercury/model/qwen2.py:27-31)."""
-    h = rnd(9, 200, seed=5)
-    parts = rnd(3, 9, 200, seed=6)
-    w = 1 + rnd(200, seed=7, scale=0.1)
+    h = rnd(rows, cols, seed=5)
+    parts = rnd(slices, rows, cols, seed=6)
+    w = 1 + rnd(cols, seed=7, scale=0.1)
     want, total = plain.rms_norm(parts.sum(0), w, 1e-6, residual=h)
     h_d = h.clone().to(DEV)
     got = ops().rmsnorm(h_d, w.to(DEV), 1e-6, torch.float32, partials=parts.to(DEV))
