@@ -18,11 +18,35 @@ __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ 
   for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = Elem<T>::load(row + i);
 }
 
+// bfloat16 rows of a multiple of 8 elements: 16 bytes in, 32 bytes out per thread and turn.
+__global__ void embed_bf16x8_kernel(const int* __restrict__ ids, const bf16_t* __restrict__ table,
+                                    float* __restrict__ out, int hidden, int vocab) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const uint4* row = (const uint4*)(table + (size_t)id * hidden);
+  float4* dst = (float4*)(out + (size_t)t * hidden);
+  for (int i = threadIdx.x; i < hidden / 8; i += blockDim.x) {
+    const uint4 u = row[i];
+    dst[2 * i] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
+                             __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
+    dst[2 * i + 1] = make_float4(__uint_as_float(u.z << 16), __uint_as_float(u.z & 0xffff0000u),
+                                 __uint_as_float(u.w << 16), __uint_as_float(u.w & 0xffff0000u));
+  }
+}
+
 extern "C" int mk_embed(const int* ids, const void* table, int dtype, float* out, int tokens,
                         int hidden, int vocab, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes T=%d H=%d V=%d", tokens,
              hidden, vocab);
   if (tokens == 0) return 0;
+  if (dtype == MK_BF16 && hidden % 8 == 0) {
+    const int chunks = hidden / 8;
+    embed_bf16x8_kernel<<<tokens, chunks >= 256 ? 256 : (chunks + 63) / 64 * 64, 0, stream>>>(
+        ids, (const bf16_t*)table, out, hidden, vocab);
+    MK_LAUNCH_CHECK("embed");
+    return 0;
+  }
   const int threads = hidden >= 256 ? 256 : 64;
   if (dtype == MK_F32)
     embed_kernel<float><<<tokens, threads, 0, stream>>>(ids, (const float*)table, out, hidden,

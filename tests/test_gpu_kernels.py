@@ -42,8 +42,9 @@ def as_dtype(x, dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-def test_embed_gathers_rows_as_float32(dtype):
-    table_h, table_d = as_dtype(rnd(1003, 168), dtype)
+@pytest.mark.parametrize("hidden", [168, 165, 3584, 8])
+def test_embed_gathers_rows_as_float32(dtype, hidden):
+    table_h, table_d = as_dtype(rnd(1003, hidden), dtype)
     ids = torch.tensor([0, 1002, 5, 5, 77], dtype=torch.int32)
     out = ops().embed(ids.to(DEV), table_d)
     assert out.dtype == torch.float32
