@@ -873,12 +873,23 @@ static double tiled_time(const TiledConfig& t, int M, int cols, int K, int halve
   const double per_unit = few ? (double)((tiles + 255) / 256) : tiles / 256.0 + 0.5;
   const double products = 2.0 * t.bm * t.bn * K * 1e-6 / slices;        // MFLOP
   const double edges = 1.5 + (double)t.bm * width * out_bytes / 35e3;  // microseconds
-  if (t.resident == 1) return per_unit * (products / t.rate + edges);
-  if (few) {
+  // With few rows of x the weights are the work: a compute unit's tiles stream their rows of
+  // W at the unit's share of HBM bandwidth (about 23.5 GB/s; tiles of 64 rows a little less,
+  // x being read again for each).  18944 x 3584 gated at 32 rows: 57.6 us in 64 x 64 tiles
+  // (3 a unit), 66.8 in 64 x 128 (2 a unit); 27648 x 5120: 117.5 (4) against 108.4 (2).
+  // (With several tile rows the rows of W are shared through the L2 and this is no bound.)
+  const double streaming =
+      M > t.bm ? 0.0 : per_unit * ((double)t.bn * K * 2.0 / slices) / (t.bn >= 128 ? 23.5e3 : 22.5e3);
+  double time;
+  if (t.resident == 1) {
+    time = per_unit * (products / t.rate + edges);
+  } else if (few) {
     const long n = (long)per_unit;
-    return (n / 2) * (products / t.rate + edges / 2) + (n % 2) * (products / t.alone + edges);
+    time = (n / 2) * (products / t.rate + edges / 2) + (n % 2) * (products / t.alone + edges);
+  } else {
+    time = per_unit / 2 * (products / t.rate + edges / 2);
   }
-  return per_unit / 2 * (products / t.rate + edges / 2);
+  return time > streaming ? time : streaming;
 }
 
 // The configuration with the least estimated time, K whole.
