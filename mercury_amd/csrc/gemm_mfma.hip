@@ -874,20 +874,25 @@ static double tiled_time(const TiledConfig& t, int M, int cols, int K, int halve
   const double products = 2.0 * t.bm * t.bn * K * 1e-6 / slices;        // MFLOP
   const double edges = 1.5 + (double)t.bm * width * out_bytes / 35e3;  // microseconds
   // With few rows of x the weights are the work: a compute unit's tiles stream their rows of
-  // W at the unit's share of HBM bandwidth (about 23.5 GB/s; tiles of 64 rows a little less,
+  // W at the unit's share of HBM bandwidth (about 26 GB/s; tiles of 64 rows a little less,
   // x being read again for each).  18944 x 3584 gated at 32 rows: 57.6 us in 64 x 64 tiles
   // (3 a unit), 66.8 in 64 x 128 (2 a unit); 27648 x 5120: 117.5 (4) against 108.4 (2).
   // (With several tile rows the rows of W are shared through the L2 and this is no bound.)
   const double streaming =
-      M > t.bm ? 0.0 : per_unit * ((double)t.bn * K * 2.0 / slices) / (t.bn >= 128 ? 23.5e3 : 22.5e3);
+      M > t.bm ? 0.0 : per_unit * ((double)t.bn * K * 2.0 / slices) / (t.bn >= 128 ? 26e3 : 22.5e3);
+  // Paired rows (gate and up) halve the columns a tile covers, so x is read twice as often:
+  // the small tiles, two to a unit, lose about a fifth of their rate to that
+  // (512 x 18944 x 3584 gated: 194 us in 128 x 128 tiles, 167 in 128 x 256).
+  const double slower = halves == 2 && t.resident == 2 ? 0.8 : 1.0;
+  const double rate = t.rate * slower, alone = t.alone * slower;
   double time;
   if (t.resident == 1) {
-    time = per_unit * (products / t.rate + edges);
+    time = per_unit * (products / rate + edges);
   } else if (few) {
     const long n = (long)per_unit;
-    time = (n / 2) * (products / t.rate + edges / 2) + (n % 2) * (products / t.alone + edges);
+    time = (n / 2) * (products / rate + edges / 2) + (n % 2) * (products / alone + edges);
   } else {
-    time = per_unit / 2 * (products / t.rate + edges / 2);
+    time = per_unit / 2 * (products / rate + edges / 2);
   }
   return time > streaming ? time : streaming;
 }
@@ -927,6 +932,10 @@ static void tiled_plan_sliced(int M, int N, int K, int* config, int* slices) {
 }
 
 extern "C" int mk_linear_tiled_configs(void) { return TILED_CONFIGS; }
+
+extern "C" int mk_gated_tiled_config(int M, int inter, int K) {
+  return tiled_config_for(M, inter, K, 2, 2);
+}
 
 extern "C" int mk_linear_tiled_config(int M, int N, int K, int out_bytes) {
   return tiled_config_for(M, N, K, 1, out_bytes);

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 7
+#define MK_ABI_VERSION 8
 
 #ifdef __cplusplus
 extern "C" {
@@ -100,6 +100,7 @@ int mk_qkv_tiled(const void* x, const void* w, const void* bias, int bias_dtype,
 
 // The gated projection for any M, tiled through LDS; config: a tile configuration, -1 for the
 // one estimated fastest.
+int mk_gated_tiled_config(int M, int inter, int K);
 int mk_gated_tiled(const void* x, const void* w, void* act, int M, int inter, int K, int config,
                    hipStream_t stream);
 

@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
 
 from . import build
 
-ABI_VERSION = 7
+ABI_VERSION = 8
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -37,6 +37,7 @@ _SIGNATURES = {
         "mk_gated_skinny": [P, P, P, I, I, I, P],
         "mk_qkv_skinny": [P, P, P, I, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_qkv_tiled": [P, P, P, I, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, P],
+        "mk_gated_tiled_config": [I, I, I],
         "mk_gated_tiled": [P, P, P, I, I, I, I, P],
         "mk_linear_tiled_slices": [I, I, I],
         "mk_linear_tiled_partials": [P, P, P, I, I, I, I, P],

@@ -254,6 +254,11 @@ def test_the_tile_configuration_follows_the_problem():
     assert lib.mk_linear_tiled_config(2048, 896, 4864, 8) == 4         # 64 x 64: 448 tiles
     assert lib.mk_linear_tiled_config(2048, 3584, 18944, 8) == 1       # 128 x 256: 224 tiles
     assert lib.mk_linear_tiled_config(40, 151936, 896, 4) in (4, 5)
+    # gate and up rows in one tile: few rows stream the weights (tiles that spread evenly over
+    # the compute units), some hundred want 128 x 256, thousands 256 x 256
+    assert lib.mk_gated_tiled_config(32, 18944, 3584) == 4 and lib.mk_gated_tiled_config(32, 27648, 5120) == 5
+    assert lib.mk_gated_tiled_config(512, 18944, 3584) == 1
+    assert lib.mk_gated_tiled_config(2048, 18944, 3584) == 0
 
 
 def test_which_skinny_projections_are_split():
