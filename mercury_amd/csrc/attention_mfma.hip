@@ -81,9 +81,12 @@ struct TableWindow {
   const int* table;
   int width, base, mine;
   __device__ __forceinline__ int page(int index, int lane) {
-    if (index < base || index >= base + 64) {  // uniform: every lane asks for the same index
+    if (index >= base + 64) {  // uniform: every lane asks for the same index, never a lower one
       base = index;
       mine = index + lane < width ? table[index + lane] : 0;
+      // Waited for here, once in 64 pages, so that no wait stands before the readlane below:
+      // that one would also wait, every time, for the keys and values asked for ahead.
+      __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0)
     }
     return __builtin_amdgcn_readlane(mine, index - base);
   }
@@ -138,7 +141,13 @@ struct TileState {
 // are kept in the base-2 domain (`c` = scale * log2 e), so every exponential is one
 // instruction.  MASKED is for blocks that some row of the tiles cannot see in full (the
 // causal edge, the window's edge, the end of the sequence); inside, nothing is tested.
-template <int D, int RT, bool MASKED>
+//
+// PERM tells which keys of the block a lane's eight scores belong to.  Without it the two
+// products of 16 keys take keys h * 16 + 0..15, and a lane holds keys h * 16 + g4 * 4 + i.
+// With it product h takes keys q * 8 + h * 4 + m (q, m = 0..3), and a lane holds the eight
+// consecutive keys g4 * 8 + 0..7: its operand of the second product is then one 16-byte
+// piece of a row of values.
+template <int D, int RT, bool MASKED, bool PERM>
 __device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBlock<D>& blk,
                                              int key0, float c, int g4) {
 #pragma unroll
@@ -152,17 +161,19 @@ __device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBloc
         sc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(blk.kf[h][k].v, st.qf[t][k].v, sc, 0, 0, 0);
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        float v = sc[i] * c;
+        float v = sc[i];
         if (MASKED) {
-          const int key = key0 + h * 16 + g4 * 4 + i;
+          const int key = key0 + (PERM ? g4 * 8 + h * 4 + i : h * 16 + g4 * 4 + i);
           const bool ok = blk.live[h] && st.row_ok[t] && key <= st.pos[t] && key >= st.lo[t];
           v = ok ? v : -INFINITY;
         }
         s[h * 4 + i] = v;
       }
     }
-    float bm = fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
-                     fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
+    // The largest raw score is also the largest scaled one (c > 0); the scale itself is
+    // applied in the fused multiply-add that subtracts the running maximum.
+    float bm = c * fmaxf(fmaxf(fmaxf(s[0], s[1]), fmaxf(s[2], s[3])),
+                         fmaxf(fmaxf(s[4], s[5]), fmaxf(s[6], s[7])));
     // The four lanes of a row exchange their maxima, and what is accumulated is rescaled,
     // only when some lane saw a score above its row's running maximum: rare once a row has
     // seen a few blocks.
@@ -179,7 +190,7 @@ __device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBloc
     const float m_use = (MASKED && st.m[t] == -INFINITY) ? 0.f : st.m[t];
     float e[8];
 #pragma unroll
-    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(s[j] - m_use);
+    for (int j = 0; j < 8; ++j) e[j] = __builtin_amdgcn_exp2f(__builtin_fmaf(s[j], c, -m_use));
     st.lsum[t] += ((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]));
     Frag pf;
     pf.u = make_uint4(pack_bf16x2(e[0], e[1]), pack_bf16x2(e[2], e[3]), pack_bf16x2(e[4], e[5]),
@@ -192,13 +203,13 @@ __device__ __forceinline__ void attend_block(TileState<D, RT>& st, const KeyBloc
 }
 
 // Blocks wholly inside what every row of the tiles sees take the unmasked path.
-template <int D, int RT>
+template <int D, int RT, bool PERM = false>
 __device__ __forceinline__ void attend(TileState<D, RT>& st, const KeyBlock<D>& blk, int key0,
                                        float c, int g4, int all_see_upto, int all_see_from) {
   if (key0 + 31 <= all_see_upto && key0 >= all_see_from)
-    attend_block<D, RT, false>(st, blk, key0, c, g4);
+    attend_block<D, RT, false, PERM>(st, blk, key0, c, g4);
   else
-    attend_block<D, RT, true>(st, blk, key0, c, g4);
+    attend_block<D, RT, true, PERM>(st, blk, key0, c, g4);
 }
 
 // RT: 16-row tiles per wavefront.  A decoded token's heads fill one tile (RT = 1, and the
@@ -340,20 +351,25 @@ __global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p
 //
 // LDS layout of a block (32 keys): keys [32][D] and values [D][32], the 16-byte chunks of
 // each row permuted so that the rows one operand read touches fall on different banks:
-//   keys    D = 64: rows of 128 bytes, chunk c of key k at c ^ ((k >> 1) & 7)
-//           D a multiple of 128: chunk c of key k at (c & ~15) | ((c ^ k) & 15)
-//           else: at (c & ~7) | ((c ^ k) & 7)
-//   values  rows of 64 bytes (32 keys), 16-byte slot s of dim j at s ^ ((j >> 2) & 3)
+//   keys    with r the operand row that key k is (staged_key_row):
+//           D = 64: rows of 128 bytes, chunk c of key k at c ^ ((r >> 1) & 7)
+//           D a multiple of 128: chunk c of key k at (c & ~15) | ((c ^ r) & 15)
+//           else: at (c & ~7) | ((c ^ r) & 7)
+//   values  rows of 64 bytes (32 keys), 16-byte slot s of dim j at s ^ ((j >> 1) & 3)
+
+// The row of a product's operand that key `key` of the block is (see PERM above).
+__device__ __forceinline__ int staged_key_row(int key) { return ((key >> 3) << 2) | (key & 3); }
 
 template <int D>
 __device__ __forceinline__ int staged_key_offset(int key, int chunk) {  // in 16-byte units
-  if (D == 64) return key * 8 + ((chunk ^ (key >> 1)) & 7);
-  if (D % 128 == 0) return key * (D / 8) + ((chunk & ~15) | ((chunk ^ key) & 15));
-  return key * (D / 8) + ((chunk & ~7) | ((chunk ^ key) & 7));
+  const int row = staged_key_row(key);
+  if (D == 64) return key * 8 + ((chunk ^ (row >> 1)) & 7);
+  if (D % 128 == 0) return key * (D / 8) + ((chunk & ~15) | ((chunk ^ row) & 15));
+  return key * (D / 8) + ((chunk & ~7) | ((chunk ^ row) & 7));
 }
 
 __device__ __forceinline__ int staged_value_offset(int dim, int slot) {  // in 16-byte units
-  return dim * 4 + ((slot ^ (dim >> 2)) & 3);
+  return dim * 4 + ((slot ^ (dim >> 1)) & 3);
 }
 
 // What one thread carries of a block between its global loads and its LDS stores.
@@ -362,6 +378,11 @@ struct StagedRegs {
   uint4 k[D / 64], v[D / 64];
 };
 
+// Thread-slot u = tid + 256 i of a block's 4 D slots: half u / (2 D) of the block (16 keys,
+// one page or a part of one), and 16 bytes t = u % (2 D) of that half's keys (a run of
+// 32 D bytes in the cache) and of its values (dim t / 2, keys (t & 1) * 8 .. + 8).  All of a
+// wavefront's slots of one i lie in one half, so a half's page is looked up once for the
+// wavefront and each load is that page's address plus what the thread adds to it.
 template <int D>
 __device__ __forceinline__ StagedRegs<D> staged_fetch(const AttnParams& p, TableWindow& tw, int b,
                                                       int b_end, int kmin, int kmax, int kvh,
@@ -369,29 +390,24 @@ __device__ __forceinline__ StagedRegs<D> staged_fetch(const AttnParams& p, Table
   StagedRegs<D> regs;
   const int ps = 1 << p.page_shift;
   const int tid = threadIdx.x & 255;   // within the four wavefronts that share the block
-  int page[2], off[2];
-#pragma unroll
-  for (int h = 0; h < 2; ++h) {
-    const int kh = (b << 5) + h * 16;
-    const bool live = b < b_end && kh <= kmax && kh + 15 >= kmin;  // uniform
-    page[h] = live ? tw.page(kh >> p.page_shift, lane) : 0;
-    off[h] = kh & (ps - 1);
-  }
-  const size_t head_elems = (size_t)ps * D;
+  // A page's address is one 64-bit product added to the cache's (a cache may hold more than
+  // 4 GB); everything within the page, the head's and the thread's share, fits 32 bits.
+  const uint32_t head_bytes = (uint32_t)ps * D * 2;
+  const uint32_t page_bytes = head_bytes * (uint32_t)p.n_kv;
+  const uint32_t head_at = (uint32_t)kvh * head_bytes;
 #pragma unroll
   for (int i = 0; i < D / 64; ++i) {
-    // keys: 16-byte chunk `chunk` of key `key` of the block
-    const int idx = tid + i * 256, key = idx / (D / 8), chunk = idx % (D / 8);
-    const bool h = key >= 16;      // per lane: selected, not indexed
-    const bf16_t* kp = p.k_cache + ((size_t)(h ? page[1] : page[0]) * p.n_kv + kvh) * head_elems +
-                       (size_t)((h ? off[1] : off[0]) + (key & 15)) * D + chunk * 8;
-    regs.k[i] = *(const uint4*)kp;
-    // values: 8 keys (slot `slot` of 4) of dim `dim`
-    const int dim = idx >> 2, slot = idx & 3;
-    const bool hv = slot >= 2;
-    const bf16_t* vp = p.v_cache + ((size_t)(hv ? page[1] : page[0]) * p.n_kv + kvh) * head_elems +
-                       (size_t)dim * ps + (hv ? off[1] : off[0]) + (slot & 1) * 8;
-    regs.v[i] = *(const uint4*)vp;
+    const int u = tid + i * 256, t = u % (2 * D);
+    const int h = __builtin_amdgcn_readfirstlane(u / (2 * D));
+    const int kh = (b << 5) + h * 16;
+    const bool live = b < b_end && kh <= kmax && kh + 15 >= kmin;   // uniform
+    const int page = live ? tw.page(kh >> p.page_shift, lane) : 0;
+    const uint32_t off = kh & (ps - 1);
+    const uint64_t page_at = (uint64_t)(uint32_t)page * page_bytes;
+    const uint32_t k_at = head_at + off * (uint32_t)(D * 2) + (uint32_t)t * 16u;
+    const uint32_t v_at = head_at + off * 2u + (uint32_t)((t >> 1) * ps * 2 + (t & 1) * 16);
+    regs.k[i] = *(const uint4*)((const char*)p.k_cache + page_at + k_at);
+    regs.v[i] = *(const uint4*)((const char*)p.v_cache + page_at + v_at);
   }
   return regs;
 }
@@ -401,35 +417,28 @@ __device__ __forceinline__ void staged_store(const StagedRegs<D>& regs, uint4* l
   const int tid = threadIdx.x & 255;
 #pragma unroll
   for (int i = 0; i < D / 64; ++i) {
-    const int idx = tid + i * 256;
-    lds_k[staged_key_offset<D>(idx / (D / 8), idx % (D / 8))] = regs.k[i];
-    lds_v[staged_value_offset(idx >> 2, idx & 3)] = regs.v[i];
+    const int u = tid + i * 256, t = u % (2 * D), h = u / (2 * D);
+    lds_k[staged_key_offset<D>(h * 16 + t / (D / 8), t % (D / 8))] = regs.k[i];
+    lds_v[staged_value_offset(t >> 1, h * 2 + (t & 1))] = regs.v[i];
   }
 }
 
-// The block's operands of this lane, out of LDS (as load_key_block takes them from the cache).
+// The block's operands of this lane, out of LDS, in the order PERM describes.
 template <int D>
 __device__ __forceinline__ void staged_operands(KeyBlock<D>& blk, const uint4* lds_k,
-                                                const uint4* lds_v, int b, int kmin, int kmax,
-                                                int lane) {
+                                                const uint4* lds_v, int lane) {
   const int r = lane & 15, g4 = lane >> 4;
 #pragma unroll
   for (int h = 0; h < 2; ++h) {
-    const int kh = (b << 5) + h * 16;
-    blk.live[h] = kh <= kmax && kh + 15 >= kmin;
+    blk.live[h] = true;   // keys outside what a row sees are masked one by one
+    const int key = ((r >> 2) << 3) + h * 4 + (r & 3);
 #pragma unroll
     for (int c = 0; c < D / 32; ++c)
-      blk.kf[h][c].u = lds_k[staged_key_offset<D>(h * 16 + r, c * 4 + g4)];
+      blk.kf[h][c].u = lds_k[staged_key_offset<D>(key, c * 4 + g4)];
   }
 #pragma unroll
   for (int dt = 0; dt < D / 16; ++dt)
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      // keys h*16 + g4*4 .. + 4 of dim dt*16 + r: half of the 16-byte slot h*2 + g4/2
-      const int dim = dt * 16 + r;
-      const uint2* slot = (const uint2*)(lds_v + staged_value_offset(dim, h * 2 + (g4 >> 1)));
-      blk.vf[dt].u2[h] = slot[g4 & 1];
-    }
+    blk.vf[dt].u = lds_v[staged_value_offset(dt * 16 + r, g4)];
 }
 
 // KG groups of four wavefronts share a workgroup's 64 * RT rows: group g takes the key blocks
@@ -438,7 +447,7 @@ __device__ __forceinline__ void staged_operands(KeyBlock<D>& blk, const uint4* l
 // last rows see thousands of keys; the groups cut that chain of dependent blocks into KG
 // shorter ones that run side by side on the same compute unit.
 template <int D, int RT, int KG>
-__global__ __launch_bounds__(64 * ATTN_WAVES * KG) void attn_staged_kernel(AttnParams p) {
+__global__ __launch_bounds__(64 * ATTN_WAVES * KG, (RT == 1 ? (KG > 2 ? KG : 2) : 1)) void attn_staged_kernel(AttnParams p) {
   static_assert(D % 64 == 0, "256 threads bring whole 16-byte chunks of 32 keys");
   constexpr int BLOCK = 32 * D / 8;                       // 16-byte units of a block's keys (or values)
   constexpr int MERGE = RT * (D / 4 + 2);                 // floats a thread hands over
@@ -487,14 +496,19 @@ __global__ __launch_bounds__(64 * ATTN_WAVES * KG) void attn_staged_kernel(AttnP
   const int wg_kmin = p.window > 0 ? max(0, pos0 + wg_row0 / G - p.window + 1) : 0;
   const int b0 = wg_kmin >> 5, b1 = (wg_kmax >> 5) + 1;
   const int last_flat = min(row0 + WAVE_ROWS - 1, rows_total - 1);
-  const int kmax = wave_has_rows ? pos0 + last_flat / G : -1;
-  const int kmin = p.window > 0 ? max(0, pos0 + row0 / G - p.window + 1) : 0;
-  const int see_upto = pos0 + row0 / G;
+  // What steers the loop is the same in every lane of a wavefront, and is said to be so (a
+  // wavefront's index comes out of threadIdx and counts as different from lane to lane):
+  // the tests on it are then scalar compares and branches, and a block's pages and addresses
+  // are worked out once for the wavefront, not in every lane.
+  auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  const int kmax = uniform(wave_has_rows ? pos0 + last_flat / G : -1);
+  const int kmin = uniform(p.window > 0 ? max(0, pos0 + row0 / G - p.window + 1) : 0);
+  const int see_upto = uniform(pos0 + row0 / G);
   const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
   const float c = p.scale * 1.44269504088896340736f;
 
   TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
-  const int first = b0 + kgroup;                        // this group's blocks: first, first + KG, ...
+  const int first = b0 + uniform(kgroup);                        // this group's blocks: first, first + KG, ...
   StagedRegs<D> ra = staged_fetch<D>(p, tw, first, b1, wg_kmin, wg_kmax, kvh, lane);
   StagedRegs<D> rb = staged_fetch<D>(p, tw, first + KG, b1, wg_kmin, wg_kmax, kvh, lane);
   KeyBlock<D> blk;
@@ -509,9 +523,8 @@ __global__ __launch_bounds__(64 * ATTN_WAVES * KG) void attn_staged_kernel(AttnP
     regs = staged_fetch<D>(p, tw, (b) + 2 * KG, b1, wg_kmin, wg_kmax, kvh, lane);       \
     __syncthreads();                                                                    \
     if (((b) << 5) <= kmax && ((b) << 5) + 31 >= kmin) {                                \
-      staged_operands<D>(blk, lds_k + (buf) * BLOCK, lds_v + (buf) * BLOCK, (b), kmin,  \
-                         kmax, lane);                                                   \
-      attend<D, RT>(st, blk, (b) << 5, c, g4, see_upto, see_from);                      \
+      staged_operands<D>(blk, lds_k + (buf) * BLOCK, lds_v + (buf) * BLOCK, lane);      \
+      attend<D, RT, true>(st, blk, (b) << 5, c, g4, see_upto, see_from);                \
     }                                                                                   \
   } while (0)
   const int iterations = (b1 - b0 + KG - 1) / KG;       // the same for every group
@@ -705,6 +718,7 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   MK_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0,
              "attention: row strides %d/%d break 16-byte alignment", q_stride, out_stride);
   MK_REQUIRE(window >= 0, "attention: negative window");
+  MK_REQUIRE(scale > 0.f, "attention: the score scale %g is not positive", (double)scale);
   MK_REQUIRE(rows_per_tile == 16 || rows_per_tile == 32 || rows_per_tile == 64,
              "attention: %d rows per tile", rows_per_tile);
   MK_REQUIRE(rows_per_tile <= mk_attention_mfma_max_rows(d),

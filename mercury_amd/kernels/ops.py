@@ -561,7 +561,8 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     if staged == -1:
         # A workgroup's chain of key blocks is cut into 2 or 4 chains side by side while that
         # leaves the chip short of wavefronts and every chain a few blocks (measured at 2,048
-        # tokens, 14 heads of 64: 62, 50, 36 us with 1, 2, 4 groups; at 8,192: 372, 323, 385).
+        # tokens, 14 heads of 64: 45, 35, 32 us with 1, 2, 4 groups; at 8,192: 264, 349, 284;
+        # 28 heads of 128 at 2,048: 100, 91 with 1, 2; at 8,192: 878, 1055).
         staged = lib.mk_attention_mfma_staged(head_dim, 16)
         while staged > 1 and (num_tiles * n_kv * 4 * staged > ATTENTION_STAGED_MAX_WAVES
                               or blocks < 4 * staged):
@@ -593,7 +594,7 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
 
 ATTENTION_TARGET_WAVES = 1024
 ATTENTION_STAGED_WORKGROUPS = 64
-ATTENTION_STAGED_MAX_WAVES = 16384
+ATTENTION_STAGED_MAX_WAVES = 8192
 ATTENTION_WIDE_TILE_WAVES = 400
 ATTENTION_MIN_BLOCKS_PER_SPLIT = 2
 
