@@ -217,7 +217,7 @@ __device__ __forceinline__ void attend(TileState<D, RT>& st, const KeyBlock<D>& 
 // share every key and value fragment the wavefront loads.  AHEAD: how many blocks of keys
 // are in flight beyond the one in the matrix cores (0, 1 or 2).
 template <int D, int RT, int AHEAD>
-__global__ __launch_bounds__(64 * ATTN_WAVES) void attn_mfma_kernel(AttnParams p) {
+__global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) void attn_mfma_kernel(AttnParams p) {
   const int lane = threadIdx.x & 63;
   // Tiles are taken from the last: under a causal mask the later tiles of a prompt read the
   // most keys, and the longest work should start first.
