@@ -878,8 +878,14 @@ static double tiled_time(const TiledConfig& t, int M, int cols, int K, int halve
   // x being read again for each).  18944 x 3584 gated at 32 rows: 57.6 us in 64 x 64 tiles
   // (3 a unit), 66.8 in 64 x 128 (2 a unit); 27648 x 5120: 117.5 (4) against 108.4 (2).
   // (With several tile rows the rows of W are shared through the L2 and this is no bound.)
+  // The largest tiles (8 wavefronts, three stages of 48 KB in flight) draw about 33 GB/s, and
+  // the chip as a whole gives these kernels about 5.9 TB/s: 27648 x 5120 gated at 64 rows runs
+  // 106 us in 128 x 256 tiles (216 units busy), 118 in 64 x 128, 135 in 64 x 64; 18944 x 3584:
+  // 60, 70, 64.
+  const double unit_rate = t.bm * t.bn >= 128 * 256 ? 33e3 : (t.bn >= 128 ? 26e3 : 22.5e3);
+  const double tile_bytes = (double)t.bn * K * 2.0 / slices;
   const double streaming =
-      M > t.bm ? 0.0 : per_unit * ((double)t.bn * K * 2.0 / slices) / (t.bn >= 128 ? 26e3 : 22.5e3);
+      M > t.bm ? 0.0 : fmax(per_unit * tile_bytes / unit_rate, tiles * tile_bytes / 5.9e6);
   // Paired rows (gate and up) halve the columns a tile covers, so x is read twice as often:
   // the small tiles, two to a unit, lose about a fifth of their rate to that
   // (512 x 18944 x 3584 gated: 194 us in 128 x 128 tiles, 167 in 128 x 256).
@@ -902,7 +908,10 @@ static int tiled_config_for(int M, int cols, int K, int halves, int out_bytes) {
   int best = -1;
   double best_time = 0.0;
   for (int c = 0; c < TILED_CONFIGS; ++c) {
-    if (M <= 64 && tiled_configs[c].bm > 64) continue;
+    // Few rows of x: tiles of 128 rows multiply padding, which costs nothing while the weights
+    // are the work, but only the paired 128 x 256 tile streams them faster than the 64-row
+    // tiles do (the head, 152064 x 5120 at 64 rows: 319 us against 306 in 64 x 128).
+    if (M <= 64 && tiled_configs[c].bm > 64 && !(halves == 2 && c == 1)) continue;
     const double time = tiled_time(tiled_configs[c], M, cols, K, halves, out_bytes, 1);
     if (best < 0 || time < best_time) best = c, best_time = time;
   }

@@ -219,7 +219,8 @@ def test_gated_projection(m, inter, k):
     torch.testing.assert_close(got.float().cpu(), plain_want, **tol(torch.bfloat16))
 
 
-@pytest.mark.parametrize("m,n,k", [(300, 520, 200), (257, 130, 64), (70, 1004, 1096), (513, 264, 8)])
+@pytest.mark.parametrize("m,n,k", [(300, 520, 200), (257, 130, 64), (70, 1004, 1096), (513, 264, 8),
+                                   (40, 776, 136)])
 def test_every_tile_configuration(m, n, k):
     """Each tile shape of the tiled projection, forced, at sizes that leave partial tiles in
     both directions and a partial last stage of K: every epilogue, and the gated form with
@@ -254,9 +255,11 @@ def test_the_tile_configuration_follows_the_problem():
     assert lib.mk_linear_tiled_config(2048, 896, 4864, 8) == 4         # 64 x 64: 448 tiles
     assert lib.mk_linear_tiled_config(2048, 3584, 18944, 8) == 1       # 128 x 256: 224 tiles
     assert lib.mk_linear_tiled_config(40, 151936, 896, 4) in (4, 5)
-    # gate and up rows in one tile: few rows stream the weights (tiles that spread evenly over
-    # the compute units), some hundred want 128 x 256, thousands 256 x 256
-    assert lib.mk_gated_tiled_config(32, 18944, 3584) == 4 and lib.mk_gated_tiled_config(32, 27648, 5120) == 5
+    # gate and up rows in one tile: few rows stream the weights, a large matrix fastest
+    # through the 128 x 256 tile's three stages (a small one in tiles that spread over the
+    # compute units); some hundred rows want 128 x 256 too, thousands 256 x 256
+    assert lib.mk_gated_tiled_config(32, 18944, 3584) == 1 and lib.mk_gated_tiled_config(32, 27648, 5120) == 1
+    assert lib.mk_gated_tiled_config(32, 4864, 896) == 4
     assert lib.mk_gated_tiled_config(512, 18944, 3584) == 1
     assert lib.mk_gated_tiled_config(2048, 18944, 3584) == 0
 
