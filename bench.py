@@ -113,10 +113,11 @@ class Bench:
         pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + PREFILL_TOKENS // BLOCK_SIZE + 8
         self.engine_cfg = EngineConfig(
             model="random", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
-            max_running=max_batch + 1, prefill_budget=prefill_budget, max_model_len=context + 128, seed=seed,
+            max_running=max_batch + 1, prefill_budget=prefill_budget,
+            max_model_len=max(context, PREFILL_TOKENS) + 128, seed=seed,
             lookahead=lookahead)
         manager = CacheManager(model.cache_slots, pages, BLOCK_SIZE, max_batch + 1, False)
-        runner = ModelRunner(model, manager, torch_dtype, device, context + 128)
+        runner = ModelRunner(model, manager, torch_dtype, device, max(context, PREFILL_TOKENS) + 128)
         self.engine = Engine(self.engine_cfg, executor=GpuExecutor(runner, Sampler(seed), lookahead=self.engine_cfg.lookahead),
                              manager=manager, eos_token_ids=())
         self.model, self.runner, self.manager = model, runner, manager
