@@ -1,0 +1,50 @@
+"""bench.py's contract: one JSON line at one GPU, a refusal with exit code 2 at more."""
+import json
+import subprocess
+import sys
+from pathlib import Path
+
+import pytest
+
+ROOT = Path(__file__).resolve().parent.parent
+
+
+def run_bench(*args):
+    return subprocess.run([sys.executable, str(ROOT / "bench.py"), *args], capture_output=True,
+                          text=True, timeout=600)
+
+
+def test_more_than_one_gpu_is_refused_in_one_line():
+    done = run_bench("--gpus", "2", "--steps", "2", "--warmup", "1")
+    assert done.returncode == 2
+    lines = [l for l in done.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1 and "--gpus 2" in lines[0]
+
+
+@pytest.mark.gpu
+def test_the_line_of_one_gpu_keeps_the_contract():
+    done = run_bench("--layers", "2", "--steps", "4", "--warmup", "1", "--context", "512")
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = [l for l in done.stdout.splitlines() if l.strip()]
+    assert len(lines) == 1
+    line = json.loads(lines[0])
+    for key in ("metric", "value", "unit", "n_gpus", "steps", "warmup", "ms_per_step",
+                "higher_is_better", "scaling", "vs_baseline", "dtype", "data", "config",
+                "prefill", "roofline", "points"):
+        assert key in line, key
+    assert line["n_gpus"] == 1 and line["steps"] == 4 and line["warmup"] == 1
+    assert line["unit"] == "tok/s" and line["dtype"] == "bf16" and line["higher_is_better"] is True
+    config = line["config"]
+    assert len(config) <= 20 and all(not isinstance(v, (dict, list)) for v in config.values())
+    assert config["layers"] == 2 and config["layers_full"] == 24 and config["global_batch"] == 8
+    assert config["hidden"] == 896 and config["vocab"] == 151936 and config["seq_len"] == 512
+    # decoded tokens a second are the batch over the step's time
+    assert line["value"] == pytest.approx(8 / (line["ms_per_step"] * 1e-3), rel=1e-3)
+    assert set(line["prefill"]) == {"value", "tokens", "ms", "frac"} and line["prefill"]["tokens"] == 2048
+    assert line["prefill"]["value"] == pytest.approx(2048 / (line["prefill"]["ms"] * 1e-3), rel=1e-3)
+    roof = line["roofline"]
+    assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
+    assert roof["frac"] == pytest.approx(roof["achieved"] / roof["peak"], rel=1e-3) and 0 < roof["frac"] < 1
+    assert 0 < line["prefill"]["frac"] < 1
+    assert set(line["points"]) == {"decode_b1", "decode_b64"}
+    assert line["points"]["decode_b64"] > line["points"]["decode_b1"] > 0
