@@ -100,12 +100,6 @@ class CacheManager:
 
     # ---- admission, growth, trimming, release
 
-    def planned_hit_tokens(self, hashes, num_tokens: int) -> int:
-        if not self.prefix_sharing or not self.groups:
-            return 0
-        return min(len(g.pool.plan_prompt(hashes, num_tokens)[0]) for g in self.groups) \
-            * self.page_size
-
     def admit(self, key, hashes, num_tokens: int):
         """Take a state slot and, in every all-keys group, the pages of a prompt of
         `num_tokens`.  Returns the number of leading tokens whose keys are already cached, or

@@ -180,10 +180,6 @@ def _mfma_eligible(x, w: torch.Tensor) -> bool:
             and x.shape[0] > 0 and x.shape[1] % 8 == 0)
 
 
-def _skinny_eligible(x, w: torch.Tensor) -> bool:
-    return _mfma_eligible(x, w) and x.shape[0] <= SKINNY_MAX_ROWS
-
-
 def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     """Float32 partial sums [P, M, N] of x W^T over P slices of K; the consumer (rmsnorm,
     rope_kv_write: their `partials` forms) adds them up in slice order.  At most 16 rows of
