@@ -260,7 +260,11 @@ def test_the_tile_configuration_follows_the_problem():
     # compute units); some hundred rows want 128 x 256 too, thousands 256 x 256
     assert lib.mk_gated_tiled_config(32, 18944, 3584) == 1 and lib.mk_gated_tiled_config(32, 27648, 5120) == 1
     assert lib.mk_gated_tiled_config(32, 4864, 896) == 4
-    assert lib.mk_gated_tiled_config(512, 18944, 3584) == 1
+    assert lib.mk_gated_tiled_config(512, 27648, 5120) == 0
+    # 256 x 192 where 256 columns leave the last round of tiles half empty: 18944 pairs of
+    # rows at 512 rows of x (158 us against 167 in 128 x 256), 4608 columns at 2,048
+    assert lib.mk_gated_tiled_config(512, 18944, 3584) == 6
+    assert lib.mk_linear_tiled_config(2048, 4608, 3584, 2) == 6
     assert lib.mk_gated_tiled_config(2048, 18944, 3584) == 0
 
 
