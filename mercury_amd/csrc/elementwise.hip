@@ -401,6 +401,8 @@ extern "C" int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const floa
 // The q/k/v projection arrives as float32 slices [p, T, (n_q + 2 n_kv) d]; this adds them up,
 // adds the bias, rotates q and k, writes q [T, n_q d] and the cache.  Sums and rotation are
 // float32; q, k and v are rounded to the storage type first, as a stored projection would be.
+// Workgroup (t, y) takes heads [y * heads_per_group, ...) of token t (a rotation pairs dims
+// of one head), so that a few tokens still occupy the chip.
 template <typename T, typename TB>
 __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_partials,
                                   size_t partial_stride, const TB* __restrict__ bias,
@@ -411,19 +413,51 @@ __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_pa
                                   const int* __restrict__ block_table, int table_stride,
                                   T* __restrict__ k_cache, T* __restrict__ v_cache,
                                   int page_shift, int n_q, int n_kv, int d, int rot,
-                                  int write_kv) {
-  extern __shared__ float vals[];  // the token's summed, biased, rounded projection row
+                                  int write_kv, int heads_per_group) {
+  extern __shared__ float vals[];  // the group's heads of the token: summed, biased, rounded
   const int t = blockIdx.x;
+  const int heads = n_q + (write_kv ? 2 * n_kv : 0);
+  const int head0 = blockIdx.y * heads_per_group;
+  const int count = (min(heads, head0 + heads_per_group) - head0) * d;  // values of this group
+  if (count <= 0) return;
   const int pos = positions[t];
   const int half = rot / 2;
   const float* cs = cos_table + (size_t)pos * half;
   const float* sn = sin_table + (size_t)pos * half;
   const int width = (n_q + 2 * n_kv) * d;
-  const float* row = partials + (size_t)t * width;
-  for (int col = threadIdx.x; col < width; col += blockDim.x) {
-    float v = sum_partials(row + col, num_partials, partial_stride);
-    if (bias) v += Elem<TB>::load(bias + col);
-    vals[col] = Elem<T>::round(v);
+  const int col0 = head0 * d;
+  const float* row = partials + (size_t)t * width + col0;
+  if ((d & 3) == 0 && (partial_stride & 3) == 0) {
+    for (int i = threadIdx.x * 4; i < count; i += blockDim.x * 4) {
+      float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+      int k = 0;   // the order of sum_partials, four values at a time
+      for (; k + 4 <= num_partials; k += 4) {
+        const float4 a = *(const float4*)(row + i + (size_t)k * partial_stride);
+        const float4 b = *(const float4*)(row + i + (size_t)(k + 1) * partial_stride);
+        const float4 c = *(const float4*)(row + i + (size_t)(k + 2) * partial_stride);
+        const float4 e = *(const float4*)(row + i + (size_t)(k + 3) * partial_stride);
+        v.x += (a.x + b.x) + (c.x + e.x);
+        v.y += (a.y + b.y) + (c.y + e.y);
+        v.z += (a.z + b.z) + (c.z + e.z);
+        v.w += (a.w + b.w) + (c.w + e.w);
+      }
+      for (; k < num_partials; ++k) {
+        const float4 a = *(const float4*)(row + i + (size_t)k * partial_stride);
+        v.x += a.x, v.y += a.y, v.z += a.z, v.w += a.w;
+      }
+      float o[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+      for (int u = 0; u < 4; ++u) {
+        if (bias) o[u] += Elem<TB>::load(bias + col0 + i + u);
+        vals[i + u] = Elem<T>::round(o[u]);
+      }
+    }
+  } else {
+    for (int i = threadIdx.x; i < count; i += blockDim.x) {
+      float v = sum_partials(row + i, num_partials, partial_stride);
+      if (bias) v += Elem<TB>::load(bias + col0 + i);
+      vals[i] = Elem<T>::round(v);
+    }
   }
   __syncthreads();
 
@@ -432,23 +466,26 @@ __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_pa
     if (j < rot) return vals[base + j] * cs[j - half] + vals[base + j - half] * sn[j - half];
     return vals[base + j];
   };
-  for (int idx = threadIdx.x; idx < n_q * d; idx += blockDim.x) {
-    const int head = idx / d, j = idx - head * d;
-    Elem<T>::store(q_out + (size_t)t * n_q * d + idx, rotated(head * d, j));
-  }
-  if (!write_kv) return;
-
+  int page = -1, off = 0;
   const int page_size = 1 << page_shift;
-  const int page = block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)];
-  if (page < 0) return;
-  const int off = pos & (page_size - 1);
-  const int k0 = n_q * d, v0 = (n_q + n_kv) * d;
-  for (int idx = threadIdx.x; idx < n_kv * d; idx += blockDim.x) {
-    const int head = idx / d, j = idx - head * d;
-    Elem<T>::store(k_cache + (((size_t)page * n_kv + head) * page_size + off) * d + j,
-                   rotated(k0 + head * d, j));
-    Elem<T>::store(v_cache + (((size_t)page * n_kv + head) * d + j) * page_size + off,
-                   vals[v0 + idx]);
+  if (write_kv) {
+    page = block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)];
+    off = pos & (page_size - 1);
+  }
+  for (int i = threadIdx.x; i < count; i += blockDim.x) {
+    const int local = i / d, j = i - local * d, head = head0 + local;
+    if (head < n_q) {
+      Elem<T>::store(q_out + ((size_t)t * n_q + head) * d + j, rotated(local * d, j));
+    } else if (page >= 0) {
+      if (head < n_q + n_kv) {
+        const int kh = head - n_q;
+        Elem<T>::store(k_cache + (((size_t)page * n_kv + kh) * page_size + off) * d + j,
+                       rotated(local * d, j));
+      } else {
+        const int vh = head - n_q - n_kv;
+        Elem<T>::store(v_cache + (((size_t)page * n_kv + vh) * d + j) * page_size + off, vals[i]);
+      }
+    }
   }
 }
 
@@ -467,15 +504,22 @@ extern "C" int mk_qkv_finish(const float* partials, int num_partials, long long 
   MK_REQUIRE(dtype == MK_BF16 || dtype == MK_F32, "qkv_finish: unknown dtype %d", dtype);
   if (tokens == 0) return 0;
   const int shift = mk_log2(page_size);
-  const size_t lds_bytes = (size_t)(n_q + 2 * n_kv) * d * sizeof(float);
-  const int threads = tokens <= 64 ? 1024 : 256;
-  MK_REQUIRE(lds_bytes <= 64 * 1024, "qkv_finish: a projection row of %zu bytes exceeds LDS",
-             lds_bytes);
+  // about two workgroups of 256 threads per compute unit, whole heads each
+  const int heads = n_q + (write_kv ? 2 * n_kv : 0);
+  int groups = (512 + tokens - 1) / tokens;
+  groups = groups < 1 ? 1 : (groups > heads ? heads : groups);
+  const int heads_per_group = (heads + groups - 1) / groups;
+  groups = (heads + heads_per_group - 1) / heads_per_group;
+  const size_t lds_bytes = (size_t)heads_per_group * d * sizeof(float);
+  const int threads = 256;
+  MK_REQUIRE(lds_bytes <= 64 * 1024, "qkv_finish: %d heads of %d values exceed LDS",
+             heads_per_group, d);
+  MK_REQUIRE(groups <= 65535, "qkv_finish: %d head groups", groups);
 #define QKV_LAUNCH(T, TB)                                                                      \
-  qkv_finish_kernel<T, TB><<<tokens, threads, lds_bytes, stream>>>(                                        \
+  qkv_finish_kernel<T, TB><<<dim3(tokens, groups), threads, lds_bytes, stream>>>(              \
       partials, num_partials, (size_t)partial_stride, (const TB*)bias, (T*)q_out, cos_table,   \
       sin_table, positions, token_seq, block_table, table_stride, (T*)k_cache, (T*)v_cache,    \
-      shift, n_q, n_kv, d, rot, write_kv)
+      shift, n_q, n_kv, d, rot, write_kv, heads_per_group)
   if (dtype == MK_BF16) {
     if (bias && bias_dtype == MK_BF16) QKV_LAUNCH(bf16_t, bf16_t);
     else QKV_LAUNCH(bf16_t, float);
