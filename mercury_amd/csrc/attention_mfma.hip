@@ -647,6 +647,50 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   }
 }
 
+// The same merge for a handful of splits, where a workgroup per row would be thousands of
+// workgroups with next to nothing to do (64 decoded tokens of 8 key/value heads in 2 splits:
+// 8,192 of them, 9 us): one workgroup per (tile, kv head), 16 threads per row with D / 16 dims
+// each, the splits added in split order.
+template <int D>
+__global__ __launch_bounds__(256) void attn_merge_rows_kernel(AttnParams p) {
+  constexpr int PER = D / 16;
+  const int tile = blockIdx.x, kvh = blockIdx.y, R = p.tile_rows, S = p.num_splits;
+  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
+  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  const int G = p.group;
+  const size_t base = ((size_t)tile * p.n_kv + kvh) * S;
+  const int sub = threadIdx.x & 15;
+  for (int r = threadIdx.x >> 4; r < R; r += 16) {
+    const int flat = row0 + r;
+    if (flat >= q_len * G) continue;
+    float mx = -INFINITY;
+    for (int s2 = 0; s2 < S; ++s2) mx = fmaxf(mx, p.part_ml[((base + s2) * R + r) * 2]);
+    float total = 0.f, o[PER];
+#pragma unroll
+    for (int i = 0; i < PER; ++i) o[i] = 0.f;
+    for (int s2 = 0; s2 < S; ++s2) {
+      const size_t slot = (base + s2) * R + r;
+      const float ms = p.part_ml[slot * 2];
+      const float w = ms == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(ms - mx);  // base-2 maxima
+      total += p.part_ml[slot * 2 + 1] * w;
+      const float2* src = (const float2*)(p.part_o + slot * D + sub * PER);
+#pragma unroll
+      for (int i = 0; i < PER / 2; ++i) {
+        const float2 v = src[i];
+        o[2 * i] += v.x * w;
+        o[2 * i + 1] += v.y * w;
+      }
+    }
+    const int tok = flat / G, head = kvh * G + flat % G;
+    const float inv = 1.f / total;
+    uint32_t* dst = (uint32_t*)(p.out + (size_t)(q0 + tok) * p.out_stride + head * D + sub * PER);
+#pragma unroll
+    for (int i = 0; i < PER / 2; ++i) dst[i] = pack_bf16x2(o[2 * i] * inv, o[2 * i + 1] * inv);
+  }
+}
+
+#define ATTN_MERGE_ROWS_MAX_SPLITS 4
+
 template <int D>
 static void launch_staged(const AttnParams& p, int rows_per_tile, int key_groups, hipStream_t stream) {
   if constexpr (D == 64 || D == 128) {   // wider heads do not fit the register file
@@ -674,7 +718,9 @@ static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stre
     // 64 rows: only instantiated where the accumulators fit the register file
     if constexpr (D <= 64) attn_mfma_kernel<D, 4, ATTN_AHEAD_64><<<grid, threads, 0, stream>>>(p);
   }
-  if (p.num_splits > 1) {
+  if (p.num_splits > 1 && p.num_splits <= ATTN_MERGE_ROWS_MAX_SPLITS) {
+    attn_merge_rows_kernel<D><<<dim3(p.num_tiles, p.n_kv), 256, 0, stream>>>(p);
+  } else if (p.num_splits > 1) {
     dim3 mgrid(p.num_tiles, p.n_kv, p.tile_rows);
     attn_merge_kernel<D><<<mgrid, 256, 0, stream>>>(p);
   }
