@@ -149,7 +149,7 @@ SKINNY_MAX_ROWS = 64
 SKINNY_SPLIT_MAX_ROWS = 16     # K-split partial sums: the skinny kernel up to here, tiles beyond
 SKINNY_SPLIT_MAX_WEIGHTS = 20 << 20   # bytes; larger matrices stream faster through the tiles' LDS ring
 TILED_MIN_ROWS = 8             # head and gated projection: the skinny kernel below, tiles from here
-FUSED_QKV_MAX_WEIGHTS = 48 << 20  # bytes; with more than 16 rows of x
+FUSED_QKV_SPLIT_WEIGHTS = 24 << 20  # bytes; from here on partial sums and a finishing kernel
 FUSED_QKV_TILED_ROWS = 256
 FUSED_QKV_MIN_WORKGROUPS = 128
 
@@ -399,9 +399,9 @@ def _qkv_fusable(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: 
 def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
     """Whether `qkv_project` runs as one kernel by itself: bfloat16 rows, K a multiple of 8,
     heads a multiple of 32 wide and rotated over their whole width or not at all, pages a
-    power of two; and not 17 to a few hundred rows over a matrix so large that tiles over
-    slices of K, followed by the rotation, stream it faster (7168 x 5120 at 64 rows: 43 us in
-    one kernel, 20 + 7 in two)."""
+    power of two; and not up to a few hundred rows over a matrix so large that partial sums
+    over slices of K, followed by the rotation, stream it faster (7168 x 5120 at 64 rows: 43 us
+    in one kernel, 20 + 7 in two)."""
     return _qkv_kernel(x, w, head_dim, rotary_dim, page_size) is not None
 
 
@@ -412,8 +412,14 @@ def _qkv_kernel(x, w, head_dim, rotary_dim, page_size):
     if not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
         return None
     m = x.shape[0]
-    if m <= 16 or (m <= SKINNY_MAX_ROWS and w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS
-                   and w.numel() * 2 <= FUSED_QKV_MAX_WEIGHTS):
+    # A large matrix streams fastest as partial sums over slices of K, the rotation and the
+    # cache write in a small kernel after them (4608 x 3584 at 8, 16, 32, 64 rows: 14.0, 13.9,
+    # 15.4, 16.5 us against 15.2, 16.1, 21.1, 30.7 in the one skinny kernel; 7168 x 5120 at 8
+    # rows: 20.9 against 23.5; 1152 x 896 the other way round: 10.6 against 6.0).
+    if (m <= FUSED_QKV_TILED_ROWS and w.numel() * 2 >= FUSED_QKV_SPLIT_WEIGHTS
+            and wants_partials(x, w)):
+        return None
+    if m <= 16 or (m <= SKINNY_MAX_ROWS and w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS):
         return "skinny"
     # many rows: partial sums would be a second pass over [rows, width] in float32
     if m > FUSED_QKV_TILED_ROWS or not wants_partials(x, w):

@@ -406,6 +406,11 @@ def test_qkv_projection_falls_back_where_the_fused_kernel_does_not_apply():
     big = torch.zeros(7168, 5120, dtype=torch.bfloat16, device=DEV)
     assert not o.fuses_qkv(torch.zeros(64, 5120, dtype=torch.bfloat16, device=DEV), big, 128, 128, 16)
     assert o.fuses_qkv(many, torch.zeros(4608, 64, dtype=torch.bfloat16, device=DEV), 128, 128, 16)
+    # a large matrix goes as partial sums and a finishing kernel at any small number of rows
+    assert not o.fuses_qkv(torch.zeros(8, 5120, dtype=torch.bfloat16, device=DEV), big, 128, 128, 16)
+    mid = torch.zeros(4608, 3584, dtype=torch.bfloat16, device=DEV)
+    assert not o.fuses_qkv(torch.zeros(64, 3584, dtype=torch.bfloat16, device=DEV), mid, 128, 128, 16)
+    assert o.fuses_qkv(torch.zeros(2048, 3584, dtype=torch.bfloat16, device=DEV), mid, 128, 128, 16)
     assert not o.fuses_qkv(x, x, 48, 48, 16)          # heads not a multiple of 32 wide
     assert not o.fuses_qkv(x, x, 64, 32, 16)          # rotation over part of the head
     assert not o.fuses_qkv(x.float(), x.float(), 64, 64, 16)
