@@ -817,7 +817,7 @@ struct TiledConfig {
   int bm, bn, resident;
   float rate, alone;
 };
-#define TILED_CONFIGS 7
+#define TILED_CONFIGS 8
 static const TiledConfig tiled_configs[TILED_CONFIGS] = {
     {256, 256, 1, 5.03f, 5.03f},  // 0: 2 stages (128 KB), 16 wavefronts
     {128, 256, 1, 4.7f, 4.7f},    // 1: 3 stages (144 KB), 8 wavefronts
@@ -826,6 +826,7 @@ static const TiledConfig tiled_configs[TILED_CONFIGS] = {
     {64, 64, 2, 1.2f, 2.0f},      // 4: 4 stages (64 KB), 4 wavefronts
     {64, 128, 1, 2.14f, 2.14f},   // 5: 4 stages (96 KB), 4 wavefronts
     {256, 192, 1, 4.9f, 4.9f},    // 6: 2 stages (112 KB), 8 wavefronts: for widths that 256 divides badly
+    {128, 192, 1, 4.45f, 4.45f},  // 7: 3 stages (120 KB), 8 wavefronts
 };
 
 template <int BM, int BN, int STAGES, int WM, int WN, int SPREAD, int EPI>
@@ -856,7 +857,8 @@ static void launch_tiled(int config, const void* x, const void* w, const void* b
     case 3: launch_tiled_cfg<128, 128, 2, 2, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
     case 4: launch_tiled_cfg<64, 64, 4, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
     case 5: launch_tiled_cfg<64, 128, 4, 1, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
-    default: launch_tiled_cfg<256, 192, 2, 4, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    case 6: launch_tiled_cfg<256, 192, 2, 4, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    default: launch_tiled_cfg<128, 192, 3, 4, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
   }
 }
 
@@ -911,9 +913,11 @@ static int tiled_config_for(int M, int cols, int K, int halves, int out_bytes) {
   double best_time = 0.0;
   for (int c = 0; c < TILED_CONFIGS; ++c) {
     // Few rows of x: tiles of 128 rows multiply padding, which costs nothing while the weights
-    // are the work, but only the paired 128 x 256 tile streams them faster than the 64-row
-    // tiles do (the head, 152064 x 5120 at 64 rows: 319 us against 306 in 64 x 128).
-    if (M <= 64 && tiled_configs[c].bm > 64 && !(halves == 2 && c == 1)) continue;
+    // are the work, but only the paired 128 x 256 and 128 x 192 tiles stream them faster than
+    // the 64-row tiles do (the head, 152064 x 5120 at 64 rows: 319 us against 306 in 64 x 128);
+    // of the two, the one whose tiles spread better over the compute units (18944 x 3584 gated
+    // at 64 rows: 198 tiles of 192 rows 54 us, 148 of 256 rows 61; 27648 x 5120: 145 and 106).
+    if (M <= 64 && tiled_configs[c].bm > 64 && !(halves == 2 && (c == 1 || c == 7))) continue;
     const double time = tiled_time(tiled_configs[c], M, cols, K, halves, out_bytes, 1);
     if (best < 0 || time < best_time) best = c, best_time = time;
   }
