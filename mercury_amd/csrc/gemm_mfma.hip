@@ -817,7 +817,7 @@ struct TiledConfig {
   int bm, bn, resident;
   float rate, alone;
 };
-#define TILED_CONFIGS 8
+#define TILED_CONFIGS 9
 static const TiledConfig tiled_configs[TILED_CONFIGS] = {
     {256, 256, 1, 5.03f, 5.03f},  // 0: 2 stages (128 KB), 16 wavefronts
     {128, 256, 1, 4.7f, 4.7f},    // 1: 3 stages (144 KB), 8 wavefronts
@@ -827,6 +827,7 @@ static const TiledConfig tiled_configs[TILED_CONFIGS] = {
     {64, 128, 1, 2.14f, 2.14f},   // 5: 4 stages (96 KB), 4 wavefronts
     {256, 192, 1, 4.9f, 4.9f},    // 6: 2 stages (112 KB), 8 wavefronts: for widths that 256 divides badly
     {128, 192, 1, 4.45f, 4.45f},  // 7: 3 stages (120 KB), 8 wavefronts
+    {64, 32, 3, 0.6f, 1.2f},      // 8: 4 stages (48 KB), 4 wavefronts: small matrices, few rows
 };
 
 template <int BM, int BN, int STAGES, int WM, int WN, int SPREAD, int EPI>
@@ -858,7 +859,8 @@ static void launch_tiled(int config, const void* x, const void* w, const void* b
     case 4: launch_tiled_cfg<64, 64, 4, 2, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
     case 5: launch_tiled_cfg<64, 128, 4, 1, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
     case 6: launch_tiled_cfg<256, 192, 2, 4, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
-    default: launch_tiled_cfg<128, 192, 3, 4, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    case 7: launch_tiled_cfg<128, 192, 3, 4, 2, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    default: launch_tiled_cfg<64, 32, 4, 4, 1, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
   }
 }
 
