@@ -86,10 +86,26 @@ __device__ __forceinline__ float load_scalar(const void* p, int is_bf16, int i) 
 // be, q and k rotated by the token's position (the four lanes' dims are 4 rotation pairs), q
 // written to q_out, k and v into the paged cache.
 // Formulas: reference mercury/model/qwen2.py:57-64, mercury/model/rope.py:19-29.
-__device__ __forceinline__ void qkv_store(const QkvTarget& p, int m, int head, int dd, float* lo,
-                                          float* hi) {
+// Where token m's keys and values go: its position and the page that holds it (-1: none).
+// Looked up once per token, before any store: the stores might alias the tables for all the
+// compiler knows, and it would fetch them again after each.
+struct QkvPlace {
+  int pos, page;
+};
+
+__device__ __forceinline__ QkvPlace qkv_place(const QkvTarget& p, int m) {
+  QkvPlace place;
+  place.pos = p.positions[m];
+  place.page = p.n_kv > 0 ? p.block_table[(size_t)p.token_seq[m] * p.table_stride +
+                                          (place.pos >> p.page_shift)]
+                          : -1;
+  return place;
+}
+
+__device__ __forceinline__ void qkv_store(const QkvTarget& p, const QkvPlace& place, int m,
+                                          int head, int dd, float* lo, float* hi) {
   const int d = p.d, half = d / 2;
-  const int pos = p.positions[m];
+  const int pos = place.pos;
 #pragma unroll
   for (int i = 0; i < 4; ++i) {
     lo[i] = Elem<bf16_t>::round(lo[i]);
@@ -117,7 +133,7 @@ __device__ __forceinline__ void qkv_store(const QkvTarget& p, int m, int head, i
     *(ushort4*)(dst + half) = hi4;
     return;
   }
-  const int page = p.block_table[(size_t)p.token_seq[m] * p.table_stride + (pos >> p.page_shift)];
+  const int page = place.page;
   if (page < 0) return;
   const int ps = 1 << p.page_shift, off = pos & (ps - 1);
   if (!is_v) {
@@ -319,7 +335,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
           hi[i] += load_scalar(p.bias, p.bias_bf16, n0 + half + g4 * 4 + i);
         }
       }
-      qkv_store(p, m, head, dd, lo, hi);
+      qkv_store(p, qkv_place(p, m), m, head, dd, lo, hi);
     } else {
       float* dst = (float*)p.out + ((size_t)(EPI == SK_PARTIAL ? slice : 0) * M + m) * N;
 #pragma unroll
@@ -727,6 +743,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
     if (m >= M) continue;
     if (EPI == EPI_QKV) {
       const int half = target.d / 2;
+      const QkvPlace place = qkv_place(target, m);
 #pragma unroll
       for (int tb = 0; tb < TN / 2; ++tb) {
         const int pair = n0 + wn / 2 + tb * 16 + g4 * 4;    // 4 pairs, all of one head
@@ -742,7 +759,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
             hi[i] += Elem<TBIAS>::load(bias + head * target.d + half + dd + i);
           }
         }
-        qkv_store(target, m, head, dd, lo, hi);
+        qkv_store(target, place, m, head, dd, lo, hi);
       }
       continue;
     }
