@@ -90,3 +90,23 @@ def test_a_long_prompt_whole_in_portions_and_decoded(shape, dtype):
     replay.check(torch.cat(rows["long"]), want["long"], dtype, "portions and decoded tail")
     replay.check(torch.cat(rows["other"]), want["other"], dtype, "the request beside it")
     assert s.manager.leaked_pages() == 0
+
+
+@pytest.mark.parametrize("shape", ["7b"])
+def test_batched_decoding_through_graphs_at_large_sizes(shape):
+    """Eight requests decoded together through captured graphs (the gated tile for 8 rows, the
+    q/k/v projection as partial sums inside a graph): every token is the plain
+    implementation's choice at its place, or within the bfloat16 bound of it."""
+    from mercury_amd import Engine, EngineConfig, SamplingParams
+    from tests.test_gpu_generate import plausible
+
+    folder, _reqs, _want = model(shape)
+    vocab = SHAPES[shape]["vocab_size"]
+    prompts = [helpers.random_tokens(vocab, 40 + 7 * i, seed=50 + i) for i in range(8)]
+    engine = Engine(EngineConfig(model=str(folder), dtype="bfloat16", num_blocks=128,
+                                 max_model_len=256))
+    got = engine.generate(prompts, SamplingParams(ignore_eos=True), max_tokens=10)
+    assert engine.leaked_blocks() == 0
+    assert any(key[0] == 8 for key in engine.runner.runner.graphs)
+    assert all(len(g) == 10 for g in got)
+    assert all(plausible(folder, p, g) for p, g in zip(prompts, got))
