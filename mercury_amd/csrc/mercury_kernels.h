@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 8
+#define MK_ABI_VERSION 9
 
 #ifdef __cplusplus
 extern "C" {
@@ -61,6 +61,12 @@ int mk_qkv_finish(const float* partials, int num_partials, long long partial_str
                   const int* positions, const int* token_seq, const int* block_table,
                   int table_stride, void* k_cache, void* v_cache, int page_size, int n_q,
                   int n_kv, int d, int rot, int write_kv, int tokens, hipStream_t stream);
+
+// out[i] = mean + std * normal(key, i) for i < n, rounded to the dtype: the values the host
+// core's fill computes for the same key (random_normal.h), so random weights are the same
+// numbers wherever they are drawn.
+int mk_fill_normal(void* out, int dtype, long long n, unsigned long long key, float mean,
+                   float std, hipStream_t stream);
 
 // ---- library "mfma": bfloat16 kernels on the matrix cores
 

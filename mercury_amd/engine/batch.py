@@ -78,28 +78,6 @@ class StepContext:
         return cached
 
 
-def context_from_spans(spans: list, device, token_ids=None) -> StepContext:
-    """A step context without a cache manager: `spans` lists (token count, start position)
-    per sequence.  Block tables are left to the caller."""
-    step = StepContext()
-    counts = [c for c, _ in spans]
-    starts = [s for _, s in spans]
-    cu = np.zeros(len(spans) + 1, dtype=np.int64)
-    np.cumsum(counts, out=cu[1:])
-    token_seq = np.repeat(np.arange(len(spans)), counts)
-    positions = np.arange(int(cu[-1])) - cu[token_seq] + np.asarray(starts)[token_seq]
-    as_dev = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=device)
-    step.num_tokens, step.num_seqs = int(cu[-1]), len(spans)
-    step.token_ids = as_dev(token_ids if token_ids is not None else np.zeros(int(cu[-1])))
-    step.positions, step.token_seq, step.cu_q = as_dev(positions), as_dev(token_seq), as_dev(cu)
-    step.kv_len = as_dev(np.asarray(starts) + np.asarray(counts))
-    step.state_slots = as_dev(np.arange(len(spans)))
-    step.spans = [(int(cu[s]), counts[s], starts[s]) for s in range(len(spans))]
-    step.max_q_len, step.max_kv_len = max(counts), max(s + c for c, s in spans)
-    step.all_decode = step.max_q_len == 1
-    return step
-
-
 class PackedStep:
     """A step flattened into one int32 host buffer (pinned when a GPU will read it), with the
     offsets of its parts: token ids, positions, token -> sequence, prefix sums of the
@@ -151,6 +129,10 @@ def pack_step(chunks: list, manager, vocab_size: int, max_positions: int, pinned
             if not 0 <= w < counts[s]:
                 raise BatchError(f"wanted index {w} outside the {counts[s]} tokens of a sequence")
             rows.append(int(cu[s]) + w)
+        if len(set(c.want)) != len(c.want):
+            # The final norm folds the last projection's partial sums into a wanted row of the
+            # residual stream; a row named twice would receive them twice.
+            raise BatchError(f"sequence {c.key!r} wants the same place twice: {sorted(c.want)}")
     slots = [manager.requests[c.key].state_slot for c in chunks]
 
     needed = max(-(-int(kv) // ps) for kv in kv_len)

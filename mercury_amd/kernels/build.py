@@ -32,6 +32,7 @@ LIBRARIES = {
         "gemm_generic.hip",
         "attention_generic.hip",
         "sampling.hip",
+        "random_fill.hip",
     ],
     "mfma": [
         "host_support.hip",

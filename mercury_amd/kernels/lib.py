@@ -7,11 +7,11 @@ does every op that would have called into it.
 from __future__ import annotations
 
 import ctypes
-from ctypes import c_char_p, c_float, c_int, c_longlong, c_void_p
+from ctypes import c_char_p, c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 from . import build
 
-ABI_VERSION = 8
+ABI_VERSION = 9
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -28,6 +28,7 @@ _SIGNATURES = {
         "mk_argmax": [P, I, I, L, P, P, P],
         "mk_sample_scratch_bytes": [I, I],
         "mk_sample": [P, I, I, L, P, P, P, P, P, P],
+        "mk_fill_normal": [P, I, L, c_ulonglong, F, F, P],
     },
     "mfma": {
         "mk_linear_skinny_slices": [I, I, I],

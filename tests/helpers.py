@@ -67,14 +67,43 @@ def random_tokens(vocab: int, count: int, seed: int) -> list:
     return torch.randint(0, vocab, (count,), generator=g).tolist()
 
 
+def context_from_spans(spans: list, device, token_ids=None):
+    """A step context without a cache manager: `spans` lists (token count, start position)
+    per sequence.  Block tables are left to the caller."""
+    from mercury_amd.engine.batch import StepContext
+
+    step = StepContext()
+    counts = [c for c, _ in spans]
+    starts = [s for _, s in spans]
+    cu = np.zeros(len(spans) + 1, dtype=np.int64)
+    np.cumsum(counts, out=cu[1:])
+    token_seq = np.repeat(np.arange(len(spans)), counts)
+    positions = np.arange(int(cu[-1])) - cu[token_seq] + np.asarray(starts)[token_seq]
+    as_dev = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=device)
+    step.num_tokens, step.num_seqs = int(cu[-1]), len(spans)
+    step.token_ids = as_dev(token_ids if token_ids is not None else np.zeros(int(cu[-1])))
+    step.positions, step.token_seq, step.cu_q = as_dev(positions), as_dev(token_seq), as_dev(cu)
+    step.kv_len = as_dev(np.asarray(starts) + np.asarray(counts))
+    step.state_slots = as_dev(np.arange(len(spans)))
+    step.spans = [(int(cu[s]), counts[s], starts[s]) for s in range(len(spans))]
+    step.max_q_len, step.max_kv_len = max(counts), max(s + c for c, s in spans)
+    step.all_decode = step.max_q_len == 1
+    return step
+
+
 class TraceRun:
     """Drives ``bin/trace_run`` as a child process, one step at a time."""
 
-    def __init__(self, folder, dtype: str, max_tokens: int):
+    def __init__(self, folder, dtype: str, max_tokens: int, block_size=None, max_live=None):
         self.out = Path(tempfile.mkdtemp(prefix="mercury_trace_"))
+        options = []
+        if block_size is not None:
+            options += ["--block-size", str(block_size)]
+        if max_live is not None:
+            options += ["--max-live", str(max_live)]
         self.proc = subprocess.Popen(
             [sys.executable, str(ROOT / "bin" / "trace_run"), "--model", str(folder), "--dtype",
-             dtype, "--out", str(self.out), "--max-tokens", str(max_tokens)],
+             dtype, "--out", str(self.out), "--max-tokens", str(max_tokens), *options],
             stdin=subprocess.PIPE, stdout=subprocess.PIPE, text=True)
         self.step_no = 0
         self.vocab = json.loads((Path(folder) / "config.json").read_text())["vocab_size"]

@@ -6,8 +6,12 @@ imports from ``mercury_amd``: the engine under test and this file only share the
 folder on disk (``config.json`` + ``model.safetensors``, the latter read through the
 ``safetensors`` package, which the engine does not use).
 
-All arithmetic runs in one floating-point type (float32 by default, float64 on request), so
-the reference's casts to the model dtype are the identity here.
+All tensors have one floating-point type, the one the weights are read in: float32 by default
+(float64 on request), where the reference's casts to the model dtype are the identity.  Read in
+bfloat16, every function rounds where the reference rounds to the model dtype (after each
+projection, sum, norm, rotation and activation), with the statistics of norms and softmax in
+float32 as there; the distance of that run from the float32 run is what bfloat16 costs the
+reference itself, which the tests use as the measure of the engine's bfloat16 error.
 """
 
 from __future__ import annotations
@@ -51,6 +55,12 @@ def read_weights(folder, dtype=torch.float32) -> dict:
 # --------------------------------------------------------------------------- parts
 
 
+def _wide(dtype):
+    """The type statistics are computed in: float32, as the reference's `.float()`
+    (mercury/model/qwen2.py:29-30), or the tensors' own when that is wider."""
+    return torch.promote_types(dtype, torch.float32)
+
+
 def rms_norm(x, weight, eps, residual=None):
     """(normalised * weight, x + residual).  mercury/model/qwen2.py:27-31.
 
@@ -59,8 +69,9 @@ def rms_norm(x, weight, eps, residual=None):
     """
     if residual is not None:
         x = x + residual
-    variance = x.pow(2).mean(-1, keepdim=True)
-    normed = x * torch.rsqrt(variance + eps)
+    wide = x.to(_wide(x.dtype))
+    variance = wide.pow(2).mean(-1, keepdim=True)
+    normed = (wide * torch.rsqrt(variance + eps)).to(x.dtype)
     return normed * weight, x
 
 
@@ -101,6 +112,8 @@ def causal_attention(q, k, v, scale, query_offset=0, window=None):
     `window`, when given, additionally hides keys with j <= p - window; the reference has
     no window, the argument exists for the cache manager's window groups.
     """
+    out_dtype = q.dtype
+    q, k, v = (t.to(_wide(out_dtype)) for t in (q, k, v))     # scores and softmax in float32
     groups = q.shape[1] // k.shape[1]
     k = k.repeat_interleave(groups, dim=1)
     v = v.repeat_interleave(groups, dim=1)
@@ -112,12 +125,13 @@ def causal_attention(q, k, v, scale, query_offset=0, window=None):
         hidden = hidden | (key_pos[None, None, :] <= query_pos[None, :, None] - window)
     scores = scores.masked_fill(hidden, float("-inf"))
     weights = torch.softmax(scores, dim=-1)
-    return torch.einsum("hqk,khd->qhd", weights, v)
+    return torch.einsum("hqk,khd->qhd", weights, v).to(out_dtype)
 
 
 def silu(z):
     """z * sigmoid(z), the activation of the gated MLP (mercury/model/qwen2.py:42)."""
-    return z / (1.0 + torch.exp(-z))
+    wide = z.to(_wide(z.dtype))
+    return (wide / (1.0 + torch.exp(-wide))).to(z.dtype)
 
 
 def gated_mlp(x, gate_w, up_w, down_w):

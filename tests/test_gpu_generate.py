@@ -36,13 +36,18 @@ def generate(eng, prompts, max_tokens=12, **params):
     return out
 
 
-def plausible(folder, prompt, tokens, fraction=0.02):
-    """Every generated token is the plain model's argmax at its place, or within the
-    bfloat16 bound of it (2% of the largest logit)."""
+def plausible(folder, prompt, tokens):
+    """Every generated token is the plain model's argmax at its place, or so close to it that
+    the bfloat16 error allowed on each of the two logits (the bound the replay tests derive
+    from the plain implementation's own bfloat16 run) can have swapped them."""
+    from tests.test_gpu_replay import BF16_SLACK, bf16_cost
+
     w, cfg = helpers.plain_model(folder)
-    logits = plain.forward_logits(w, cfg, prompt + tokens)[len(prompt) - 1:-1]
+    whole = plain.forward_logits(w, cfg, prompt + tokens)
+    allowed = 2 * BF16_SLACK * bf16_cost(folder, cfg, prompt + tokens, whole)
+    logits = whole[len(prompt) - 1:-1]
     chosen = logits[torch.arange(len(tokens)), torch.tensor(tokens)]
-    return bool((logits.max(-1).values - chosen <= 2 * fraction * logits.abs().max()).all())
+    return bool((logits.max(-1).values - chosen <= allowed).all())
 
 
 @pytest.mark.parametrize("name", ["A", "B", "C"])
@@ -101,7 +106,9 @@ def test_every_policy_produces_the_same_tokens():
 
 
 def test_temperature_sampling_is_per_request_reproducible():
-    """(BASELINE configuration B: temperature 0.8 under a seeded generator.)  A request draws
+    """Tiny configuration B with its own workload: pages of 8 tokens, prompts of 1, 9, 40 and
+    64 tokens of which two share their first 24, portions of 16 beside decoded tokens,
+    temperature 0.8 under a seeded generator.  A request draws
     the same tokens alone, in a batch and cut into portions of 16."""
     folder = helpers.model_folder("B")
     vocab = 1000
@@ -113,7 +120,8 @@ def test_temperature_sampling_is_per_request_reproducible():
     def run(which, **kw):
         from mercury_amd import SamplingParams
 
-        eng = engine("B", block_size=8, num_blocks=64, seed=5, **kw)
+        kw.setdefault("seed", 5)
+        eng = engine("B", block_size=8, num_blocks=64, **kw)
         outs = {}
         for i in which:
             eng.submit(f"req{i}", prompts[i], 6, lambda e, i=i: outs.setdefault(i, []).append(e),
@@ -127,10 +135,10 @@ def test_temperature_sampling_is_per_request_reproducible():
     for i in range(4):
         assert run([i])[i] == batched[i]
     assert len({tuple(v) for v in batched.values()}) == 4
-    other_seed = engine("B", block_size=8, num_blocks=64, seed=6)
-    from mercury_amd import SamplingParams
-    assert other_seed.generate([prompts[3]], SamplingParams(temperature=0.8), 6) != [batched[3]] \
-        or True  # a different seed may coincide on a peaked distribution; the run must succeed
+    # another seed draws other tokens: over four requests of six tokens from a flat
+    # distribution (the largest probability is a few per cent) at least one draw differs
+    other = run(range(4), prefill_budget=16, seed=6)
+    assert any(other[i] != batched[i] for i in range(4))
 
 
 def test_command_line_generates_and_writes_random_weights(tmp_path):

@@ -576,7 +576,7 @@ def run_attention(q_h, k_h, v_h, dtype, pages_per_seq, page, num_pages, seq_lens
     """q_h: list per sequence of [q_len, n_q, d] (the last q_len positions of the sequence);
     k_h/v_h: list per sequence of [seq_len, n_kv, d].  `hide_before`: per sequence, the number
     of leading pages to drop from the table (-1) and to poison, as after a window passed."""
-    from mercury_amd.engine.batch import context_from_spans
+    from tests.helpers import context_from_spans
 
     n_q, d = q_h[0].shape[1:]
     n_kv = k_h[0].shape[1]

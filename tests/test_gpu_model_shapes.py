@@ -54,7 +54,8 @@ def model(shape):
         reqs = {"long": helpers.random_tokens(cfg["vocab_size"], 700, seed=1),
                 "other": helpers.random_tokens(cfg["vocab_size"], 90, seed=2)}
         want = {k: plain.forward_logits(weights, plain_cfg, v) for k, v in reqs.items()}
-        _MODELS[shape] = (folder, reqs, want)
+        cost = {k: replay.bf16_cost(folder, plain_cfg, v, want[k]) for k, v in reqs.items()}
+        _MODELS[shape] = (folder, reqs, want, cost)
     return _MODELS[shape]
 
 
@@ -67,10 +68,13 @@ CASES = [(shape, dtype) for shape in sorted(SHAPES) for dtype in ("float32", "bf
 
 @pytest.mark.parametrize("shape,dtype", CASES)
 def test_a_long_prompt_whole_in_portions_and_decoded(shape, dtype):
-    folder, reqs, want = model(shape)
-    s = replay.session(folder, dtype, 1024)
+    from mercury_amd.engine.replay import ReplaySession
+
+    folder, reqs, want, cost = model(shape)
+    s = ReplaySession(folder, dtype, 1024)
     long, other = reqs["long"], reqs["other"]
-    replay.check(s.step([replay.entry("w", long)], ["w"]), want["long"], dtype, "whole")
+    replay.check(s.step([replay.entry("w", long)], ["w"]), want["long"], dtype, "whole",
+                 cost["long"])
 
     # the prompt in three portions: the second beside the other request's prompt, the third of
     # 40 tokens by itself (few rows over the large matrices); then its last 40 tokens one at a
@@ -87,8 +91,10 @@ def test_a_long_prompt_whole_in_portions_and_decoded(shape, dtype):
                       replay.entry("other", other[50 + i:51 + i])], ["long", "other"] if last else [])
         rows["long"].append(out[:1])
         rows["other"].append(out[1:])
-    replay.check(torch.cat(rows["long"]), want["long"], dtype, "portions and decoded tail")
-    replay.check(torch.cat(rows["other"]), want["other"], dtype, "the request beside it")
+    replay.check(torch.cat(rows["long"]), want["long"], dtype, "portions and decoded tail",
+                 cost["long"])
+    replay.check(torch.cat(rows["other"]), want["other"], dtype, "the request beside it",
+                 cost["other"])
     assert s.manager.leaked_pages() == 0
 
 
@@ -100,7 +106,7 @@ def test_batched_decoding_through_graphs_at_large_sizes(shape):
     from mercury_amd import Engine, EngineConfig, SamplingParams
     from tests.test_gpu_generate import plausible
 
-    folder, _reqs, _want = model(shape)
+    folder, _reqs, _want, _cost = model(shape)
     vocab = SHAPES[shape]["vocab_size"]
     prompts = [helpers.random_tokens(vocab, 40 + 7 * i, seed=50 + i) for i in range(8)]
     engine = Engine(EngineConfig(model=str(folder), dtype="bfloat16", num_blocks=128,

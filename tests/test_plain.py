@@ -99,6 +99,89 @@ def test_slot_mapping_vectors():
     assert slots[:16] == [7 * 16 + i for i in range(16)] and slots[16:] == [16 + i for i in range(4)]
 
 
+def _library_attention(x, w, prefix, cfg, cos, sin):
+    """The attention layer from library routines only: `F.linear`, the rotation (pinned
+    above), and `F.scaled_dot_product_attention` with its default scale, which is
+    1 / sqrt(head size): the reference's `head_dim ** -0.5` (mercury/model/qwen2.py:54)."""
+    F = torch.nn.functional
+    n_q, n_kv, d = cfg["num_attention_heads"], cfg["num_key_value_heads"], cfg["head_dim"]
+    t = x.shape[0]
+    q = F.linear(x, w[prefix + "q_proj.weight"], w[prefix + "q_proj.bias"]).view(t, n_q, d)
+    k = F.linear(x, w[prefix + "k_proj.weight"], w[prefix + "k_proj.bias"]).view(t, n_kv, d)
+    v = F.linear(x, w[prefix + "v_proj.weight"], w[prefix + "v_proj.bias"]).view(t, n_kv, d)
+    q, k = plain.apply_rotary(q, k, cos, sin)
+    k, v = (z.repeat_interleave(n_q // n_kv, 1) for z in (k, v))
+    out = F.scaled_dot_product_attention(q.transpose(0, 1)[None], k.transpose(0, 1)[None],
+                                         v.transpose(0, 1)[None], is_causal=True)[0]
+    return F.linear(out.transpose(0, 1).reshape(t, n_q * d), w[prefix + "o_proj.weight"])
+
+
+def test_the_score_scale_is_the_library_default():
+    """A scale of 1, of 1/d or a missing scale fails this; so does a bias on the output
+    projection or none on q/k/v."""
+    for name in ("A", "C"):
+        w, cfg = helpers.plain_model(helpers.model_folder(name, std=0.3))
+        g = torch.Generator().manual_seed(4)
+        x = torch.randn(19, cfg["hidden_size"], generator=g)
+        cos, sin = plain.rotary_table(cfg["head_dim"], range(19), cfg["rope_theta"])
+        prefix = "model.layers.0.self_attn."
+        want = _library_attention(x, w, prefix, cfg, cos, sin)
+        got = plain.attention_layer(x, w, prefix, cfg, cos, sin)
+        torch.testing.assert_close(got, want, atol=1e-5, rtol=1e-4)
+
+
+def test_the_layers_are_pre_norm_around_a_running_sum():
+    """The reference carries `residual` through its norms (mercury/model/qwen2.py:82-94,
+    :110-114).  Written out, that is h <- h + attention(norm(h)); h <- h + mlp(norm(h)) from
+    h = embedding, and norm(h) at the end: composed here from library routines
+    (`F.rms_norm`, `F.linear`, `F.silu`, library attention).  A norm after the sum instead of
+    before it, a forgotten sum, or the final norm applied to the last layer's output alone
+    fails this."""
+    F = torch.nn.functional
+    for name in ("A", "B", "C"):
+        w, cfg = helpers.plain_model(helpers.model_folder(name, std=0.2))
+        eps, width = cfg["rms_norm_eps"], (cfg["hidden_size"],)
+        tokens = helpers.random_tokens(cfg["vocab_size"], 23, seed=8)
+        cos, sin = plain.rotary_table(cfg["head_dim"], range(len(tokens)), cfg["rope_theta"])
+        h = w["model.embed_tokens.weight"][torch.tensor(tokens)]
+        for i in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{i}."
+            a = F.rms_norm(h, width, w[p + "input_layernorm.weight"], eps)
+            h = h + _library_attention(a, w, p + "self_attn.", cfg, cos, sin)
+            m = F.rms_norm(h, width, w[p + "post_attention_layernorm.weight"], eps)
+            h = h + F.linear(F.silu(F.linear(m, w[p + "mlp.gate_proj.weight"]))
+                             * F.linear(m, w[p + "mlp.up_proj.weight"]), w[p + "mlp.down_proj.weight"])
+        y = F.rms_norm(h, width, w["model.norm.weight"], eps)
+        head = w["model.embed_tokens.weight"] if cfg["tie_word_embeddings"] else w["lm_head.weight"]
+        want = F.linear(y, head)
+        got = plain.forward_logits(w, cfg, tokens)
+        assert want.abs().max() > 0.5       # weights wide enough that every part matters
+        torch.testing.assert_close(got, want, atol=2e-5, rtol=1e-4)
+        # and every part does matter: without the sums the logits are others
+        for drop in ("self_attn.o_proj.weight", "mlp.down_proj.weight"):
+            cut = {k: (torch.zeros_like(v) if k.endswith(drop) else v) for k, v in w.items()}
+            assert (plain.forward_logits(cut, cfg, tokens) - got).abs().max() > 1e-2
+
+
+def test_bfloat16_run_rounds_where_the_reference_rounds():
+    """Read in bfloat16 the plain implementation keeps every tensor in bfloat16 (the
+    reference's casts, mercury/model/qwen2.py:27-31, mercury/model/rope.py:46-47) and stays
+    close to the float32 run: a fraction of a per cent of the logits' range, not more."""
+    folder = helpers.model_folder("B")
+    w, cfg = helpers.plain_model(folder)
+    tokens = helpers.random_tokens(cfg["vocab_size"], 60, seed=3)
+    exact = plain.forward_logits(w, cfg, tokens)
+    rounded = plain.forward_logits(plain.read_weights(folder, torch.bfloat16), cfg, tokens)
+    assert rounded.dtype == torch.bfloat16
+    gap = float((rounded.float() - exact).abs().max())
+    assert 0 < gap < 0.03 * float(exact.abs().max())
+    normed, summed = plain.rms_norm(torch.full((1, 8), 3.0, dtype=torch.bfloat16),
+                                    torch.ones(8, dtype=torch.bfloat16), 1e-6,
+                                    residual=torch.full((1, 8), 0.0078125, dtype=torch.bfloat16))
+    assert summed.dtype == normed.dtype == torch.bfloat16
+    assert float(summed[0, 0]) == 3.0       # the sum itself is rounded to bfloat16 first
+
+
 def test_whole_model_invariants():
     folder = helpers.model_folder("B")
     w, cfg = helpers.plain_model(folder)
