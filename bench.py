@@ -95,32 +95,21 @@ class Bench:
                  lookahead: bool = True, prefill_budget: int = 8192):
         import torch
 
-        from mercury_amd.cache import CacheManager, PageHasher
-        from mercury_amd.config import EngineConfig, build_model
-        from mercury_amd.engine.engine import Engine
-        from mercury_amd.engine.executor import GpuExecutor
-        from mercury_amd.engine.runner import ModelRunner
-        from mercury_amd.sampling import Sampler
-        from mercury_amd.weights import RandomSource, load_weights
+        from mercury_amd import Engine, EngineConfig
 
         self.torch = torch
         self.cfg = cfg
-        device = torch.device("cuda:0")
         t0 = time.time()
-        model = build_model(cfg)
-        torch_dtype = torch.bfloat16 if dtype == "bfloat16" else torch.float32
-        load_weights(model, RandomSource(model, seed, 0.02, torch_dtype, device), torch_dtype, device)
         pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + PREFILL_TOKENS // BLOCK_SIZE + 8
         self.engine_cfg = EngineConfig(
-            model="random", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
+            model="random", random_weights=True, weight_seed=seed, weight_std=0.02,
+            device="cuda:0", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
             max_running=max_batch + 1, prefill_budget=prefill_budget,
             max_model_len=max(context, PREFILL_TOKENS) + 128, seed=seed,
             lookahead=lookahead)
-        manager = CacheManager(model.cache_slots, pages, BLOCK_SIZE, max_batch + 1, False)
-        runner = ModelRunner(model, manager, torch_dtype, device, max(context, PREFILL_TOKENS) + 128)
-        self.engine = Engine(self.engine_cfg, executor=GpuExecutor(runner, Sampler(seed), lookahead=self.engine_cfg.lookahead),
-                             manager=manager, eos_token_ids=())
-        self.model, self.runner, self.manager = model, runner, manager
+        self.engine = Engine(self.engine_cfg, model_config=cfg, eos_token_ids=())
+        self.runner, self.manager = self.engine.executor.runner, self.engine.manager
+        self.model = model = self.runner.model
         self.rng = torch.Generator().manual_seed(seed)
         self.counter = 0
         print(f"[bench] model ready in {time.time() - t0:.1f} s: "

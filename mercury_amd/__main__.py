@@ -17,7 +17,12 @@ def build_parser() -> argparse.ArgumentParser:
     sub = parser.add_subparsers(dest="command", required=True)
 
     g = sub.add_parser("generate", help="generate tokens for prompts given as token ids")
-    g.add_argument("--model", required=True, help="folder with config.json and safetensors weights")
+    g.add_argument("--model", default=None, help="folder with config.json and safetensors weights")
+    g.add_argument("--random-config", default=None, metavar="CONFIG_JSON",
+                   help="instead of --model: a config.json (or a folder with one) whose model "
+                        "gets random weights, drawn from --weight-seed")
+    g.add_argument("--weight-seed", type=int, default=0)
+    g.add_argument("--weight-std", type=float, default=0.02)
     g.add_argument("--prompt-ids", action="append", default=[],
                    help="one prompt as comma- or space-separated token ids; may be repeated")
     g.add_argument("--prompt-file", default=None,
@@ -65,7 +70,7 @@ def parse_prompt(text: str) -> list:
 def run_generate(args) -> int:
     from .config.engine_config import EngineConfig
     from .engine.engine import Engine
-    from .engine.request import SamplingParams
+    from .engine import SamplingParams
 
     prompts = [parse_prompt(p) for p in args.prompt_ids]
     if args.prompt_file:
@@ -74,8 +79,12 @@ def run_generate(args) -> int:
     if not prompts:
         print("no prompts: give --prompt-ids or --prompt-file", file=sys.stderr)
         return 2
+    if (args.model is None) == (args.random_config is None):
+        print("give exactly one of --model and --random-config", file=sys.stderr)
+        return 2
     cfg = EngineConfig(
-        model=args.model, device=args.device, dtype=args.dtype, block_size=args.block_size,
+        model=args.model or args.random_config, random_weights=args.model is None,
+        weight_seed=args.weight_seed, weight_std=args.weight_std, device=args.device, dtype=args.dtype, block_size=args.block_size,
         num_blocks=args.num_blocks, max_running=args.max_running,
         prefill_budget=args.prefill_budget, max_model_len=args.max_model_len, policy=args.policy,
         aging_tokens_per_s=args.aging_tokens_per_s, max_wait_s=args.max_wait_s,

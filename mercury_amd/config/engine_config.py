@@ -34,6 +34,12 @@ class EngineConfig:
     aging_tokens_per_s, max_wait_s, scan_limit   parameters of the policies
     cryptographic_hashes   SHA-256 page hashes instead of the fast 64-bit ones
     seed             seed of the per-request sampling streams
+    random_weights   draw the weights instead of reading them: `model` then names a folder
+                     with a ``config.json`` (or that file), or the engine is given the
+                     configuration as a dict; weight_seed and weight_std (the normal
+                     deviates' spread; norm weights are 1 + deviate) say which weights,
+                     weight_dtype the storage type they are rounded to, as a checkpoint's
+                     would be, before the engine converts them to its own dtype
     """
 
     model: str = ""
@@ -56,6 +62,11 @@ class EngineConfig:
     cryptographic_hashes: bool = False
     seed: int = 0
 
+    random_weights: bool = False
+    weight_seed: int = 0
+    weight_std: float = 0.02
+    weight_dtype: str = "bfloat16"
+
     idle_sleep_s: float = 5e-4
     max_step_records: int = 500_000
     debug_invariants: bool = False
@@ -73,6 +84,8 @@ class EngineConfig:
             raise ValueError(
                 f"unsupported dtype {self.dtype!r}; this engine runs {sorted(set(_DTYPE_BY_NAME))}"
             )
+        if self.weight_dtype not in _DTYPE_BY_NAME:
+            raise ValueError(f"unsupported weight_dtype {self.weight_dtype!r}")
         if self.block_size <= 0 or self.block_size & (self.block_size - 1):
             raise ValueError("block_size must be a positive power of two")
         if self.max_running <= 0:

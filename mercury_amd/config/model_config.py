@@ -19,7 +19,10 @@ class ConfigError(ValueError):
 
 
 def read_config_json(folder) -> dict:
-    path = Path(folder) / "config.json"
+    """The parsed ``config.json`` of a model folder (or the file itself, when given that)."""
+    path = Path(folder)
+    if path.is_dir() or path.name != "config.json":
+        path = path / "config.json"
     if not path.is_file():
         raise FileNotFoundError(f"no config.json under {folder}")
     return json.loads(path.read_text())

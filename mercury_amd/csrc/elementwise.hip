@@ -322,7 +322,7 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
                                      const int* __restrict__ block_table, int table_stride,
                                      T* __restrict__ k_cache, T* __restrict__ v_cache,
                                      int page_shift, int n_q, int n_kv, int d, int rot,
-                                     int write_kv) {
+                                     int interleaved, int write_kv) {
   const int t = blockIdx.x;
   const int pos = positions[t];
   const int half = rot / 2;
@@ -330,14 +330,16 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
   const float* sn = sin_table + (size_t)pos * half;
   T* row = qkv + (size_t)t * row_stride;
 
-  // q heads: pairwise, in place.
+  // q heads: pairwise, in place.  Pair j is dims (j, j + half), or (2j, 2j + 1) when the
+  // layout is interleaved.
   for (int idx = threadIdx.x; idx < n_q * half; idx += blockDim.x) {
     const int head = idx / half, j = idx - head * half;
     T* x = row + head * d;
-    const float a = Elem<T>::load(x + j), b = Elem<T>::load(x + j + half);
+    const int ia = interleaved ? 2 * j : j, ib = interleaved ? 2 * j + 1 : j + half;
+    const float a = Elem<T>::load(x + ia), b = Elem<T>::load(x + ib);
     const float c = cs[j], s = sn[j];
-    Elem<T>::store(x + j, a * c - b * s);
-    Elem<T>::store(x + j + half, b * c + a * s);
+    Elem<T>::store(x + ia, a * c - b * s);
+    Elem<T>::store(x + ib, b * c + a * s);
   }
   if (!write_kv) return;
 
@@ -353,7 +355,11 @@ __global__ void rope_kv_write_kernel(T* __restrict__ qkv, int row_stride,
     const size_t dst = (((size_t)page * n_kv + head) * page_size + off) * d + j;
     const T* x = k_src + head * d;
     float y;
-    if (j < half) {
+    if (interleaved && j < rot) {
+      const int pair = j >> 1;
+      y = (j & 1) ? Elem<T>::load(x + j) * cs[pair] + Elem<T>::load(x + j - 1) * sn[pair]
+                  : Elem<T>::load(x + j) * cs[pair] - Elem<T>::load(x + j + 1) * sn[pair];
+    } else if (j < half) {
       y = Elem<T>::load(x + j) * cs[j] - Elem<T>::load(x + j + half) * sn[j];
     } else if (j < rot) {
       y = Elem<T>::load(x + j) * cs[j - half] + Elem<T>::load(x + j - half) * sn[j - half];
@@ -370,7 +376,7 @@ extern "C" int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const floa
                                 const int* positions, const int* token_seq,
                                 const int* block_table, int table_stride, void* k_cache,
                                 void* v_cache, int page_size, int n_q, int n_kv, int d, int rot,
-                                int write_kv, int tokens, hipStream_t stream) {
+                                int interleaved, int write_kv, int tokens, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv >= 0 && d > 0, "rope: bad sizes");
   MK_REQUIRE(rot >= 0 && rot <= d && rot % 2 == 0, "rope: rotary width %d not in [0, %d] / even",
              rot, d);
@@ -384,12 +390,12 @@ extern "C" int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const floa
     rope_kv_write_kernel<float><<<tokens, threads, 0, stream>>>(
         (float*)qkv, row_stride, cos_table, sin_table, positions, token_seq, block_table,
         table_stride, (float*)k_cache, (float*)v_cache, mk_log2(page_size), n_q, n_kv, d, rot,
-        write_kv);
+        interleaved, write_kv);
   else if (dtype == MK_BF16)
     rope_kv_write_kernel<bf16_t><<<tokens, threads, 0, stream>>>(
         (bf16_t*)qkv, row_stride, cos_table, sin_table, positions, token_seq, block_table,
         table_stride, (bf16_t*)k_cache, (bf16_t*)v_cache, mk_log2(page_size), n_q, n_kv, d, rot,
-        write_kv);
+        interleaved, write_kv);
   else
     MK_REQUIRE(false, "rope: unknown dtype %d", dtype);
   MK_LAUNCH_CHECK("rope_kv_write");

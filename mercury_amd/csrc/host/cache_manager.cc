@@ -113,13 +113,13 @@ int CacheManager::leaked_pages() const {
 
 const Sequence& CacheManager::sequence(const std::string& key) const {
   auto it = sequences_.find(key);
-  if (it == sequences_.end()) throw std::out_of_range("'" + key + "' holds nothing in the cache");
+  if (it == sequences_.end()) throw UnknownSequence(key);
   return it->second;
 }
 
 Sequence& CacheManager::mutable_sequence(const std::string& key) {
   auto it = sequences_.find(key);
-  if (it == sequences_.end()) throw std::out_of_range("'" + key + "' holds nothing in the cache");
+  if (it == sequences_.end()) throw UnknownSequence(key);
   return it->second;
 }
 
@@ -240,7 +240,7 @@ void CacheManager::commit(const std::string& key, const std::vector<PageHash>& c
 
 void CacheManager::release(const std::string& key) {
   auto it = sequences_.find(key);
-  if (it == sequences_.end()) throw std::out_of_range("'" + key + "' holds nothing in the cache");
+  if (it == sequences_.end()) throw UnknownSequence(key);
   for (int g = 0; g < (int)groups_.size(); ++g) {
     std::vector<int> live;
     for (int page : it->second.tables[g]) {

@@ -34,6 +34,13 @@ struct GroupSpec {
   }
 };
 
+// A key that names no admitted sequence.
+class UnknownSequence : public std::out_of_range {
+ public:
+  explicit UnknownSequence(const std::string& key)
+      : std::out_of_range("'" + key + "' holds nothing in the cache") {}
+};
+
 class StateSlots {
  public:
   explicit StateSlots(int count);

@@ -1,0 +1,193 @@
+#include "dispatch.h"
+
+#include <algorithm>
+
+#include "kernels.h"
+
+namespace mercury {
+
+namespace {
+// Thresholds, each with the measurement that set it.
+constexpr int kSkinnyMaxRows = 64;
+// K-split partial sums: the skinny kernel up to here, tiles beyond.
+constexpr int kSkinnySplitMaxRows = 16;
+// Larger matrices stream faster through the tiled kernel's ring of LDS buffers
+// (5120 x 27648 at 8 rows: 57 against 50 us; 896 x 4864: 4.8 against 5.4).
+constexpr int64_t kSkinnySplitMaxWeights = 20ll << 20;
+// Head and gated projection: the skinny kernel below this many rows, tiles from here (the
+// head, 152064 x 3584, at 1, 8, 16, 64 rows: skinny 188, 204, 238, 429 us; tiles 187, 191,
+// 198, 221).
+constexpr int kTiledMinRows = 8;
+// A q/k/v matrix from this size on goes as partial sums and a finishing kernel (4608 x 3584 at
+// 8, 16, 32, 64 rows: 14.0, 13.9, 15.4, 16.5 us against 15.2, 16.1, 21.1, 30.7 in the one
+// skinny kernel; 1152 x 896 the other way round: 10.6 against 6.0).
+constexpr int64_t kFusedQkvSplitWeights = 24ll << 20;
+constexpr int kFusedQkvTiledRows = 256;
+constexpr int kFusedQkvMinWorkgroups = 128;
+
+constexpr int kAttentionTargetWaves = 1024;
+constexpr int kAttentionStagedWorkgroups = 64;
+constexpr int kAttentionStagedMaxWaves = 8192;
+constexpr int kAttentionWideTileWaves = 400;
+constexpr int kAttentionMinBlocksPerSplit = 2;
+// Beyond this the merge of the parts costs more than the shorter chains save (one sequence
+// of 16,384 tokens, 28 heads of 128: 25 us with 256 parts, 17 with 64 or 128).
+constexpr int kAttentionMaxSplits = 128;
+
+bool partials_by_skinny(int m, int n, int k) {
+  return m <= kSkinnySplitMaxRows && (int64_t)n * k * 2 < kSkinnySplitMaxWeights;
+}
+}  // namespace
+
+bool mfma_eligible(int x_dtype, int w_dtype, int m, int k) {
+  return x_dtype == kBF16 && w_dtype == kBF16 && m > 0 && k % 8 == 0;
+}
+
+bool wants_partials(int x_dtype, int w_dtype, int m, int n, int k) {
+  if (!mfma_eligible(x_dtype, w_dtype, m, k)) return false;
+  const KernelTable& t = need_mfma();
+  if (partials_by_skinny(m, n, k)) return !t.mk_linear_skinny_unsplit(m, n, k);
+  return t.mk_linear_tiled_slices(m, n, k) > 1;
+}
+
+PartialsPlan plan_partials(int m, int n, int k) {
+  const KernelTable& t = need_mfma();
+  PartialsPlan plan;
+  plan.skinny = partials_by_skinny(m, n, k);
+  plan.slices = plan.skinny ? t.mk_linear_skinny_slices(m, n, k) : t.mk_linear_tiled_slices(m, n, k);
+  return plan;
+}
+
+LinearKind choose_linear(int x_dtype, int m, int n, int k, bool has_bias, bool accumulate,
+                         int out_dtype, int force) {
+  (void)n;
+  bool mfma = force == 2 || (force == 0 && x_dtype == kBF16 && k % 8 == 0);
+  if (!mfma) return LinearKind::GENERIC;
+  if (x_dtype != kBF16 || k % 8) {
+    throw KernelError("linear: the matrix-core kernels take bfloat16 with K % 8 == 0");
+  }
+  if (m < kTiledMinRows && out_dtype == kF32 && !has_bias && !accumulate) return LinearKind::SKINNY;
+  if (m <= kSkinnySplitMaxRows && accumulate) return LinearKind::SKINNY_ACC;
+  return LinearKind::TILED;
+}
+
+bool fuses_gating(int x_dtype, int w_dtype, int m, int k, int rows_of_w) {
+  return x_dtype == kBF16 && w_dtype == kBF16 && m > 0 && k % 8 == 0 && rows_of_w % 2 == 0;
+}
+
+bool gated_is_skinny(int m) { return m < kTiledMinRows; }
+
+bool qkv_fusable(int x_dtype, int w_dtype, int m, int k, int head_dim, int rotary_dim,
+                 int page_size, bool half_layout) {
+  return mfma_eligible(x_dtype, w_dtype, m, k) && head_dim % 32 == 0 &&
+         (rotary_dim == 0 || rotary_dim == head_dim) && (half_layout || rotary_dim == 0) &&
+         page_size > 0 && (page_size & (page_size - 1)) == 0;
+}
+
+QkvKind choose_qkv(int x_dtype, int w_dtype, int m, int width, int k, int head_dim,
+                   int rotary_dim, int page_size, bool half_layout) {
+  const bool half = half_layout || rotary_dim == 0;
+  auto unfused = [&]() {
+    // the finishing kernel rotates in the half-split layout only
+    return half && wants_partials(x_dtype, w_dtype, m, width, k) ? QkvKind::PARTIALS_FINISH
+                                                                 : QkvKind::LINEAR_ROPE;
+  };
+  if (!qkv_fusable(x_dtype, w_dtype, m, k, head_dim, rotary_dim, page_size, half_layout)) {
+    return unfused();
+  }
+  const bool partials = wants_partials(x_dtype, w_dtype, m, width, k);
+  if (m <= kFusedQkvTiledRows && (int64_t)width * k * 2 >= kFusedQkvSplitWeights && partials) {
+    return QkvKind::PARTIALS_FINISH;
+  }
+  if (m <= 16 || (m <= kSkinnyMaxRows && width / 32 >= kFusedQkvMinWorkgroups)) return QkvKind::SKINNY;
+  // many rows: partial sums would be a second pass over [rows, width] in float32
+  if (m > kFusedQkvTiledRows || !partials) return QkvKind::TILED;
+  return QkvKind::PARTIALS_FINISH;
+}
+
+int count_tiles(const std::vector<int>& counts, int group, int tile_rows) {
+  int total = 0;
+  for (int c : counts) total += (c * group + tile_rows - 1) / tile_rows;
+  return total;
+}
+
+void build_tiles(const std::vector<int>& counts, int group, int tile_rows, std::vector<int>& seq,
+                 std::vector<int>& row0) {
+  for (int s = 0; s < (int)counts.size(); ++s) {
+    const int n = (counts[s] * group + tile_rows - 1) / tile_rows;
+    for (int i = 0; i < n; ++i) {
+      seq.push_back(s);
+      row0.push_back(i * tile_rows);
+    }
+  }
+}
+
+AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, int n_kv, int window,
+                             const std::vector<int>& counts, int max_q_len, int max_kv_len,
+                             int force, int tile_rows, int staged_in, int splits_in,
+                             int split_blocks_in) {
+  AttentionPlan plan;
+  plan.mfma = force == 2;
+  if (force == 0 && dtype == kBF16) {
+    plan.mfma = need_mfma().mk_attention_mfma_supported(head_dim, page_size) != 0;
+  }
+  if (!plan.mfma) return plan;
+  if (dtype != kBF16) throw KernelError("attention: the matrix-core kernel takes bfloat16 only");
+  const KernelTable& t = need_mfma();
+  const int group = n_q / n_kv;
+  // Tiles of 16 rows, the keys split when the tiles alone would leave most of the chip idle
+  // (decoding); wider tiles, whose rows share every key fragment a wavefront loads, when
+  // there are plenty (prompts).
+  const int span = window ? std::min(max_kv_len, window + max_q_len) : max_kv_len;
+  const int blocks = std::max(1, (span + 31) / 32);
+  int rows = 16;
+  long long total_rows = 0;
+  for (int c : counts) total_rows += c;
+  total_rows *= group;
+  // 64-row tiles exist but run at one wavefront per SIMD; 32 rows measured fastest
+  const int max_rows = std::min(32, t.mk_attention_mfma_max_rows(head_dim));
+  while (rows < max_rows && (total_rows / (rows * 2)) * n_kv >= kAttentionWideTileWaves) rows *= 2;
+  if (tile_rows > 0) rows = tile_rows;
+  int staged = staged_in;
+  const bool split_forced = splits_in > 0;
+  if (staged < 0) {
+    // prompts: plenty of rows per sequence, enough workgroups of 64 of them; 16 rows a
+    // wavefront measured faster than 32 there
+    const bool yes = !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 64 &&
+                     (total_rows / 64) * n_kv >= kAttentionStagedWorkgroups &&
+                     t.mk_attention_mfma_staged(head_dim, 16) != 0;
+    staged = yes ? -1 : 0;
+    if (yes) rows = 16;
+  }
+  plan.rows = rows;
+  plan.tile_rows = staged ? rows * 4 : rows;
+  plan.num_tiles = count_tiles(counts, group, plan.tile_rows);
+  if (staged == -1) {
+    // A workgroup's chain of key blocks is cut into 2 or 4 chains side by side while that
+    // leaves the chip short of wavefronts and every chain a few blocks (measured at 2,048
+    // tokens, 14 heads of 64: 45, 35, 32 us with 1, 2, 4 groups; at 8,192: 264, 349, 284;
+    // 28 heads of 128 at 2,048: 100, 91 with 1, 2; at 8,192: 878, 1055).
+    staged = t.mk_attention_mfma_staged(head_dim, 16);
+    while (staged > 1 && ((long long)plan.num_tiles * n_kv * 4 * staged > kAttentionStagedMaxWaves ||
+                          blocks < 4 * staged)) {
+      staged /= 2;
+    }
+  }
+  plan.staged = staged;
+  const long long waves = std::max<long long>(1, (long long)plan.num_tiles * n_kv);
+  if (!staged && waves < kAttentionTargetWaves) {
+    // decoding, and short prompt portions over a long prefix (16 tokens over 2,032: 47 us as
+    // one chain of key blocks per wavefront, 23 split): every tile's own range of keys in
+    // equal parts
+    const int by_blocks = std::max(1, blocks / kAttentionMinBlocksPerSplit);
+    const int by_waves = (int)((kAttentionTargetWaves + waves - 1) / waves);
+    plan.splits = std::max(1, std::min({by_blocks, by_waves, kAttentionMaxSplits}));
+  }
+  if (split_forced) {
+    plan.splits = splits_in;
+    plan.split_blocks = split_blocks_in;
+  }
+  return plan;
+}
+
+}  // namespace mercury

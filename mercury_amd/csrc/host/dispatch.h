@@ -1,0 +1,74 @@
+// Which kernel runs an operation of a given shape.  These decisions are pure functions of
+// sizes and element types; the Python faces of the kernels (kernels/ops.py) and the step
+// programs (program.cc) both ask here, so that what the tests exercise kernel by kernel is
+// what a step launches.
+#pragma once
+
+#include <cstdint>
+#include <vector>
+
+namespace mercury {
+
+constexpr int kF32 = 0, kBF16 = 1;
+
+inline int element_size(int dtype) { return dtype == kBF16 ? 2 : 4; }
+
+// ---- projections
+
+// bfloat16 operands with K a multiple of 8 and at least one row: what the matrix-core
+// projections take.
+bool mfma_eligible(int x_dtype, int w_dtype, int m, int k);
+
+// Whether x W^T is best computed as float32 partial sums over slices of K that the consumer
+// (a norm, or the rotation and cache write) adds up: few enough rows over a matrix large
+// enough for bandwidth to matter that whole-K workgroups would leave compute units idle.
+bool wants_partials(int x_dtype, int w_dtype, int m, int n, int k);
+
+struct PartialsPlan {
+  bool skinny = false;     // weights straight from HBM into the matrix cores (few rows)
+  int slices = 1;
+};
+PartialsPlan plan_partials(int m, int n, int k);
+
+enum class LinearKind { GENERIC = 0, SKINNY = 1, SKINNY_ACC = 2, TILED = 3 };
+// force: 0 auto, 1 the float32-arithmetic kernel, 2 the matrix-core kernels.
+LinearKind choose_linear(int x_dtype, int m, int n, int k, bool has_bias, bool accumulate,
+                         int out_dtype, int force = 0);
+
+// The gated projection act = silu(x Wg^T) * (x Wu^T) as one matrix-core kernel.
+bool fuses_gating(int x_dtype, int w_dtype, int m, int k, int rows_of_w);
+bool gated_is_skinny(int m);
+
+enum class QkvKind { SKINNY = 0, TILED = 1, PARTIALS_FINISH = 2, LINEAR_ROPE = 3 };
+// SKINNY / TILED: projection, bias, rotation and cache write in one kernel.  PARTIALS_FINISH:
+// K-split partial sums, then a small kernel that adds them up, rotates and writes.
+// LINEAR_ROPE: the projection (whole), then the rotation and cache-write kernel.
+QkvKind choose_qkv(int x_dtype, int w_dtype, int m, int width, int k, int head_dim,
+                   int rotary_dim, int page_size, bool half_layout);
+bool qkv_fusable(int x_dtype, int w_dtype, int m, int k, int head_dim, int rotary_dim,
+                 int page_size, bool half_layout);
+
+// ---- attention
+
+struct AttentionPlan {
+  bool mfma = false;
+  int rows = 16;          // rows per wavefront tile
+  int staged = 0;         // 0, or how many groups of four wavefronts share a workgroup's keys
+  int splits = 1;
+  int split_blocks = 0;
+  int tile_rows = 16;     // rows per entry of the tile list: rows, or 4 * rows when staged
+  int num_tiles = 0;
+};
+
+// counts: tokens per sequence this step.  overrides < 0 (or 0 for splits) leave the choice
+// to the step's size.
+AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, int n_kv, int window,
+                             const std::vector<int>& counts, int max_q_len, int max_kv_len,
+                             int force = 0, int tile_rows = -1, int staged = -1,
+                             int splits = 0, int split_blocks = 0);
+int count_tiles(const std::vector<int>& counts, int group, int tile_rows);
+// tile_seq and tile_row0, `num_tiles` entries each, appended to `out`.
+void build_tiles(const std::vector<int>& counts, int group, int tile_rows, std::vector<int>& seq,
+                 std::vector<int>& row0);
+
+}  // namespace mercury

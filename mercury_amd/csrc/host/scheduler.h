@@ -121,6 +121,7 @@ class Scheduler {
             SchedulerOptions options);
 
   const SchedulerOptions& options() const { return options_; }
+  SchedulerOptions& mutable_options() { return options_; }
   const std::vector<RequestPtr>& waiting() const { return waiting_; }
   const std::vector<RequestPtr>& running() const { return running_; }
   const Stats& stats() const { return stats_; }

@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 9
+#define MK_ABI_VERSION 10
 
 #ifdef __cplusplus
 extern "C" {
@@ -32,12 +32,13 @@ int mk_silu_mul(const void* gate_up, void* out, int dtype, int tokens, int inter
 
 // Rotary encoding of the q and k heads of qkv [T, row_stride] (q in place) and the write of
 // rotated k into the paged key cache [pages, n_kv, page_size, d] and of raw v into the value
-// cache, which is transposed within a page: [pages, n_kv, d, page_size].
+// cache, which is transposed within a page: [pages, n_kv, d, page_size].  The first `rot`
+// dims of a head turn, pair j being dims (j, j + rot/2), or (2j, 2j + 1) when `interleaved`.
 int mk_rope_kv_write(void* qkv, int dtype, int row_stride, const float* cos_table,
                      const float* sin_table, int table_positions, const int* positions,
                      const int* token_seq, const int* block_table, int table_stride,
                      void* k_cache, void* v_cache, int page_size, int n_q, int n_kv, int d,
-                     int rot, int write_kv, int tokens, hipStream_t stream);
+                     int rot, int interleaved, int write_kv, int tokens, hipStream_t stream);
 
 // y = x W^T (+ bias) with float32 FMA.  accumulate: y (float32) += instead of =.
 int mk_linear_generic(const void* x, const void* w, int dtype, const void* bias, int bias_dtype,

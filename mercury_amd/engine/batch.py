@@ -133,7 +133,7 @@ def pack_step(chunks: list, manager, vocab_size: int, max_positions: int, pinned
             # The final norm folds the last projection's partial sums into a wanted row of the
             # residual stream; a row named twice would receive them twice.
             raise BatchError(f"sequence {c.key!r} wants the same place twice: {sorted(c.want)}")
-    slots = [manager.requests[c.key].state_slot for c in chunks]
+    slots = [manager.sequence(c.key).state_slot for c in chunks]
 
     needed = max(-(-int(kv) // ps) for kv in kv_len)
     width = needed if table_width is None else table_width

@@ -1,10 +1,15 @@
-"""The engine loop: take commands, schedule, execute, route tokens, finish and free
-(reference: mercury/engine.py:28-300).
+"""The engine: the public entry point around the host core's loop.
 
-One thread owns everything that touches the cache.  Clients talk to it through `submit` and
-`abort` (a queue) and hear back through a per-request `sink` callable that receives
-:class:`StreamEvent` objects; `generate` wraps that into a blocking call that returns token
-lists.
+The host core (C++) keeps the requests, the scheduler, the cache bookkeeping and the step log;
+it decides, and reports what happened as a list of events.  This class owns what is Python's
+to own: the command queue through which other threads talk to the engine thread, the optional
+engine thread itself, the per-request sinks the events are delivered to, and the executor that
+runs a plan on the GPU (reference for the API and its meanings: mercury/engine.py:28-300).
+
+    engine = Engine(EngineConfig(model=folder))
+    engine.submit(rid, prompt_ids, max_tokens, sink)      # from any thread
+    engine.step()                                         # or engine.start() for a thread
+    tokens = engine.generate([[1, 2, 3]], SamplingParams(), max_tokens=16)   # blocking
 """
 
 from __future__ import annotations
@@ -12,31 +17,14 @@ from __future__ import annotations
 import queue
 import threading
 import time
-from dataclasses import dataclass
 from typing import Callable
 
-from ..cache.hashing import PageHasher
-from ..cache.manager import CacheManager
+from ..cache import CacheManager, PageHasher
 from ..config.engine_config import EngineConfig
-from .metrics import EngineMetrics, StepRecord
-from .request import Request, RequestState, SamplingParams
-from .scheduler import Scheduler
+from ..hostcore import core as _core
 
-
-@dataclass(slots=True)
-class StreamEvent:
-    """kind: "token" (token, index), "done" (finish_reason: "length" | "stop" | "abort"),
-    "preempted", or "error" (message)."""
-
-    rid: str
-    kind: str
-    token: int | None = None
-    index: int = 0
-    finish_reason: str | None = None
-    message: str | None = None
-    t: float = 0.0
-
-
+StreamEvent = _core.StreamEvent
+SamplingParams = _core.SamplingParams
 Sink = Callable[[StreamEvent], None]
 
 
@@ -55,27 +43,33 @@ def autosize_blocks(cfg: EngineConfig, kv_bytes_per_token: int, device) -> int:
 
 
 class Engine:
-    """`Engine(cfg)` loads the model folder `cfg.model` onto the GPU.  Tests pass `executor`
-    (anything with `execute(plan)`) and, with it, the cache manager it checks against."""
+    """`Engine(cfg)` loads the model folder `cfg.model` onto the GPU, or, with
+    `cfg.random_weights`, builds the model that `model_config` (a ``config.json`` as a dict) or
+    the ``config.json`` at `cfg.model` describes and draws its weights from `cfg.weight_seed`.
+    Tests pass `executor` (anything with `execute(plan)`) and, with it, the cache manager it
+    checks against."""
 
     def __init__(self, cfg: EngineConfig, executor=None, manager: CacheManager | None = None,
-                 clock: Callable[[], float] = time.perf_counter, eos_token_ids=None):
+                 clock: Callable[[], float] = time.perf_counter, eos_token_ids=None,
+                 model_config: dict | None = None):
         self.cfg = cfg
         self.clock = clock
         self.hasher = PageHasher(cfg.block_size, cfg.cryptographic_hashes)
         if executor is None:
-            executor, manager, eos = self._load(cfg)
+            executor, manager, eos = self._load(cfg, model_config)
             eos_token_ids = eos if eos_token_ids is None else eos_token_ids
         elif manager is None:
             raise ValueError("an engine with its own executor needs the cache manager it uses")
         self.executor, self.manager = executor, manager
         self.runner = executor  # the reference's name for this seam
-        self.eos_ids = set(eos_token_ids or ())
-        self.sched = Scheduler(
+        self.core = _core.EngineCore(
             manager, self.hasher, policy=cfg.policy, max_running=cfg.max_running,
             prefill_budget=cfg.prefill_budget, aging_tokens_per_s=cfg.aging_tokens_per_s,
-            max_wait_s=cfg.max_wait_s, scan_limit=cfg.scan_limit)
-        self.metrics = EngineMetrics(max_steps=cfg.max_step_records)
+            max_wait_s=cfg.max_wait_s, scan_limit=cfg.scan_limit,
+            max_model_len=cfg.max_model_len, eos_ids=sorted(eos_token_ids or ()),
+            max_step_records=cfg.max_step_records)
+        self.sched = self.core.scheduler
+        self.metrics = self.core      # counters, summary(), step_records()
         self._commands: queue.Queue = queue.Queue()
         self._sinks: dict = {}
         self._wake, self._stop = threading.Event(), threading.Event()
@@ -83,25 +77,46 @@ class Engine:
         self._lock = threading.Lock()
         self._submitted = 0
 
+    @property
+    def eos_ids(self) -> set:
+        """Token ids that end a request (unless it asked to ignore them)."""
+        return set(self.core.eos_ids)
+
+    @eos_ids.setter
+    def eos_ids(self, ids) -> None:
+        self.core.eos_ids = sorted(ids)
+
     @staticmethod
-    def _load(cfg: EngineConfig):
+    def _load(cfg: EngineConfig, model_config: dict | None):
+        import torch
+
+        from ..config.model_config import read_config_json
+        from ..config.registry import build_model
         from ..sampling.sampler import Sampler
-        from ..weights.loader import load_model_folder
+        from ..weights.loader import load_model_folder, load_weights
+        from ..weights.random_init import RandomSource
         from .executor import GpuExecutor
         from .runner import ModelRunner, require_gpu
 
-        import torch
-
         device = torch.device(cfg.device)
         require_gpu(device)
-        model = load_model_folder(cfg.model, cfg.torch_dtype, device)
+        if cfg.random_weights:
+            model = build_model(model_config if model_config is not None
+                                else read_config_json(cfg.model))
+            from ..config.engine_config import _DTYPE_BY_NAME
+
+            stored = _DTYPE_BY_NAME[cfg.weight_dtype]
+            load_weights(model, RandomSource(model, cfg.weight_seed, cfg.weight_std, stored, device),
+                         cfg.torch_dtype, device)
+        elif model_config is not None:
+            raise ValueError("model_config is only for random_weights; a model folder brings its own")
+        else:
+            model = load_model_folder(cfg.model, cfg.torch_dtype, device)
         if model.max_positions:
             cfg.validate_against(model.max_positions)
         has_state = any(layer.mixer.state_spec() is not None for layer in model.layers)
         if cfg.num_blocks < 0:
-            elem = torch.empty((), dtype=cfg.torch_dtype).element_size()
-            per_token = sum(2 * s.kv_heads * s.head_dim * elem for s in model.cache_slots.values())
-            cfg.num_blocks = autosize_blocks(cfg, per_token, device)
+            cfg.num_blocks = autosize_blocks(cfg, model.kv_bytes_per_token(cfg.torch_dtype), device)
             cfg.validate_against(model.max_positions or cfg.max_model_len)
         manager = CacheManager(model.cache_slots, cfg.num_blocks, cfg.block_size, cfg.max_running,
                                has_state)
@@ -113,10 +128,10 @@ class Engine:
     # ---------------------------------------------------------------- lifecycle
 
     def start(self) -> None:
+        """Run the loop on a thread of its own until `shutdown`."""
         if self._thread is not None:
             return
-        self.metrics.started_at = self.clock()
-        self._thread = threading.Thread(target=self._run, name="mercury-engine", daemon=True)
+        self._thread = threading.Thread(target=self._run, name="mercury-amd-engine", daemon=True)
         self._thread.start()
 
     def shutdown(self, timeout: float = 5.0) -> None:
@@ -137,32 +152,24 @@ class Engine:
     def submit(self, rid: str, prompt_ids: list, max_tokens: int, sink: Sink,
                params: SamplingParams | None = None, session_id: str | None = None,
                arrival: float | None = None) -> None:
-        params = params or SamplingParams()
+        """Queue a request.  A request that can never run (an empty prompt, more tokens than
+        one request may hold) is answered at once with an "error" event and not queued."""
         arrival = self.clock() if arrival is None else arrival
-        ceiling = min(self.cfg.max_model_len, self.manager.capacity_tokens())
-        if not prompt_ids:
-            self._reject(rid, sink, "prompt must contain at least one token")
+        why = self.core.refusal(len(prompt_ids), max_tokens)
+        if why is not None:
+            self.core.count_rejected()
+            sink(StreamEvent(rid=rid, kind="error", message=why, t=self.clock()))
             return
-        if len(prompt_ids) + max_tokens > ceiling:
-            self._reject(rid, sink,
-                         f"prompt ({len(prompt_ids)}) + max_tokens ({max_tokens}) exceeds the "
-                         f"{ceiling}-token ceiling of this engine")
-            return
-        r = Request(rid=rid, prompt=list(prompt_ids), max_tokens=max_tokens, arrival=arrival,
-                    hashes=self.hasher.hashes(prompt_ids), params=params, session_id=session_id)
+        request = self.core.make_request(rid, prompt_ids, max_tokens, arrival, params, session_id)
         with self._lock:
             self._sinks[rid] = sink
             self._submitted += 1
-        self._commands.put(("add", r))
+        self._commands.put(("add", request))
         self._wake.set()
 
     def abort(self, rid: str) -> None:
         self._commands.put(("abort", rid))
         self._wake.set()
-
-    def _reject(self, rid: str, sink: Sink, message: str) -> None:
-        self.metrics.counters["rejected_requests"] += 1
-        sink(StreamEvent(rid=rid, kind="error", message=message, t=self.clock()))
 
     def generate(self, prompts: list, params=None, max_tokens: int = 16) -> list:
         """Blocking: run every prompt (a list of token ids each) to completion and return the
@@ -185,7 +192,8 @@ class Engine:
             return sink
 
         for i, prompt in enumerate(prompts):
-            self.submit(f"gen-{base + i}", prompt, budgets[i], sink_for(i), params=params[i])
+            self.submit(f"gen-{base + i}", prompt, budgets[i], sink_for(i),
+                        params=params[i])
         if errors:
             raise ValueError("; ".join(f"prompt {i}: {m}" for i, m in sorted(errors.items())))
         self._drain_commands()
@@ -196,32 +204,23 @@ class Engine:
     # ---------------------------------------------------------------- the loop
 
     def step(self):
-        t_start = time.perf_counter()
+        """One pass: take commands, plan, run the plan, apply its results.  Returns the step's
+        record, or None when there was nothing to run."""
+        started = time.perf_counter()
         self._drain_commands()
-        plan = self.sched.schedule(self.clock())
-        for r in plan.preempted:
-            self._emit(r, StreamEvent(rid=r.rid, kind="preempted", t=self.clock()))
+        plan, events = self.core.schedule(self.clock())
+        self._deliver(events)
         if not plan:
-            self.metrics.counters["idle_steps"] += 1
+            self.core.count_idle()
             return None
-
         result = self.executor.execute(plan)
         now = self.clock()
-        for work, token in zip(plan.work, result.tokens):
-            self._advance(work, token, now)
-
+        self._deliver(self.core.advance(plan, result.tokens, now))
         if self.cfg.debug_invariants:
             self.manager.check_invariants()
-
-        record = StepRecord(
-            t=now, num_prefill=len(plan.prefill), num_decode=len(plan.decode),
-            prefill_tokens=plan.num_prefill_tokens, sched_s=plan.sched_seconds,
-            prepare_s=result.prepare_seconds, forward_s=result.forward_seconds,
-            step_s=time.perf_counter() - t_start, waiting=len(self.sched.waiting),
-            running=len(self.sched.running), free_blocks=self.manager.num_available(),
-            preempted=len(plan.preempted))
-        self.metrics.add_step(record)
-        return record
+        return self.core.log_step(plan, now, result.prepare_seconds, result.forward_seconds,
+                                  getattr(result, "device_seconds", 0.0),
+                                  time.perf_counter() - started)
 
     def _drain_commands(self) -> None:
         while True:
@@ -230,60 +229,25 @@ class Engine:
             except queue.Empty:
                 return
             if kind == "add":
-                self.sched.add(payload)
+                self.core.add(payload)
                 continue
-            r = self.sched.abort(payload)
-            if r is None:
+            events = self.core.abort(payload, self.clock())
+            if not events:
                 with self._lock:
-                    self._sinks.pop(payload, None)
+                    self._sinks.pop(payload, None)    # already finished, or never queued
+            self._deliver(events)
+
+    def _deliver(self, events: list) -> None:
+        for event in events:
+            closing = event.kind == "done"
+            with self._lock:
+                sink = self._sinks.pop(event.rid, None) if closing else self._sinks.get(event.rid)
+            if sink is None:
                 continue
-            self.metrics.counters["aborted_requests"] += 1
-            r.finished_at = self.clock()
-            self.metrics.add_finished(r.record())
-            self._emit(r, StreamEvent(rid=r.rid, kind="done", finish_reason="abort",
-                                      t=r.finished_at), close=True)
-
-    def _advance(self, work, token, now: float) -> None:
-        """The step wrote keys and values for the work's tokens: note it, offer the pages that
-        became full to the prefix cache, give back what a window passed, and, when the work
-        completed the sequence, take the sampled token."""
-        r = work.request
-        r.num_computed = work.start + work.count
-        full = r.num_computed // self.cfg.block_size
-        if self.manager.prefix_sharing and full > len(r.hashes):
-            self.hasher.extend(r.hashes, r.tokens[:r.num_computed])
-        self.manager.commit(r.rid, r.hashes, full)
-        self.manager.trim(r.rid, r.num_computed)
-        if token is None:
-            return
-        index = len(r.out)
-        r.append(int(token))
-        if r.first_token_at is None:
-            r.first_token_at = now
-        self._emit(r, StreamEvent(rid=r.rid, kind="token", token=int(token), index=index, t=now))
-        if len(r.out) >= r.max_tokens:
-            self._finish(r, "length", now)
-        elif not r.params.ignore_eos and int(token) in self.eos_ids:
-            self._finish(r, "stop", now)
-
-    def _finish(self, r: Request, reason: str, now: float) -> None:
-        r.state = RequestState.FINISHED
-        r.finish_reason = reason
-        r.finished_at = now
-        self.sched.drop(r)
-        self.metrics.counters["finished_requests"] += 1
-        self.metrics.add_finished(r.record())
-        self._emit(r, StreamEvent(rid=r.rid, kind="done", finish_reason=reason, t=now), close=True)
-
-    def _emit(self, r: Request, event: StreamEvent, close: bool = False) -> None:
-        with self._lock:
-            sink = self._sinks.pop(r.rid, None) if close else self._sinks.get(r.rid)
-        if sink is None:
-            return
-        try:
-            sink(event)
-        except Exception:
-            self.abort(r.rid)  # a sink that raises means nobody is listening any more
+            try:
+                sink(event)
+            except Exception:
+                self.abort(event.rid)   # a sink that raises means nobody is listening any more
 
     # ---------------------------------------------------------------- reporting
 
@@ -299,7 +263,7 @@ class Engine:
             },
             "allocator": self.manager.snapshot(),
             "scheduler": self.sched.snapshot(),
-            "engine": self.metrics.summary(),
+            "engine": self.core.summary(),
             "submitted": self._submitted,
         }
 
@@ -307,4 +271,4 @@ class Engine:
         return self.manager.leaked_pages()
 
     def drain_request_records(self) -> list:
-        return self.metrics.drain_finished()
+        return self.core.drain_finished()

@@ -91,7 +91,7 @@ class GpuExecutor:
         self.kv_bytes = runner.kv_bytes
         manager = runner.manager
         self.lookahead = (bool(lookahead) and runner.use_graphs and not runner.states
-                          and all(g.spec.window is None for g in manager.groups))
+                          and all(g.window is None for g in manager.groups))
         self._ahead: _Ahead | None = None
         self._ring = _PinnedRing(max(256, runner.max_graph_batch))
         self.stats = {"ahead_started": 0, "ahead_used": 0}
@@ -107,7 +107,8 @@ class GpuExecutor:
         else:
             chunks = []
             for w in work:
-                tokens = w.request.tokens[w.start:w.start + w.count]
+                tokens = (w.request.tokens[w.start:w.start + w.count] if w.count > 1
+                          else [w.request.token_at(w.start)])
                 chunks.append(SeqChunk(w.request.rid, tokens, w.start,
                                        [w.count - 1] if w.emits else []))
             logits = self.runner.step(chunks)
@@ -135,7 +136,7 @@ class GpuExecutor:
         for w, rid, start, token in zip(work, ahead.rids, ahead.starts, ahead.fed):
             r = w.request
             if (r.rid != rid or w.start != start or w.count != 1 or not w.emits
-                    or r.tokens[start] != token):
+                    or r.token_at(start) != token):
                 return False
         return True
 

@@ -41,7 +41,7 @@ class ReplaySession:
                  page_size: int = DEFAULT_PAGE_SIZE, max_live: int = DEFAULT_MAX_LIVE):
         import torch
 
-        from ..cache.manager import CacheManager
+        from ..cache import CacheManager
         from ..config.engine_config import _DTYPE_BY_NAME
         from ..weights.loader import load_model_folder
         from .runner import ModelRunner

@@ -49,7 +49,7 @@ class DecodeGraph:
         self.copied = None                                 # the last copy of `host` to the device
         self.row_record = [None] * n                       # whose pages a table row mirrors
         self.row_pages = [[0] * n for _ in packed.widths]  # and how many of them
-        self.appendable = [g.spec.window is None for g in runner.manager.groups]
+        self.appendable = [g.window is None for g in runner.manager.groups]
         # Once outside the capture: loads libraries, fills the context's tile tables.
         side = torch.cuda.Stream(device=runner.device)
         side.wait_stream(torch.cuda.current_stream(runner.device))
@@ -77,14 +77,14 @@ class DecodeGraph:
             raise BatchError(f"a sequence would pass the limit of {max_positions} tokens")
         np.add(self.positions, 1, out=self.kv_len)
         ps = manager.page_size
-        requests = manager.requests
         for s in range(n):
             c = chunks[s]
-            record = requests[c.key]
+            record = manager.sequence(c.key)
             need = c.start // ps + 1
-            same = record is self.row_record[s]
+            # a key stands for one admission: its state slot and pages change only by growing
+            same = (c.key, record.state_slot) == self.row_record[s]
             if not same:
-                self.row_record[s] = record
+                self.row_record[s] = (c.key, record.state_slot)
                 self.slots[s] = record.state_slot
             for g, table in enumerate(self.tables):
                 have = self.row_pages[g][s]
@@ -142,17 +142,17 @@ class ModelRunner:
         # page] per cache slot.
         self.kv = {}
         for slot, spec in model.cache_slots.items():
-            group = manager.group_of_slot[slot]
-            pages = manager.groups[group].pool.num_pages
+            pages = manager.groups[manager.group_of(slot)].pool.num_pages
+            kv_dtype = spec.dtype or dtype
             self.kv[slot] = (
-                torch.zeros((pages, spec.kv_heads, self.page_size, spec.head_dim), dtype=dtype, device=device),
-                torch.zeros((pages, spec.kv_heads, spec.head_dim, self.page_size), dtype=dtype, device=device))
+                torch.zeros((pages, spec.kv_heads, self.page_size, spec.head_dim), dtype=kv_dtype, device=device),
+                torch.zeros((pages, spec.kv_heads, spec.v_dim, self.page_size), dtype=kv_dtype, device=device))
         self.caches = {}
         for n, call in enumerate(model.calls):
             if call.cache is None:
                 continue
             k, v = self.kv[call.cache]
-            self.caches[n] = LayerCache(k, v, manager.group_of_slot[call.cache], self.page_size,
+            self.caches[n] = LayerCache(k, v, manager.group_of(call.cache), self.page_size,
                                         call.writes)
         # Per-request state of fixed size, one tensor per layer that declares it.
         self.states = {}
@@ -167,7 +167,8 @@ class ModelRunner:
         return sum(t.numel() * t.element_size() for kv in self.kv.values() for t in kv)
 
     def kv_bytes_per_token(self) -> int:
-        return sum(2 * k.shape[1] * k.shape[3] * k.element_size() for k, _ in self.kv.values())
+        return sum(k.shape[1] * (k.shape[3] + v.shape[2]) * k.element_size()
+                   for k, v in self.kv.values())
 
     def build(self, chunks: list) -> StepContext:
         return build_step(chunks, self.manager, self.model.vocab_size, self.max_model_len,

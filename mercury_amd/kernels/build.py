@@ -56,6 +56,15 @@ HIPCC_FLAGS = [
 ]
 
 
+# The host core: C++ (pybind11) for the cache manager, the scheduler, step packing and the
+# launch sequence of a step.  Compiled with the host compiler; it reaches the kernel libraries
+# through dlopen, so it links against the HIP runtime only.
+HOST_NAME = "host"
+HOST_DIR = CSRC / "host"
+HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off", "-pthread",
+              "-D__HIP_PLATFORM_AMD__", "-Wall", "-Wno-unused-function"]
+
+
 class BuildError(RuntimeError):
     pass
 
@@ -89,17 +98,25 @@ def library_dirs() -> list:
 
 
 def library_name(name: str) -> str:
-    return f"libmercury_{name}.so"
+    return "mercury_host.so" if name == HOST_NAME else f"libmercury_{name}.so"
 
 
 def _sources(name: str) -> list:
+    if name == HOST_NAME:
+        return sorted(HOST_DIR.glob("*.cc"))
     return [CSRC / s for s in LIBRARIES[name]]
 
 
 def source_hash(name: str) -> str:
     digest = hashlib.sha256()
-    digest.update(" ".join(HIPCC_FLAGS).encode())
-    for path in _sources(name) + sorted(CSRC.glob("*.h")):
+    headers = sorted(CSRC.glob("*.h"))
+    if name == HOST_NAME:
+        digest.update(" ".join(HOST_FLAGS).encode())
+        digest.update(sys.version.encode())
+        headers += sorted(HOST_DIR.glob("*.h"))
+    else:
+        digest.update(" ".join(HIPCC_FLAGS).encode())
+    for path in _sources(name) + headers:
         digest.update(path.name.encode())
         digest.update(path.read_bytes())
     return digest.hexdigest()
@@ -146,9 +163,38 @@ def _run_with_heartbeat(cmd: list, what: str) -> None:
         raise BuildError(f"compiling {what} failed:\n{' '.join(cmd)}\n{output}")
 
 
+def _host_compiler() -> str:
+    for candidate in (os.environ.get("CXX"), shutil.which("g++"), shutil.which("c++")):
+        if candidate and Path(candidate).exists():
+            return candidate
+    raise BuildError("no C++ compiler was found for the host core (looked at $CXX, g++, c++)")
+
+
+def _rocm_root() -> Path:
+    for candidate in (os.environ.get("ROCM_PATH"), "/opt/rocm"):
+        if candidate and (Path(candidate) / "include" / "hip").is_dir():
+            return Path(candidate)
+    raise BuildError("the ROCm headers were not found (looked at $ROCM_PATH and /opt/rocm)")
+
+
+def _host_commands(sources: list, objects: list, target: Path) -> tuple:
+    import sysconfig
+
+    import pybind11
+
+    cxx, rocm = _host_compiler(), _rocm_root()
+    includes = ["-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"],
+                "-I", str(rocm / "include"), "-I", str(CSRC), "-I", str(HOST_DIR)]
+    compiles = [[cxx, *HOST_FLAGS, *includes, "-c", str(src), "-o", str(obj)]
+                for src, obj in zip(sources, objects)]
+    link = [cxx, "-shared", "-pthread", "-o", str(target), *map(str, objects),
+            "-L", str(rocm / "lib"), f"-Wl,-rpath,{rocm / 'lib'}", "-lamdhip64", "-ldl"]
+    return compiles, link
+
+
 def build_library(name: str, force: bool = False, verbose: bool = True) -> Path:
-    """Compile one library and return its path."""
-    if name not in LIBRARIES:
+    """Compile one library (a kernel library, or the host core "host") and return its path."""
+    if name != HOST_NAME and name not in LIBRARIES:
         raise BuildError(f"unknown kernel library {name!r}; known: {sorted(LIBRARIES)}")
     if not force:
         found = find_library(name)
@@ -157,21 +203,37 @@ def build_library(name: str, force: bool = False, verbose: bool = True) -> Path:
     out_dir = next((d for d in library_dirs() if _writable(d)), None)
     if out_dir is None:
         raise BuildError("no writable folder for the kernel library")
-    hipcc = _hipcc()
     obj_dir = out_dir / "obj"
     obj_dir.mkdir(parents=True, exist_ok=True)
     sources = _sources(name)
-    if verbose:
-        _say(f"compiling kernel library '{name}' for {ARCH}: {len(sources)} sources -> {out_dir}")
-    objects, threads, errors = [], [], []
-    for src in sources:
-        obj = obj_dir / f"{name}-{src.stem}.o"
-        objects.append(obj)
-        cmd = [hipcc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+    objects = [obj_dir / f"{name}-{src.stem}.o" for src in sources]
+    target = out_dir / library_name(name)
+    partial = out_dir / (library_name(name) + f".{os.getpid()}.tmp")
+    if name == HOST_NAME:
+        if verbose:
+            _say(f"compiling the host core: {len(sources)} sources -> {out_dir}")
+        compiles, link = _host_commands(sources, objects, partial)
+    else:
+        hipcc = _hipcc()
+        if verbose:
+            _say(f"compiling kernel library '{name}' for {ARCH}: {len(sources)} sources -> {out_dir}")
+        compiles = [[hipcc, *HIPCC_FLAGS, "-I", str(CSRC), "-c", str(src), "-o", str(obj)]
+                    for src, obj in zip(sources, objects)]
+        link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", "-o",
+                str(partial), *map(str, objects)]
+    threads, errors = [], []
+    headers = b"".join(p.read_bytes() for p in sorted(CSRC.glob("*.h")) + sorted(HOST_DIR.glob("*.h")))
+    for src, obj, cmd in zip(sources, objects, compiles):
+        # An object whose command, source and headers are what they were is kept.
+        wanted = hashlib.sha256(" ".join(cmd).encode() + src.read_bytes() + headers).hexdigest()
+        mark = obj.with_suffix(".o.stamp")
+        if obj.is_file() and mark.is_file() and mark.read_text().strip() == wanted:
+            continue
 
-        def work(cmd=cmd, src=src):
+        def work(cmd=cmd, src=src, mark=mark, wanted=wanted):
             try:
                 _run_with_heartbeat(cmd, src.name)
+                mark.write_text(wanted + "\n")
                 if verbose:
                     _say(f"compiled {src.name}")
             except BuildError as e:  # collected and raised on the calling thread
@@ -184,11 +246,7 @@ def build_library(name: str, force: bool = False, verbose: bool = True) -> Path:
         thread.join()
     if errors:
         raise errors[0]
-    target = out_dir / library_name(name)
-    partial = out_dir / (library_name(name) + f".{os.getpid()}.tmp")
-    cmd = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", "-o",
-           str(partial), *map(str, objects)]
-    _run_with_heartbeat(cmd, library_name(name))
+    _run_with_heartbeat(link, library_name(name))
     os.replace(partial, target)
     _stamp(target).write_text(source_hash(name) + "\n")
     if verbose:
@@ -197,7 +255,8 @@ def build_library(name: str, force: bool = False, verbose: bool = True) -> Path:
 
 
 def build_all(force: bool = True, verbose: bool = True) -> dict:
-    return {name: build_library(name, force=force, verbose=verbose) for name in LIBRARIES}
+    return {name: build_library(name, force=force, verbose=verbose)
+            for name in [*LIBRARIES, HOST_NAME]}
 
 
 if __name__ == "__main__":

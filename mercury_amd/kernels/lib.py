@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 from . import build
 
-ABI_VERSION = 9
+ABI_VERSION = 10
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -21,7 +21,7 @@ _SIGNATURES = {
         "mk_embed": [P, P, I, P, I, I, I, P],
         "mk_rmsnorm": [P, P, I, L, P, I, F, P, P, I, I, I, P],
         "mk_silu_mul": [P, P, I, I, I, P],
-        "mk_rope_kv_write": [P, I, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
+        "mk_rope_kv_write": [P, I, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, P],
         "mk_linear_generic": [P, P, I, P, I, P, I, I, I, I, I, I, I, P],
         "mk_attention_generic": [P, I, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
         "mk_qkv_finish": [P, I, L, P, I, P, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],

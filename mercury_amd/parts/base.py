@@ -59,12 +59,25 @@ class TensorSpec:
 
 @dataclass(frozen=True)
 class CacheSpec:
-    """Per-token cache need of a mixer: keys and values of `kv_heads` heads of `head_dim`,
-    all earlier tokens (`window` None) or the last `window` of them."""
+    """Per-token cache need of a mixer: keys of `kv_heads` heads of `head_dim` and values of as
+    many heads of `value_dim` (default: the keys' width), stored as `dtype` (default: the
+    model's compute dtype); all earlier tokens (`window` None) or the last `window` of them."""
 
     kv_heads: int
     head_dim: int
     window: int | None = None
+    value_dim: int | None = None
+    dtype: torch.dtype | None = None
+
+    @property
+    def v_dim(self) -> int:
+        return self.head_dim if self.value_dim is None else self.value_dim
+
+    def as_tuple(self) -> tuple:
+        """(kv_heads, key width, value width, dtype code or -1, window or 0): what the cache
+        manager groups slots by."""
+        code = -1 if self.dtype is None else {torch.float32: 0, torch.bfloat16: 1}[self.dtype]
+        return (self.kv_heads, self.head_dim, self.v_dim, code, self.window or 0)
 
 
 @dataclass(frozen=True)

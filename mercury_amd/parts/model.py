@@ -75,7 +75,7 @@ class DecoderModel(Part):
                 writers[call.cache] = spec
             elif call.cache not in writers:
                 raise ValueError(f"entry {n} reads cache slot {call.cache} before it is written")
-            elif (writers[call.cache].kv_heads, writers[call.cache].head_dim) != (spec.kv_heads, spec.head_dim):
+            elif writers[call.cache].as_tuple()[:4] != spec.as_tuple()[:4]:
                 raise ValueError(f"entry {n} reads cache slot {call.cache} of another shape")
         self.cache_slots = writers  # slot -> CacheSpec
 
@@ -113,6 +113,15 @@ class DecoderModel(Part):
     def prepare(self, max_positions: int, device) -> None:
         for layer in self.layers:
             layer.prepare(max_positions, device)
+
+    def kv_bytes_per_token(self, dtype: torch.dtype) -> int:
+        """Bytes of keys and values one token adds to the cache, over all cache slots
+        (reference: mercury/config.py:73-81)."""
+        total = 0
+        for spec in self.cache_slots.values():
+            elem = torch.empty((), dtype=spec.dtype or dtype).element_size()
+            total += spec.kv_heads * (spec.head_dim + spec.v_dim) * elem
+        return total
 
     def decode_weight_bytes(self) -> int:
         """Bytes of weights a step reads once: every layer the execution list runs, the final

@@ -49,7 +49,7 @@ class Sampler:
 
     def sample(self, logits: torch.Tensor, requests: list) -> list:
         """One token per row of float32 logits [n, V]; row i belongs to requests[i], whose
-        next output index is len(request.out)."""
+        next output index is request.num_out."""
         if not requests:
             if logits.shape[0]:
                 raise ValueError(f"{logits.shape[0]} rows of logits for no requests")
@@ -67,7 +67,7 @@ class Sampler:
         temps = [float(r.params.temperature) for r in requests]
         top_ps = [float(r.params.top_p) for r in requests]
         us = [uniform_for(self.seed if r.params.seed is None else r.params.seed, r.rid,
-                          len(r.out) + ahead) for r in requests]
+                          r.num_out + ahead) for r in requests]
         packed = self._to_device([temps, top_ps, us], logits.device)
         nucleus = packed[1] if any(p < 1.0 for p in top_ps) else None
         return ops.sample(logits, packed[0], nucleus, packed[2])

@@ -41,8 +41,8 @@ class DeterministicExecutor:
             need = -(-(work.start + work.count) // ps)
             if len(table) < need:
                 raise AssertionError(f"{r.rid}: {len(table)} pages cover less than {need}")
-            first = 0 if group.spec.window is None else \
-                max(0, work.start - group.spec.window + 1) // ps
+            first = 0 if group.window is None else \
+                max(0, work.start - group.window + 1) // ps
             live = table[first:need]
             if any(p < 0 for p in live):
                 raise AssertionError(f"{r.rid}: a page the step reads was given back")
@@ -54,10 +54,10 @@ class DeterministicExecutor:
         tokens = []
         for w in plan.work:
             self._check(w)
-            tokens.append(self.token_for(w.request.rid, len(w.request.out)) if w.emits else None)
+            tokens.append(self.token_for(w.request.rid, w.request.num_out) if w.emits else None)
         self.steps += 1
         self.prefill_tokens_seen += plan.num_prefill_tokens
-        self.decode_tokens_seen += len(plan.decode)
+        self.decode_tokens_seen += plan.num_decode
         if self.step_delay:
             time.sleep(self.step_delay)
         return ExecResult(tokens=tokens, forward_seconds=time.perf_counter() - started)

@@ -1,10 +1,12 @@
 """Random-weights mode: draw every tensor a model declares from a seed, and write a model
 folder (``config.json`` + ``model.safetensors``) that loads like any checkpoint.
 
-Each tensor has its own generator, seeded from (seed, tensor name), so the values do not
-depend on the order in which tensors are drawn.  Matrices, biases and embeddings are
-N(0, std); norm weights are 1 + N(0, std).  Values are drawn in float32 and then rounded to
-the storage dtype.
+The generator is the engine's own and counter-based: element i of a tensor is a function of
+(seed, tensor name, i) alone, computed by the same float32 code on the host (the host core)
+and on the GPU (the fill kernel), bit for bit, so that weights drawn on the device for a model
+too large to write out are the very numbers a written folder would hold.  Matrices, biases
+and embeddings are N(0, std); norm weights are 1 + N(0, std).  Values are computed in float32
+and then rounded to the storage dtype.
 """
 
 from __future__ import annotations
@@ -17,29 +19,47 @@ import torch
 
 from .safetensors_io import save_file
 
+_DTYPE_CODE = {torch.float32: 0, torch.bfloat16: 1}
 
-def _generator(seed: int, name: str, device="cpu") -> torch.Generator:
+
+def stream_key(seed: int, name: str) -> int:
+    """The 64-bit key of a tensor's random stream."""
     digest = hashlib.blake2b(f"{seed}:{name}".encode(), digest_size=8).digest()
-    g = torch.Generator(device=device)
-    g.manual_seed(int.from_bytes(digest, "little") & (2**63 - 1))
-    return g
+    return int.from_bytes(digest, "little")
+
+
+def fill_normal(out: torch.Tensor, key: int, mean: float, std: float) -> torch.Tensor:
+    """out[i] = mean + std * normal(key, i) over the flattened tensor, on the host or on the
+    GPU, wherever `out` lives."""
+    if out.dtype not in _DTYPE_CODE or not out.is_contiguous():
+        raise ValueError("random fill takes contiguous float32 or bfloat16 tensors")
+    code = _DTYPE_CODE[out.dtype]
+    if out.is_cuda:
+        from ..kernels import lib as _lib
+
+        lib = _lib.load("core")
+        with torch.cuda.device(out.device):
+            _lib.check(lib, lib.mk_fill_normal(out.data_ptr(), code, out.numel(), key, float(mean),
+                                               float(std), torch.cuda.current_stream().cuda_stream),
+                       "fill_normal")
+    else:
+        from ..hostcore import core
+
+        core.fill_normal(out.data_ptr(), code, out.numel(), key, float(mean), float(std))
+    return out
 
 
 def random_tensor(name: str, spec, seed: int, std: float, dtype: torch.dtype,
                   device="cpu") -> torch.Tensor:
-    """One declared tensor.  Drawn on `device`: the values for a seed are fixed per kind of
-    device (the CPU's are the ones a written model folder holds)."""
+    """One declared tensor, drawn where it is wanted."""
     if spec.role == "table":
         raise ValueError(f"{name}: integer tables have no random initialisation")
     if spec.init == "zeros":
         return torch.zeros(spec.shape, dtype=dtype, device=device)
-    t = torch.randn(spec.shape, generator=_generator(seed, name, device), dtype=torch.float32,
-                    device=device) * std
-    if spec.init == "one_plus_normal":
-        t += 1.0
-    elif spec.init != "normal":
+    if spec.init not in ("normal", "one_plus_normal"):
         raise ValueError(f"{name}: unknown initialisation {spec.init!r}")
-    return t.to(dtype)
+    out = torch.empty(spec.shape, dtype=dtype, device=device)
+    return fill_normal(out, stream_key(seed, name), 1.0 if spec.init == "one_plus_normal" else 0.0, std)
 
 
 def random_state(model, seed: int, std: float = 0.02, dtype: torch.dtype = torch.bfloat16) -> dict:

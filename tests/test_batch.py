@@ -36,8 +36,8 @@ def test_a_mixed_step_is_laid_out_by_sequence():
     assert step.logit_rows.tolist() == [0, 2, 3]
     assert step.spans == [(0, 3, 18), (3, 1, 8), (4, 3, 0)]
     assert (step.max_q_len, step.max_kv_len, step.all_decode) == (3, 21, False)
-    assert step.fresh_slots == [m.requests["c"].state_slot]
-    assert step.state_slots.tolist() == [m.requests[k].state_slot for k in "abc"]
+    assert step.fresh_slots == [m.sequence("c").state_slot]
+    assert step.state_slots.tolist() == [m.sequence(k).state_slot for k in "abc"]
     table = step.block_tables[0]
     assert table.shape == (3, 3)                          # 21 tokens need 3 pages of 8
     assert table[0].tolist() == m.table("a", 0)

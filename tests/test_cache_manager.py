@@ -19,7 +19,7 @@ OTHER = CacheSpec(kv_heads=1, head_dim=32, window=None)
 def test_slots_with_the_same_need_share_a_group():
     m = CacheManager({0: FULL, 1: WINDOW, 2: FULL, 3: OTHER, 4: WINDOW}, 16, PS, 4)
     assert [g.slots for g in m.groups] == [[0, 2], [1, 4], [3]]
-    assert m.group_of_slot == {0: 0, 2: 0, 1: 1, 4: 1, 3: 2}
+    assert {s: m.group_of(s) for s in range(5)} == {0: 0, 2: 0, 1: 1, 4: 1, 3: 2}
     assert not m.prefix_sharing                       # a window group cannot share prefixes
     assert CacheManager({0: FULL, 1: OTHER}, 16, PS, 4).prefix_sharing
     assert not CacheManager({0: FULL}, 16, PS, 4, has_state=True).prefix_sharing

@@ -7,7 +7,7 @@ import random
 
 import pytest
 
-from mercury_amd.engine.request import SamplingParams
+from mercury_amd.engine import SamplingParams
 from mercury_amd.parts import CacheSpec
 from tests.engine_harness import FULL, build
 

@@ -258,7 +258,7 @@ def test_toy_architecture_registered_built_and_stepped(tmp_path):
     want = {k: plain_toy_logits(w, cfg, v) for k, v in reqs.items()}
 
     s = ReplaySession(folder, "float32", 256)
-    assert [g.spec.window for g in s.manager.groups] == [None, 24]
+    assert [g.window for g in s.manager.groups] == [None, 24]
     assert not s.manager.prefix_sharing and list(s.runner.states) == [1]
     for key, tokens in reqs.items():
         got = s.step([{"id": key, "tokens": tokens, "want": list(range(len(tokens)))}], [key])
@@ -349,7 +349,9 @@ def register_routed_toy():
     return build
 
 
-def plain_routed_logits(w, cfg, tokens):
+def plain_routed_logits(w, cfg, tokens, margins=None):
+    """Logits of the routed toy model; `margins`, a list, receives per layer the gap between
+    every token's two largest router probabilities."""
     eps, d = cfg["rms_norm_eps"], cfg["head_dim"]
     n_q, n_kv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
     t = len(tokens)
@@ -375,8 +377,12 @@ def plain_routed_logits(w, cfg, tokens):
         q, k = rotate(q, k, i)
         h = h + plain.causal_attention(q, k, v, d ** -0.5).reshape(t, -1) @ w[p + "mixer.o_proj.weight"].T
         x = plain.rms_norm(h, w[p + "norm2.weight"], eps)[0]
-        scores = torch.softmax(x @ w[p + "mlp.router.weight"].T, dim=-1)
+        scores = torch.softmax(x.float() @ w[p + "mlp.router.weight"].float().T, dim=-1)
         weight, choice = scores.max(-1)
+        if margins is not None:
+            top = scores.topk(2, dim=-1).values
+            margins.append(top[:, 0] - top[:, 1])
+        weight = weight.to(h.dtype)
         out = torch.zeros_like(h)
         for e in range(3):
             gu, down = w[p + f"mlp.experts.{e}.gate_up.weight"], w[p + f"mlp.experts.{e}.down.weight"]
@@ -399,8 +405,14 @@ def test_routed_feed_forward_and_other_position_encodings(tmp_path):
     config = {**helpers.TINY_A, "architectures": ["TestRoutedLM"], "hidden_size": 64, "head_dim": 32,
               "num_attention_heads": 2, "num_key_value_heads": 1, "intermediate_size": 48,
               "tie_word_embeddings": False}
-    folder = write_random_model(tmp_path / "routed", config, seed=4, std=0.3, dtype=torch.float32)
+    from mercury_amd.weights import save_file
+
+    folder = write_random_model(tmp_path / "routed", config, seed=8, std=0.1, dtype=torch.float32)
     w = load_file(str(folder / "model.safetensors"))
+    # routers with wide weights: most tokens' choice of expert is far from a tie
+    # (copies: the loaded tensors are views of the very file that is rewritten here)
+    w = {k: (v * 16 if "router" in k else v.clone()) for k, v in w.items()}
+    save_file(w, folder / "model.safetensors")
     cfg = plain.read_config(folder)
     tokens = helpers.random_tokens(512, 70, 3)
     want = plain_routed_logits(w, cfg, tokens)
@@ -423,14 +435,24 @@ def test_routed_feed_forward_and_other_position_encodings(tmp_path):
 
     # bfloat16 (the matrix-core kernels take head size 32; rotation over half a head goes the
     # unfused way, no rotation the fused one).  Routing is discontinuous: a token whose two
-    # best router logits lie within bfloat16's rounding goes to another expert than in
-    # float32, and every later token attends to it.  So this is a check that the path runs
-    # and stays near (the first rows, before any such token, within the bound of the replay
-    # tests; the typical row within a few percent of the largest logit; a wrong rotation or
-    # expert would be off by the size of the logits themselves), not a bound on rounding.
+    # best router probabilities lie within bfloat16's rounding may go to another expert than
+    # in float32, and every later token attends to it.  So the comparison covers the tokens
+    # before the first one whose routing is that close in any layer; up to there the bound is
+    # the one the replay tests derive: the distance of the plain implementation's own
+    # bfloat16 run from its float32 run, times the slack.
+    from tests.test_gpu_replay import BF16_SLACK
+
+    margins = []
+    plain_routed_logits(w, cfg, tokens, margins)
+    fragile = (torch.stack(margins).amin(0) < 0.2).nonzero().flatten()
+    safe = int(fragile[0]) if fragile.numel() else len(tokens)
+    assert safe >= 16, f"the seed makes token {safe} fragile; pick weights with a later one"
+    w16 = {k: v.to(torch.bfloat16) for k, v in w.items()}
+    want16 = plain_routed_logits({k: v.float() for k, v in w16.items()}, cfg, tokens)
+    rounded = plain_routed_logits(w16, cfg, tokens).float()
+    cost = float((rounded[:safe] - want16[:safe]).abs().max())
     b = ReplaySession(folder, "bfloat16", 256)
     got = b.step([{"id": "w", "tokens": tokens, "want": list(range(70))}], ["w"])
     assert torch.isfinite(got).all()
-    error = (got - want).abs().amax(-1)
-    assert float(error[:4].max()) <= 0.02 * float(want.abs().max())
-    assert float(error.median()) <= 0.05 * float(want.abs().max())
+    error = (got[:safe] - want16[:safe]).abs().max()
+    assert float(error) <= BF16_SLACK * cost, (float(error), cost, safe)

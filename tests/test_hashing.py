@@ -44,7 +44,31 @@ def test_hashes_are_the_same_in_every_process_and_differ_by_mode():
     tokens = list(range(32))
     fast, strong = PageHasher(16), PageHasher(16, cryptographic=True)
     assert fast.hashes(tokens) == PageHasher(16).hashes(tokens)
-    assert fast.hashes(tokens)[0] == 0xD85847B14FA46C4   # not Python's per-process hash()
+    assert fast.hashes(tokens)[0] == 16304858532140510287   # not Python's per-process hash()
     assert strong.hashes(tokens) != fast.hashes(tokens)
     assert all(0 <= x < 2**128 for x in strong.hashes(tokens))
     assert strong.page_hash(strong.hashes(tokens)[0], tokens[16:32]) == strong.hashes(tokens)[1]
+
+
+def test_the_strong_mode_is_sha256_of_parent_and_tokens():
+    """The host core's own SHA-256 against hashlib's: the published vector for "abc", and a
+    page hash recomputed here from its definition (parent as 16 bytes, tokens as 8-byte
+    integers, little-endian; the first 128 bits of the digest, little-endian)."""
+    import hashlib
+    from array import array
+
+    from mercury_amd.hostcore import core
+
+    assert core.sha256(b"abc").hex() == \
+        "ba7816bf8f01cfea414140de5dae2223b00361a396177a9cb410ff61f20015ad"
+    for size in (0, 55, 56, 63, 64, 65, 200):
+        data = bytes(range(256))[:size] if size <= 256 else b""
+        assert core.sha256(data) == hashlib.sha256(data).digest()
+    strong = PageHasher(16, cryptographic=True)
+    tokens = [7, 0, 2**31 - 1] + list(range(13))
+    parent = 0
+    for _ in range(2):
+        payload = parent.to_bytes(16, "little") + array("q", tokens).tobytes()
+        want = int.from_bytes(hashlib.sha256(payload).digest()[:16], "little")
+        assert strong.page_hash(parent, tokens) == want
+        parent = want

@@ -7,8 +7,8 @@ from __future__ import annotations
 import random
 
 from mercury_amd.cache import CacheManager, PageHasher
-from mercury_amd.engine.request import Request, RequestState
-from mercury_amd.engine.scheduler import Scheduler
+from mercury_amd.engine import Request, RequestState
+from mercury_amd.engine import Scheduler
 from mercury_amd.parts import CacheSpec
 from tests.engine_harness import FULL, build
 
@@ -88,12 +88,12 @@ def test_aging_arithmetic():
     shared = list(range(2048))
     warm(manager, shared)
     cold = request("cold", [99_999] * 80, 0.0)
-    assert sched._score(cold, 1.0) < sched._score(request("h1", shared + [7] * 16, 1.0), 1.0)
-    assert sched._score(cold, 2.0) > sched._score(request("h2", shared + [7] * 16, 2.0), 2.0)
+    assert sched.score(cold, 1.0) < sched.score(request("h1", shared + [7] * 16, 1.0), 1.0)
+    assert sched.score(cold, 2.0) > sched.score(request("h2", shared + [7] * 16, 2.0), 2.0)
     hot = request("hot", shared + [7] * 16, 1.0)
-    assert all(sched._score(cold, t) < sched._score(hot, t) for t in (2.0, 5.0, 20.0))
+    assert all(sched.score(cold, t) < sched.score(hot, t) for t in (2.0, 5.0, 20.0))
     sched.max_wait_s = 5.0
-    assert sched._score(cold, 5.0) == float("inf")
+    assert sched.score(cold, 5.0) == float("inf")
 
 
 def test_scan_limit_bounds_the_scoring():
@@ -148,7 +148,7 @@ def test_preemption_takes_the_newest_admitted_and_requeues_by_arrival():
     assert rids(plan.preempted) == ["r3", "r2"] and rids(sched.running) == ["r0", "r1"]
     assert rids(w.request for w in plan.work) == ["r0", "r1"]
     victim = plan.preempted[0]
-    assert victim.state is RequestState.WAITING and victim.num_computed == 0
+    assert victim.state == RequestState.WAITING and victim.num_computed == 0
     assert victim.preemptions == 1 and not manager.holds("r3")
     assert rids(sched.waiting) == ["r2", "r3"]                    # back in arrival order
     assert len(victim.hashes) == 2                                # rehashed over prompt + output

@@ -95,3 +95,24 @@ def test_no_weights_is_a_clear_error(tmp_path):
     (tmp_path / "config.json").write_text(json.dumps(TINY_A))
     with pytest.raises(FileNotFoundError, match="no safetensors"):
         FolderSource(tmp_path)
+
+
+def test_random_weights_are_a_function_of_seed_name_and_index():
+    """The engine's own generator: normal deviates from (seed, tensor name, element index)
+    alone, so a tensor's values do not depend on what else is drawn, or where."""
+    import torch
+
+    from mercury_amd.weights.random_init import fill_normal, stream_key
+
+    a = fill_normal(torch.empty(200_000), stream_key(3, "w"), 0.0, 1.0)
+    assert torch.equal(a[:1000], fill_normal(torch.empty(1000), stream_key(3, "w"), 0.0, 1.0))
+    assert not torch.equal(a[:1000], fill_normal(torch.empty(1000), stream_key(4, "w"), 0.0, 1.0))
+    assert not torch.equal(a[:1000], fill_normal(torch.empty(1000), stream_key(3, "v"), 0.0, 1.0))
+    # a standard normal: moments, tails, symmetry
+    assert abs(float(a.mean())) < 0.01 and abs(float(a.std()) - 1.0) < 0.01
+    assert abs(float((a.abs() > 1.959964).float().mean()) - 0.05) < 0.003
+    assert abs(float((a > 0).float().mean()) - 0.5) < 0.005
+    assert abs(float((a ** 4).mean()) - 3.0) < 0.1
+    # scaled, shifted, and rounded to bfloat16 from the float32 value
+    b = fill_normal(torch.empty(1000, dtype=torch.bfloat16), stream_key(3, "w"), 1.0, 0.02)
+    assert torch.equal(b, (1.0 + 0.02 * a[:1000]).to(torch.bfloat16))
