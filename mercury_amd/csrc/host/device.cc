@@ -265,15 +265,16 @@ void bind_device(py::module_& m) {
       }), py::arg("manager"), py::arg("vocab_size"), py::arg("max_positions"),
            py::arg("pinned") = true)
       .def("pack", [](StepPacker& packer, py::handle chunks, std::shared_ptr<Program> program,
-                      int table_width, bool check_ids) {
+                      int table_width, bool check_ids, int kv_bound) {
         Chunks c(chunks);
-        return packer.pack(c.seqs, program.get(), table_width, check_ids);
-      }, py::arg("chunks"), py::arg("program") = nullptr, py::arg("table_width") = -1,
-           py::arg("check_ids") = true)
+        return packer.pack(c.seqs, program.get(), table_width, check_ids, kv_bound);
+      }, py::keep_alive<0, 1>(), py::arg("chunks"), py::arg("program") = nullptr,
+           py::arg("table_width") = -1, py::arg("check_ids") = true, py::arg("kv_bound") = 0)
       .def("pack_plan", [](StepPacker& packer, const Plan& plan, std::shared_ptr<Program> program,
-                           int table_width) {
-        return packer.pack_plan(plan, program.get(), table_width);
-      }, py::arg("plan"), py::arg("program") = nullptr, py::arg("table_width") = -1)
+                           int table_width, int kv_bound) {
+        return packer.pack_plan(plan, program.get(), table_width, kv_bound);
+      }, py::keep_alive<0, 1>(), py::arg("plan"), py::arg("program") = nullptr,
+           py::arg("table_width") = -1, py::arg("kv_bound") = 0)
       .def("upload", [](StepPacker& packer, const PackedStep& step, uintptr_t device,
                         uintptr_t stream) {
         packer.upload(step, as_ptr<void>(device), as_ptr<void>(stream));

@@ -1,6 +1,6 @@
 #include "step_batch.h"
 
-#include <hip/hip_runtime_api.h>
+#include "hip_api.h"
 
 #include <algorithm>
 #include <cstdlib>
@@ -13,7 +13,7 @@ namespace mercury {
 
 namespace {
 void hip_check(hipError_t e, const char* what) {
-  if (e != hipSuccess) throw KernelError(std::string(what) + ": " + hipGetErrorString(e));
+  if (e != hipSuccess) throw KernelError(std::string(what) + ": " + hip().error_string(e));
 }
 }  // namespace
 
@@ -64,9 +64,9 @@ StepPacker::StepPacker(std::shared_ptr<CacheManager> manager, int vocab_size, in
 
 StepPacker::~StepPacker() {
   for (Slot& s : ring_) {
-    if (s.event) (void)hipEventDestroy((hipEvent_t)s.event);
+    if (s.event) (void)hip().event_destroy((hipEvent_t)s.event);
     if (s.data) {
-      if (s.pinned) (void)hipHostFree(s.data); else std::free(s.data);
+      if (s.pinned) (void)hip().host_free(s.data); else std::free(s.data);
     }
   }
 }
@@ -76,18 +76,18 @@ int32_t* StepPacker::acquire(size_t ints, int& slot_index) {
   next_ = (next_ + 1) % (int)ring_.size();
   Slot& s = ring_[slot_index];
   if (s.in_flight) {
-    hip_check(hipEventSynchronize((hipEvent_t)s.event), "waiting for a step buffer's copy");
+    hip_check(hip().event_synchronize((hipEvent_t)s.event), "waiting for a step buffer's copy");
     s.in_flight = false;
   }
   if (s.capacity < ints) {
     if (s.data) {
-      if (s.pinned) (void)hipHostFree(s.data); else std::free(s.data);
+      if (s.pinned) (void)hip().host_free(s.data); else std::free(s.data);
     }
     const size_t capacity = std::max<size_t>(ints + ints / 2, 4096);
     s.pinned = pinned_;
     if (pinned_) {
       void* p = nullptr;
-      hip_check(hipHostMalloc(&p, capacity * sizeof(int32_t), hipHostMallocDefault),
+      hip_check(hip().host_malloc(&p, capacity * sizeof(int32_t), hipHostMallocDefault),
                 "allocating a pinned step buffer");
       s.data = (int32_t*)p;
     } else {
@@ -100,7 +100,7 @@ int32_t* StepPacker::acquire(size_t ints, int& slot_index) {
 }
 
 PackedStep StepPacker::pack(const std::vector<SeqInput>& seqs, const Program* program,
-                            int table_width, bool check_ids) {
+                            int table_width, bool check_ids, int kv_bound) {
   if (seqs.empty()) throw BatchError("a step needs at least one sequence");
   PackedStep p;
   const int page = manager_->page_size();
@@ -122,6 +122,7 @@ PackedStep StepPacker::pack(const std::vector<SeqInput>& seqs, const Program* pr
     p.max_kv_len = std::max(p.max_kv_len, s.start + s.count);
     needed = std::max(needed, (s.start + s.count + page - 1) / page);
   }
+  p.max_kv_len = std::max(p.max_kv_len, kv_bound);
   const int width = table_width < 0 ? needed : table_width;
   if (width < needed) {
     throw BatchError("block tables of width " + std::to_string(width) + " cannot hold " +
@@ -214,7 +215,8 @@ PackedStep StepPacker::pack(const std::vector<SeqInput>& seqs, const Program* pr
   return p;
 }
 
-PackedStep StepPacker::pack_plan(const Plan& plan, const Program* program, int table_width) {
+PackedStep StepPacker::pack_plan(const Plan& plan, const Program* program, int table_width,
+                                 int kv_bound) {
   std::vector<SeqInput> seqs;
   seqs.reserve(plan.work.size());
   for (const Work& w : plan.work) {
@@ -226,19 +228,20 @@ PackedStep StepPacker::pack_plan(const Plan& plan, const Program* program, int t
     if (w.emits) in.want.push_back(w.count - 1);
     seqs.push_back(std::move(in));
   }
-  return pack(seqs, program, table_width);
+  return pack(seqs, program, table_width, true, kv_bound);
 }
 
 void StepPacker::upload(const PackedStep& step, void* device, void* stream) {
   Slot& s = ring_.at((size_t)step.ring_slot);
-  hip_check(hipMemcpyAsync(device, step.host, step.total * sizeof(int32_t), hipMemcpyHostToDevice,
-                           (hipStream_t)stream), "copying a step to the device");
+  hip_check(hip().memcpy_async(device, step.host, step.total * sizeof(int32_t),
+                               hipMemcpyHostToDevice, (hipStream_t)stream),
+            "copying a step to the device");
   if (!s.event) {
     hipEvent_t e;
-    hip_check(hipEventCreateWithFlags(&e, hipEventDisableTiming), "creating an event");
+    hip_check(hip().event_create(&e, hipEventDisableTiming), "creating an event");
     s.event = e;
   }
-  hip_check(hipEventRecord((hipEvent_t)s.event, (hipStream_t)stream), "recording an event");
+  hip_check(hip().event_record((hipEvent_t)s.event, (hipStream_t)stream), "recording an event");
   s.in_flight = true;
 }
 

@@ -65,9 +65,12 @@ class StepPacker {
 
   // table_width < 0: as many columns as the longest sequence needs.  `program` may be null
   // (then no tile lists are laid out).  `check_ids` off when the ids are not the host's to know.
+  // kv_bound > 0: the step is planned (attention key splits) as if its longest sequence had
+  // that many tokens, as a captured graph needs that later, longer steps will replay.
   PackedStep pack(const std::vector<SeqInput>& seqs, const Program* program, int table_width,
-                  bool check_ids = true);
-  PackedStep pack_plan(const Plan& plan, const Program* program, int table_width);
+                  bool check_ids = true, int kv_bound = 0);
+  PackedStep pack_plan(const Plan& plan, const Program* program, int table_width,
+                       int kv_bound = 0);
   // Copy the packed buffer to `device` on `stream`; the buffer's place in the ring is free
   // again once the copy has run.
   void upload(const PackedStep& step, void* device, void* stream);

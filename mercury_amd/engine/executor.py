@@ -19,22 +19,27 @@ class ExecResult:
     complete its sequence (a prompt portion that is not the last)."""
 
     tokens: list = field(default_factory=list)
-    prepare_seconds: float = 0.0
-    forward_seconds: float = 0.0
+    prepare_seconds: float = 0.0      # packing the step and copying it to the device (host)
+    forward_seconds: float = 0.0      # the rest of the host's wall clock, the wait included
+    device_seconds: float = 0.0       # the step's kernels, by events on the device
 
 
 class _Pending:
     """Tokens on their way from the device into pinned host memory: `wait()` gives them as a
-    list."""
+    list.  `began` is the event recorded before the step's first kernel."""
 
-    def __init__(self, tokens_dev, host, done):
-        self.host, self.done = host[:tokens_dev.shape[0]], done
+    def __init__(self, tokens_dev, host, done, began=None):
+        self.host, self.done, self.began = host[:tokens_dev.shape[0]], done, began
         self.host.copy_(tokens_dev, non_blocking=True)
         self.done.record()
 
     def wait(self) -> list:
         self.done.synchronize()
         return self.host.tolist()
+
+    def device_seconds(self) -> float:
+        """Time on the device from the step's first kernel to its tokens' copy (after wait)."""
+        return 1e-3 * self.began.elapsed_time(self.done) if self.began is not None else 0.0
 
 
 class _PinnedRing:
@@ -47,19 +52,24 @@ class _PinnedRing:
 
         self.size = size
         self.buffers = [torch.empty(size, dtype=torch.int32, pin_memory=True) for _ in range(depth)]
-        self.events = [torch.cuda.Event() for _ in range(depth)]
+        self.events = [torch.cuda.Event(enable_timing=True) for _ in range(depth)]
+        self.starts = [torch.cuda.Event(enable_timing=True) for _ in range(depth)]
         self.next = 0
+
+    def begin(self):
+        """Record, now, the start event of the step whose tokens the next `pending` carries."""
+        self.starts[self.next].record()
 
     def pending(self, tokens_dev) -> _Pending:
         import torch
 
         n = tokens_dev.shape[0]
-        if n > self.size:
-            return _Pending(tokens_dev, torch.empty(n, dtype=torch.int32, pin_memory=True),
-                            torch.cuda.Event())
         i = self.next
         self.next = (i + 1) % len(self.buffers)
-        return _Pending(tokens_dev, self.buffers[i], self.events[i])
+        if n > self.size:
+            return _Pending(tokens_dev, torch.empty(n, dtype=torch.int32, pin_memory=True),
+                            torch.cuda.Event(enable_timing=True), self.starts[i])
+        return _Pending(tokens_dev, self.buffers[i], self.events[i], self.starts[i])
 
 
 @dataclass
@@ -90,8 +100,8 @@ class GpuExecutor:
         self.model_config = runner.model.config
         self.kv_bytes = runner.kv_bytes
         manager = runner.manager
-        self.lookahead = (bool(lookahead) and runner.use_graphs and not runner.states
-                          and all(g.window is None for g in manager.groups))
+        self.lookahead = (bool(lookahead) and runner.use_graphs and runner.program is not None
+                          and not runner.states and all(g.window is None for g in manager.groups))
         self._ahead: _Ahead | None = None
         self._ring = _PinnedRing(max(256, runner.max_graph_batch))
         self.stats = {"ahead_started": 0, "ahead_used": 0}
@@ -105,14 +115,9 @@ class GpuExecutor:
             self.stats["ahead_used"] += 1
             self.runner.last_prepare_seconds = 0.0
         else:
-            chunks = []
-            for w in work:
-                tokens = (w.request.tokens[w.start:w.start + w.count] if w.count > 1
-                          else [w.request.token_at(w.start)])
-                chunks.append(SeqChunk(w.request.rid, tokens, w.start,
-                                       [w.count - 1] if w.emits else []))
-            logits = self.runner.step(chunks)
-            emitting = [w.request for w in work if w.emits]
+            self._ring.begin()
+            logits = self.runner.step_plan(plan)
+            emitting = plan.emitting
             tokens_dev = self.sampler.launch(logits, emitting) if emitting else None
             pending = self._ring.pending(tokens_dev) if emitting else None
         if self.lookahead and plan.steady:
@@ -127,6 +132,8 @@ class GpuExecutor:
             self._ahead.fed = result.tokens
         result.prepare_seconds = self.runner.last_prepare_seconds
         result.forward_seconds = time.perf_counter() - started - result.prepare_seconds
+        if pending is not None:
+            result.device_seconds = pending.device_seconds()
         return result
 
     @staticmethod
@@ -146,7 +153,7 @@ class GpuExecutor:
         step that is asked for) or a page the next positions need cannot be had."""
         manager = self.runner.manager
         chunks = [SeqChunk(w.request.rid, [0], w.start + 1, [0]) for w in work]
-        if not self.runner.captured(chunks):
+        if not self.runner.captured(len(chunks), max(c.start for c in chunks) + 1):
             return None
         if any(c.start + 1 > self.runner.max_model_len for c in chunks):
             return None
@@ -156,7 +163,8 @@ class GpuExecutor:
         for c in chunks:
             if not manager.grow(c.key, c.start, c.start + 1):
                 return None
-        logits = self.runner.step_graphed(chunks, ids=tokens_dev)
+        self._ring.begin()
+        logits = self.runner.step_ahead(chunks, tokens_dev)
         requests = [w.request for w in work]
         next_dev = self.sampler.launch(logits, requests, ahead=1)
         self.stats["ahead_started"] += 1

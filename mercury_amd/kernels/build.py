@@ -58,7 +58,7 @@ HIPCC_FLAGS = [
 
 # The host core: C++ (pybind11) for the cache manager, the scheduler, step packing and the
 # launch sequence of a step.  Compiled with the host compiler; it reaches the kernel libraries
-# through dlopen, so it links against the HIP runtime only.
+# and the HIP runtime through dlopen/dlsym, so it links against neither.
 HOST_NAME = "host"
 HOST_DIR = CSRC / "host"
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off", "-pthread",
@@ -187,8 +187,8 @@ def _host_commands(sources: list, objects: list, target: Path) -> tuple:
                 "-I", str(rocm / "include"), "-I", str(CSRC), "-I", str(HOST_DIR)]
     compiles = [[cxx, *HOST_FLAGS, *includes, "-c", str(src), "-o", str(obj)]
                 for src, obj in zip(sources, objects)]
-    link = [cxx, "-shared", "-pthread", "-o", str(target), *map(str, objects),
-            "-L", str(rocm / "lib"), f"-Wl,-rpath,{rocm / 'lib'}", "-lamdhip64", "-ldl"]
+    # No HIP runtime is linked: the core finds, at run time, the one the process already uses.
+    link = [cxx, "-shared", "-pthread", "-o", str(target), *map(str, objects), "-ldl"]
     return compiles, link
 
 

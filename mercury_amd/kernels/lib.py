@@ -87,6 +87,11 @@ def load(name: str = "core") -> ctypes.CDLL:
         fn = getattr(lib, fn_name)
         fn.argtypes = argtypes
         fn.restype = c_longlong if fn_name in _RETURNS_SIZE else c_int
+    # The host core launches a step's kernels itself and decides which kernel runs what: it
+    # opens the same library.
+    from ..hostcore import core
+
+    core.load_kernels(name, str(path))
     _loaded[name] = lib
     return lib
 

@@ -145,39 +145,39 @@ def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Te
 # --------------------------------------------------------------------------------- projection
 
 
-SKINNY_MAX_ROWS = 64
-SKINNY_SPLIT_MAX_ROWS = 16     # K-split partial sums: the skinny kernel up to here, tiles beyond
-SKINNY_SPLIT_MAX_WEIGHTS = 20 << 20   # bytes; larger matrices stream faster through the tiles' LDS ring
-TILED_MIN_ROWS = 8             # head and gated projection: the skinny kernel below, tiles from here
-FUSED_QKV_SPLIT_WEIGHTS = 24 << 20  # bytes; from here on partial sums and a finishing kernel
-FUSED_QKV_TILED_ROWS = 256
-FUSED_QKV_MIN_WORKGROUPS = 128
+def _core():
+    from ..hostcore import core
+
+    return core
+
+
+def _ensure(x: torch.Tensor):
+    """The libraries an operand of this dtype may need, loaded (into this process and into the
+    host core, which makes the choices below)."""
+    _lib.load("core")
+    if x.dtype == torch.bfloat16:
+        _lib.load("mfma")
+    return _core()
+
+
+SKINNY_MAX_ROWS = 64           # most rows the fused skinny q/k/v kernel takes
+
+# Which kernel runs a projection, a q/k/v projection or an attention of given sizes is decided
+# in the host core (csrc/host/dispatch.cc), where the measurements behind every threshold are
+# written down; the step programs ask the same functions.
 
 
 def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
     """Whether x W^T is best computed as K-split float32 partial sums (`linear_partials`):
     bfloat16 x of few enough rows, and a matrix large enough for bandwidth to matter, that
     whole-K workgroups would leave compute units idle or unevenly loaded."""
-    if not _mfma_eligible(x, w):
-        return False
-    lib = _lib.load("mfma")
-    m, (n, k) = x.shape[0], w.shape
-    if _partials_by_skinny(m, n, k):
-        return not lib.mk_linear_skinny_unsplit(m, n, k)
-    return lib.mk_linear_tiled_slices(m, n, k) > 1
-
-
-def _partials_by_skinny(m: int, n: int, k: int) -> bool:
-    """Few rows over a matrix of modest size: weights straight from HBM into the matrix cores.
-    More rows re-read x too often that way, and a large matrix streams faster through the
-    tiled kernel's ring of LDS buffers (5120 x 27648 at 8 rows: 57 against 50 us; 896 x 4864:
-    4.8 against 5.4)."""
-    return m <= SKINNY_SPLIT_MAX_ROWS and n * k * 2 < SKINNY_SPLIT_MAX_WEIGHTS
+    core = _ensure(x)
+    return core.wants_partials(dtype_code(x.dtype), dtype_code(w.dtype), x.shape[0], w.shape[0],
+                               w.shape[1])
 
 
 def _mfma_eligible(x, w: torch.Tensor) -> bool:
-    return (x.dtype == torch.bfloat16 and w.dtype == torch.bfloat16
-            and x.shape[0] > 0 and x.shape[1] % 8 == 0)
+    return _core().mfma_eligible(dtype_code(x.dtype), dtype_code(w.dtype), x.shape[0], x.shape[1])
 
 
 def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
@@ -191,13 +191,11 @@ def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
     m, k = x.shape
     n = w.shape[0]
     lib = _lib.load("mfma")
-    if _partials_by_skinny(m, n, k):
-        slices = lib.mk_linear_skinny_slices(m, n, k)
-        out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+    skinny, slices = _core().plan_partials(m, n, k)
+    out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
+    if skinny:
         code = lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream())
     else:
-        slices = lib.mk_linear_tiled_slices(m, n, k)
-        out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
         code = lib.mk_linear_tiled_partials(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream())
     _lib.check(lib, code, "linear_partials")
     return out
@@ -205,8 +203,10 @@ def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
 
 def fuses_gating(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
     """Whether `gated_projection` takes these operands (bfloat16, K a multiple of 8)."""
-    return (x.dtype == torch.bfloat16 and w_gate_up.dtype == torch.bfloat16
-            and x.shape[0] > 0 and x.shape[1] % 8 == 0 and w_gate_up.shape[0] % 2 == 0)
+    if x.dtype not in _DTYPE_CODE or w_gate_up.dtype not in _DTYPE_CODE:
+        return False
+    return _core().fuses_gating(dtype_code(x.dtype), dtype_code(w_gate_up.dtype), x.shape[0],
+                                x.shape[1], w_gate_up.shape[0])
 
 
 def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor,
@@ -224,7 +224,7 @@ def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor,
     lib = _lib.load("mfma")
     # From 8 rows on the tiled kernel streams the weights faster than the skinny one
     # (18944 x 3584 at 1, 8, 16, 32 rows: skinny 50, 57, 63, 80 us; tiles 55, 55, 55, 58).
-    skinny = m < TILED_MIN_ROWS
+    skinny = _core().gated_is_skinny(m)
     if skinny and tile_config is None:
         code = lib.mk_gated_skinny(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream())
     else:
@@ -267,21 +267,19 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
         raise KernelArgumentError(f"linear: out {tuple(out.shape)} is not [{m}, {n}]")
     if m == 0:
         return out
-    if kernel == "auto":
-        kernel = "mfma" if x.dtype == torch.bfloat16 and k % 8 == 0 else "generic"
-    if kernel == "mfma":
-        if x.dtype != torch.bfloat16 or k % 8:
-            raise KernelArgumentError("linear: the matrix-core kernels take bfloat16 with K % 8 == 0")
+    if kernel == "mfma" and (x.dtype != torch.bfloat16 or k % 8):
+        raise KernelArgumentError("linear: the matrix-core kernels take bfloat16 with K % 8 == 0")
+    # 0: the float32-arithmetic kernel; 1: a few rows straight from HBM into the matrix cores;
+    # 2: the same, added into `out`; 3: tiles through LDS
+    kind = _ensure(x).choose_linear(dtype_code(x.dtype), m, n, k, bias is not None, accumulate,
+                                    dtype_code(out_dtype), {"auto": 0, "generic": 1, "mfma": 2}[kernel])
+    if kind != 0:
         lib = _lib.load("mfma")
-        # A few rows straight from HBM into the matrix cores; from 8 rows on the tiles' ring of
-        # LDS buffers streams the weights faster (the head, 152064 x 3584, at 1, 8, 16, 64
-        # rows: skinny 188, 204, 238, 429 us; tiles 187, 191, 198, 221).
-        if (m < TILED_MIN_ROWS and out_dtype == torch.float32 and bias is None
-                and not accumulate):
+        if kind == 1:
             _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, 1, _stream()),
                        "linear")
             return out
-        if m <= SKINNY_SPLIT_MAX_ROWS and accumulate:
+        if kind == 2:
             _lib.check(lib, lib.mk_linear_skinny_acc(
                 _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
                 _ptr(out), m, n, k, _stream()), "linear")
@@ -320,16 +318,21 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor
                   positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                   k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, n_q: int,
                   n_kv: int, head_dim: int, rotary_dim: int, write_kv: bool = True,
-                  bias: torch.Tensor | None = None, out_dtype: torch.dtype | None = None):
+                  bias: torch.Tensor | None = None, out_dtype: torch.dtype | None = None,
+                  interleaved: bool = False):
     """Rotate q and k by their absolute positions; write k into the paged key cache
     [pages, n_kv, page_size, head_dim] and v into the value cache
     [pages, n_kv, head_dim, page_size] at the slots the block table gives.
 
+    The first `rotary_dim` dims of a head turn; pair j is dims (j, j + rotary_dim/2), or
+    (2j, 2j + 1) when `interleaved`.
     qkv [T, (n_q + 2 n_kv) d] in the compute dtype is rotated in place (q part) and returned.
     qkv as float32 partial sums [P, T, width] is summed (plus `bias`) first, and the rotated q
     comes back as a new [T, n_q d] tensor of `out_dtype`."""
     _dev(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache, bias)
     if qkv.dim() == 3:
+        if interleaved and rotary_dim:
+            raise KernelArgumentError("rope: partial sums are finished in the half-split layout only")
         return _qkv_finish(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache,
                            n_q, n_kv, head_dim, rotary_dim, write_kv, bias, out_dtype)
     if bias is not None:
@@ -356,7 +359,7 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor
         _ptr(qkv), dtype_code(qkv.dtype), row, _ptr(cos), _ptr(sin), table_positions,
         _ptr(positions), _ptr(token_seq), _ptr(block_table), block_table.shape[1],
         _ptr(k_cache), _ptr(v_cache), page_size, n_q, n_kv, head_dim, rotary_dim,
-        int(write_kv), tokens, _stream()), "rope_kv_write")
+        int(bool(interleaved)), int(write_kv), tokens, _stream()), "rope_kv_write")
     return qkv
 
 
@@ -391,9 +394,12 @@ def _qkv_finish(parts, cos, sin, positions, token_seq, block_table, k_cache, v_c
     return q
 
 
-def _qkv_fusable(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
-    return (_mfma_eligible(x, w) and head_dim % 32 == 0 and rotary_dim in (0, head_dim)
-            and page_size > 0 and page_size & (page_size - 1) == 0)
+def _qkv_fusable(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int,
+                 half_layout: bool = True) -> bool:
+    if x.dtype not in _DTYPE_CODE or w.dtype not in _DTYPE_CODE:
+        return False
+    return _core().qkv_fusable(dtype_code(x.dtype), dtype_code(w.dtype), x.shape[0], x.shape[1],
+                               head_dim, rotary_dim, page_size, half_layout)
 
 
 def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
@@ -402,29 +408,17 @@ def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int
     power of two; and not up to a few hundred rows over a matrix so large that partial sums
     over slices of K, followed by the rotation, stream it faster (7168 x 5120 at 64 rows: 43 us
     in one kernel, 20 + 7 in two)."""
-    return _qkv_kernel(x, w, head_dim, rotary_dim, page_size) is not None
+    return _qkv_kernel(x, w, head_dim, rotary_dim, page_size) in ("skinny", "tiled")
 
 
-def _qkv_kernel(x, w, head_dim, rotary_dim, page_size):
+def _qkv_kernel(x, w, head_dim, rotary_dim, page_size, half_layout: bool = True):
     """ "skinny" (up to 64 rows: weights straight into the matrix cores, one workgroup per 32
     rows of W with all of K), "tiled" (any number of rows, through LDS, where whole-K tiles
-    are the faster projection anyway), or None."""
-    if not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
-        return None
-    m = x.shape[0]
-    # A large matrix streams fastest as partial sums over slices of K, the rotation and the
-    # cache write in a small kernel after them (4608 x 3584 at 8, 16, 32, 64 rows: 14.0, 13.9,
-    # 15.4, 16.5 us against 15.2, 16.1, 21.1, 30.7 in the one skinny kernel; 7168 x 5120 at 8
-    # rows: 20.9 against 23.5; 1152 x 896 the other way round: 10.6 against 6.0).
-    if (m <= FUSED_QKV_TILED_ROWS and w.numel() * 2 >= FUSED_QKV_SPLIT_WEIGHTS
-            and wants_partials(x, w)):
-        return None
-    if m <= 16 or (m <= SKINNY_MAX_ROWS and w.shape[0] // 32 >= FUSED_QKV_MIN_WORKGROUPS):
-        return "skinny"
-    # many rows: partial sums would be a second pass over [rows, width] in float32
-    if m > FUSED_QKV_TILED_ROWS or not wants_partials(x, w):
-        return "tiled"
-    return None
+    are the faster projection anyway), "partials" (K-split partial sums, then the finishing
+    kernel) or "plain" (the projection, then the rotation and cache-write kernel)."""
+    kind = _ensure(x).choose_qkv(dtype_code(x.dtype), dtype_code(w.dtype), x.shape[0], w.shape[0],
+                                 x.shape[1], head_dim, rotary_dim, page_size, half_layout)
+    return ("skinny", "tiled", "partials", "plain")[kind]
 
 
 def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor | None,
@@ -432,7 +426,7 @@ def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor
                 block_table: torch.Tensor, k_cache: torch.Tensor | None,
                 v_cache: torch.Tensor | None, n_q: int, n_kv: int, head_dim: int,
                 rotary_dim: int, write_kv: bool = True, fused: bool | None = None,
-                tile_config: int = -1) -> torch.Tensor:
+                tile_config: int = -1, interleaved: bool = False) -> torch.Tensor:
     """q, k, v = x W^T + bias for W = [q heads | k heads | v heads]; q and k rotated by their
     positions; k and v written to the paged cache (`write_kv`; otherwise W holds the query
     heads only).  Returns the rotated q [T, n_q d].
@@ -446,21 +440,23 @@ def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor
     if w.shape[0] != width or w.shape[1] != x.shape[1]:
         raise KernelArgumentError(f"qkv_project: W {tuple(w.shape)} is not [{width}, {x.shape[1]}]")
     page_size = k_cache.shape[2] if write_kv and k_cache is not None else 1
+    half = not (interleaved and rotary_dim)
     if fused is None:
-        kernel = _qkv_kernel(x, w, head_dim, rotary_dim, page_size)
+        kernel = _qkv_kernel(x, w, head_dim, rotary_dim, page_size, half)
     elif not fused:
-        kernel = None
-    elif not _qkv_fusable(x, w, head_dim, rotary_dim, page_size):
+        kernel = "partials" if half and wants_partials(x, w) else "plain"
+    elif not _qkv_fusable(x, w, head_dim, rotary_dim, page_size, half):
         raise KernelArgumentError("qkv_project: these operands cannot take the fused kernel")
     else:
         kernel = "skinny" if x.shape[0] <= SKINNY_MAX_ROWS and tile_config < 0 else "tiled"
-    if kernel is None:
-        if wants_partials(x, w):
-            return rope_kv_write(linear_partials(x, w), cos, sin, positions, token_seq,
-                                 block_table, k_cache, v_cache, n_q, heads_kv, head_dim,
-                                 rotary_dim, write_kv, bias=bias, out_dtype=x.dtype)
+    if kernel == "partials":
+        return rope_kv_write(linear_partials(x, w), cos, sin, positions, token_seq,
+                             block_table, k_cache, v_cache, n_q, heads_kv, head_dim,
+                             rotary_dim, write_kv, bias=bias, out_dtype=x.dtype)
+    if kernel == "plain":
         return rope_kv_write(linear(x, w, bias), cos, sin, positions, token_seq, block_table,
-                             k_cache, v_cache, n_q, heads_kv, head_dim, rotary_dim, write_kv)
+                             k_cache, v_cache, n_q, heads_kv, head_dim, rotary_dim, write_kv,
+                             interleaved=not half)
     tokens, k = x.shape
     _dev(x, w, bias, cos, sin, positions, token_seq, block_table, k_cache, v_cache)
     _i32(positions, "positions")
@@ -521,10 +517,15 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     page_size = _check_caches("attention", k_cache, v_cache, n_kv, head_dim, q.dtype)
     if out is None:
         out = torch.empty((tokens, n_q * head_dim), dtype=q.dtype, device=q.device)
-    use_mfma = kernel == "mfma"
-    if kernel == "auto" and q.dtype == torch.bfloat16:
-        use_mfma = bool(_lib.load("mfma").mk_attention_mfma_supported(head_dim, page_size))
-    if not use_mfma:
+    counts = [count for _first, count, _start in step.spans]
+    plan = _ensure(q).plan_attention(
+        dtype_code(q.dtype), head_dim, page_size, n_q, n_kv, int(window or 0), counts,
+        step.max_q_len, step.max_kv_len, force={"auto": 0, "generic": 1, "mfma": 2}[kernel],
+        tile_rows=-1 if tile_rows is None else int(tile_rows),
+        staged=-1 if staged is None else int(staged),
+        splits=split_override[0] if split_override is not None else 0,
+        split_blocks=split_override[1] if split_override is not None else 0)
+    if not plan["mfma"]:
         lib = _lib.load("core")
         _lib.check(lib, lib.mk_attention_generic(
             _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
@@ -532,55 +533,10 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
             block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
             int(window or 0), tokens, _stream()), "attention")
         return out
-    if q.dtype != torch.bfloat16:
-        raise KernelArgumentError("attention: the matrix-core kernel takes bfloat16 only")
     lib = _lib.load("mfma")
     group = n_q // n_kv
-    # Tiles of 16 rows, the keys split when the tiles alone would leave most of the chip idle
-    # (decoding); wider tiles, whose rows share every key fragment a wavefront loads, when
-    # there are plenty (prompts).
-    span = step.max_kv_len if not window else min(step.max_kv_len, window + step.max_q_len)
-    blocks = max(1, -(-span // 32))
-    rows = 16
-    total_rows = sum(count for _first, count, _start in step.spans) * group
-    # 64-row tiles exist but run at one wavefront per SIMD; 32 rows measured fastest
-    max_rows = min(32, lib.mk_attention_mfma_max_rows(head_dim))
-    while rows < max_rows and (total_rows // (rows * 2)) * n_kv >= ATTENTION_WIDE_TILE_WAVES:
-        rows *= 2
-    if tile_rows is not None:
-        rows = tile_rows
-    if staged is None:
-        # prompts: plenty of rows per sequence, enough workgroups of 64 of them; 16 rows a
-        # wavefront measured faster than 32 there
-        staged = (split_override is None and tile_rows is None
-                  and step.max_q_len * group >= 64
-                  and (total_rows // 64) * n_kv >= ATTENTION_STAGED_WORKGROUPS
-                  and bool(lib.mk_attention_mfma_staged(head_dim, 16)))
-        if staged:
-            rows = 16
-            staged = -1       # as many key groups as pay, once the tiles are counted
-    tile_seq, tile_row0, num_tiles = step.tiles(group, rows * 4 if staged else rows)
-    if staged == -1:
-        # A workgroup's chain of key blocks is cut into 2 or 4 chains side by side while that
-        # leaves the chip short of wavefronts and every chain a few blocks (measured at 2,048
-        # tokens, 14 heads of 64: 45, 35, 32 us with 1, 2, 4 groups; at 8,192: 264, 349, 284;
-        # 28 heads of 128 at 2,048: 100, 91 with 1, 2; at 8,192: 878, 1055).
-        staged = lib.mk_attention_mfma_staged(head_dim, 16)
-        while staged > 1 and (num_tiles * n_kv * 4 * staged > ATTENTION_STAGED_MAX_WAVES
-                              or blocks < 4 * staged):
-            staged //= 2
-    splits, split_blocks = 1, 0
-    waves = max(1, num_tiles * n_kv)
-    if staged:
-        pass
-    elif waves < ATTENTION_TARGET_WAVES:
-        # decoding, and short prompt portions over a long prefix (16 tokens over 2,032: 47 us
-        # as one chain of key blocks per wavefront, 23 split): every tile's own range of keys
-        # in equal parts
-        splits = max(1, min(blocks // ATTENTION_MIN_BLOCKS_PER_SPLIT or 1,
-                            -(-ATTENTION_TARGET_WAVES // waves), ATTENTION_MAX_SPLITS))
-    if split_override is not None:
-        splits, split_blocks = split_override
+    rows, staged, splits, split_blocks = plan["rows"], plan["staged"], plan["splits"], plan["split_blocks"]
+    tile_seq, tile_row0, num_tiles = step.tiles(group, plan["tile_rows"])
     part_o = part_ml = None
     if splits > 1:
         part_o = torch.empty((num_tiles, n_kv, splits, rows, head_dim), dtype=torch.float32, device=q.device)
@@ -592,16 +548,6 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
         int(window or 0), rows, int(staged), splits, split_blocks, _ptr(part_o), _ptr(part_ml),
         _stream()), "attention")
     return out
-
-
-ATTENTION_TARGET_WAVES = 1024
-ATTENTION_STAGED_WORKGROUPS = 64
-ATTENTION_STAGED_MAX_WAVES = 8192
-ATTENTION_WIDE_TILE_WAVES = 400
-ATTENTION_MIN_BLOCKS_PER_SPLIT = 2
-# beyond this the merge of the parts costs more than the shorter chains save (one sequence of
-# 16,384 tokens, 28 heads of 128: 25 us with 256 parts, 17 with 64 or 128)
-ATTENTION_MAX_SPLITS = 128
 
 
 # ----------------------------------------------------------------------------------- sampling

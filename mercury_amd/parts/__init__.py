@@ -1,8 +1,8 @@
 """Layer parts: mixers, feed-forwards, norms, position encodings, blocks, the decoder."""
 
 from .attention import Attention
-from .base import (CacheSpec, FeedForward, LayerCache, Mixer, Norm, Part, PositionEncoding,
-                   StateSpec, TensorSpec)
+from .base import (CacheSpec, FeedForward, LayerCache, Mixer, Norm, Part, PositionDescriptor,
+                   PositionEncoding, StateSpec, TensorSpec)
 from .block import PreNormBlock
 from .feedforward import GatedMLP
 from .model import DecoderModel, LayerCall
@@ -20,7 +20,8 @@ register_block("pre_norm")(PreNormBlock)
 
 __all__ = [
     "Attention", "CacheSpec", "DecoderModel", "FeedForward", "GatedMLP", "LayerCache",
-    "LayerCall", "Mixer", "NoPosition", "Norm", "Part", "PositionEncoding", "PreNormBlock",
+    "LayerCall", "Mixer", "NoPosition", "Norm", "Part", "PositionDescriptor", "PositionEncoding",
+    "PreNormBlock",
     "RMSNorm", "RotaryPosition", "StateSpec", "TensorSpec", "build_part", "known",
     "register_block", "register_ffn", "register_mixer", "register_norm", "register_position",
 ]

@@ -78,17 +78,51 @@ class Attention(Mixer):
 
     # ---- one step
 
+    @property
+    def lowerable(self) -> bool:
+        """The host core runs this attention itself when the kernels can apply its position
+        encoding."""
+        return self.position.describe() is not None
+
+    def lower(self, program, cache) -> None:
+        pos = self.position.describe()
+        bias_code = lambda t: ops.dtype_code(t.dtype) if t is not None else ops.F32
+        ptr = lambda t: 0 if t is None else t.data_ptr()
+        if cache.k.dtype != self.w_qkv.dtype:
+            raise ValueError("the kernels keep keys and values in the compute dtype")
+        program.attention(
+            w_qkv=self.w_qkv.data_ptr(), b_qkv=ptr(self.b_qkv), b_qkv_dtype=bias_code(self.b_qkv),
+            w_o=self.w_o.data_ptr(), b_o=ptr(self.b_o), b_o_dtype=bias_code(self.b_o),
+            n_q=self.n_q, n_kv=self.n_kv, head_dim=self.head_dim, rotary_dim=pos.rotary_dim,
+            cos=ptr(pos.cos), sin=ptr(pos.sin),
+            table_positions=0 if pos.cos is None else pos.cos.shape[0],
+            interleaved=pos.interleaved, k_cache=cache.k.data_ptr(), v_cache=cache.v.data_ptr(),
+            group=cache.group, page_size=cache.page_size, scale=self.scale,
+            window=self.window or 0, writes=cache.writes)
+
     def forward(self, x, step, cache, state, accum):
         n_q, n_kv, d = self.n_q, self.n_kv, self.head_dim
         table = step.block_tables[cache.group]
-        pos = self.position
+        pos = self.position.describe()
         w, b = self.w_qkv, self.b_qkv
         if not cache.writes:
             # Reads a cache another entry fills: only the queries are projected.
             w, b = w[:n_q * d], None if b is None else b[:n_q * d]
         k_cache, v_cache = (cache.k, cache.v) if cache.writes else (None, None)
-        q = ops.qkv_project(x, w, b, pos.cos, pos.sin, step.positions, step.token_seq, table,
-                            k_cache, v_cache, n_q, n_kv, d, pos.rotary_dim, cache.writes)
+        if pos is not None:
+            q = ops.qkv_project(x, w, b, pos.cos, pos.sin, step.positions, step.token_seq, table,
+                                k_cache, v_cache, n_q, n_kv, d, pos.rotary_dim, cache.writes,
+                                interleaved=pos.interleaved)
+        else:
+            # The encoding applies itself: project, let it transform q and k where they lie,
+            # then write keys and values to the cache as they are.
+            q = ops.linear(x, w, b)
+            heads_kv = n_kv if cache.writes else 0
+            q_part = q[:, :n_q * d].view(-1, n_q, d)
+            k_part = q[:, n_q * d:(n_q + heads_kv) * d].view(-1, heads_kv, d) if heads_kv else None
+            self.position.apply(q_part, k_part, step.positions)
+            ops.rope_kv_write(q, None, None, step.positions, step.token_seq, table, k_cache,
+                              v_cache, n_q, heads_kv, d, 0, cache.writes)
         attended = ops.attention(q, q.shape[1], cache.k, cache.v, step, table, n_q, n_kv, d,
                                  self.scale, self.window)
         if self.b_o is None and ops.wants_partials(attended, self.w_o):

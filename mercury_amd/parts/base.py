@@ -28,6 +28,14 @@ Interfaces
 ``Mixer.cache_spec()`` / ``Mixer.state_spec()``
     what the cache manager must provide: pages of keys and values (all of them or a window),
     and/or a fixed-size state per request.
+``PositionEncoding.describe()`` / ``PositionEncoding.apply(q, k, positions)``
+    how the encoding transforms queries and keys: as a :class:`PositionDescriptor` the
+    kernels apply themselves (fused into the projection where they can), or, when `describe`
+    returns None, by the part's own `apply` on the projected q and k.
+``Part.lower(program, ...)``
+    optional: append the part's operations to a step program of the host core, which then
+    launches them without coming back to Python (``csrc/host/program.*``).  A part without
+    `lower` is run through its `forward`; a model may mix both kinds, layer by layer.
 """
 
 from __future__ import annotations
@@ -106,6 +114,19 @@ class LayerCache:
     writes: bool = True
 
 
+@dataclass(frozen=True)
+class PositionDescriptor:
+    """A position encoding as the kernels understand it: the first `rotary_dim` dims of every
+    query and key head are turned by the angle tables `cos` / `sin` ([positions, rotary_dim/2],
+    float32), pair j being dims (j, j + rotary_dim/2) of the head, or (2j, 2j + 1) when
+    `interleaved`.  rotary_dim 0: queries and keys stay as projected."""
+
+    rotary_dim: int = 0
+    cos: torch.Tensor | None = None
+    sin: torch.Tensor | None = None
+    interleaved: bool = False
+
+
 class Part:
     """Base of all parts: declares tensors, receives them."""
 
@@ -124,6 +145,13 @@ class Part:
         """Bytes of weights one step reads from this part (for roofline accounting)."""
         return 0
 
+    # A part that can hand its work to the host core defines
+    #     lower(self, program, ...) -> None
+    # appending its operations to `program`; `lowerable` says whether it does (a part may
+    # decide by its parameters, e.g. an attention whose position encoding applies itself
+    # cannot).
+    lowerable = False
+
 
 class Norm(Part):
     def forward(self, h, out_dtype, rows=None, partials=None):
@@ -132,12 +160,21 @@ class Norm(Part):
 
 class PositionEncoding(Part):
     """Turns absolute positions into a transform of q and k.  `prepare` builds whatever tables
-    the transform needs for positions [0, max_positions)."""
-
-    rotary_dim = 0
+    the transform needs for positions [0, max_positions).  The mixer asks `describe()`; an
+    encoding the kernels cannot express returns None there and transforms q and k itself in
+    `apply`."""
 
     def prepare(self, max_positions: int, device) -> None:
         pass
+
+    def describe(self) -> PositionDescriptor | None:
+        return PositionDescriptor()
+
+    def apply(self, q: torch.Tensor, k: torch.Tensor | None, positions: torch.Tensor) -> None:
+        """Transform, in place, the projected queries q [T, n_q, d] and keys k [T, n_kv, d]
+        (views into one buffer; k is None when the layer reads another layer's keys) of the
+        tokens at `positions` (int32 [T], absolute)."""
+        raise NotImplementedError
 
 
 class Mixer(Part):

@@ -31,6 +31,18 @@ class PreNormBlock(Part):
     def graph_safe(self) -> bool:
         return all(part.graph_safe for _, part in self._children())
 
+    def lowerable_with(self, state) -> bool:
+        """Whether the host core can run the whole layer: every part hands over its work and
+        the mixer keeps no state of its own."""
+        return state is None and all(part.lowerable for _, part in self._children())
+
+    def lower(self, program, cache) -> None:
+        self.norm_mixer.lower(program)
+        self.mixer.lower(program, cache)
+        if self.ffn is not None:
+            self.norm_ffn.lower(program)
+            self.ffn.lower(program)
+
     def param_specs(self) -> dict:
         specs = {}
         for key, part in self._children():

@@ -16,6 +16,7 @@ class GatedMLP(FeedForward):
     ``down_proj``."""
 
     graph_safe = True
+    lowerable = True
 
     def __init__(self, hidden: int, intermediate: int, activation: str = "silu"):
         if activation not in ACTIVATIONS:
@@ -41,6 +42,9 @@ class GatedMLP(FeedForward):
 
     def weight_bytes(self) -> int:
         return sum(t.numel() * t.element_size() for t in (self.w_gate_up, self.w_down))
+
+    def lower(self, program) -> None:
+        program.gated_mlp(self.w_gate_up.data_ptr(), self.w_down.data_ptr(), self.intermediate)
 
     def forward(self, x, step, accum):
         if ops.fuses_gating(x, self.w_gate_up):

@@ -131,6 +131,30 @@ class DecoderModel(Part):
         total += self.head.numel() * self.head.element_size()
         return total
 
+    # ---- as a program of the host core
+
+    def compile(self, caches: dict, states: dict):
+        """The step as a program: embedding, every execution-list entry whose layer hands its
+        work over (the others stay with the caller, as one `host` operation each), final norm
+        and head."""
+        from ..hostcore import core
+
+        if not getattr(self.final_norm, "lowerable", False):
+            return None
+        program = core.Program(ops.dtype_code(self.dtype), self.hidden_size, self.vocab_size)
+        program.embed(self.embedding.data_ptr(), ops.dtype_code(self.embedding.dtype), self.vocab_size)
+        for n, call in enumerate(self.calls):
+            layer = self.layers[call.layer]
+            can = getattr(layer, "lowerable_with", None)
+            if can is not None and can(states.get(call.layer)):
+                layer.lower(program, caches.get(n))
+            else:
+                program.host(n)
+        norm = self.final_norm
+        program.head(norm.weight.data_ptr(), ops.dtype_code(norm.weight.dtype), norm.eps,
+                     self.head.data_ptr())
+        return program
+
     # ---- one step
 
     def forward(self, step, caches: dict, states: dict) -> torch.Tensor:

@@ -17,6 +17,7 @@ class RMSNorm(Norm):
     """
 
     graph_safe = True
+    lowerable = True
 
     def __init__(self, size: int, eps: float):
         self.size = int(size)
@@ -31,6 +32,9 @@ class RMSNorm(Norm):
 
     def forward(self, h, out_dtype, rows=None, partials=None):
         return ops.rmsnorm(h, self.weight, self.eps, out_dtype, rows=rows, partials=partials)
+
+    def lower(self, program) -> None:
+        program.norm(self.weight.data_ptr(), ops.dtype_code(self.weight.dtype), self.eps)
 
     def weight_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()

@@ -4,12 +4,13 @@ from __future__ import annotations
 
 import torch
 
-from .base import PositionEncoding
+from .base import PositionDescriptor, PositionEncoding
 
 
 class RotaryPosition(PositionEncoding):
-    """Rotary encoding in the half-split layout: dims j and j + rotary_dim/2 of a head form a
-    pair that is turned by the angle position * theta^(-2j/rotary_dim).
+    """Rotary encoding: dims j and j + rotary_dim/2 of a head (the half-split layout; with
+    `interleaved`, dims 2j and 2j + 1) form a pair that is turned by the angle
+    position * theta^(-2j/rotary_dim).
 
     The angle table is built as the reference builds it (mercury/model/rope.py:37-47):
     inverse frequencies, positions and their outer product in float32, then cos and sin.
@@ -18,9 +19,11 @@ class RotaryPosition(PositionEncoding):
     within the sequence, so keys can be cached after rotation.
     """
 
-    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None):
+    def __init__(self, head_dim: int, theta: float, rotary_dim: int | None = None,
+                 interleaved: bool = False):
         self.head_dim = int(head_dim)
         self.theta = float(theta)
+        self.interleaved = bool(interleaved)
         self.rotary_dim = int(head_dim if rotary_dim is None else rotary_dim)
         if self.rotary_dim % 2 or not 0 < self.rotary_dim <= self.head_dim:
             raise ValueError(f"rotary width {self.rotary_dim} must be even and within the head")
@@ -38,10 +41,12 @@ class RotaryPosition(PositionEncoding):
         self.cos = angles.cos().contiguous().to(device)
         self.sin = angles.sin().contiguous().to(device)
 
+    def describe(self) -> PositionDescriptor:
+        return PositionDescriptor(self.rotary_dim, self.cos, self.sin, self.interleaved)
+
 
 class NoPosition(PositionEncoding):
     """Queries and keys are used as projected."""
 
-    rotary_dim = 0
-    cos = None
-    sin = None
+    def describe(self) -> PositionDescriptor:
+        return PositionDescriptor()

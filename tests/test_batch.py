@@ -5,12 +5,23 @@ from __future__ import annotations
 import pytest
 
 from mercury_amd.cache import CacheManager
-from mercury_amd.engine.batch import BatchError, SeqChunk, context_from_packed, pack_step
+from mercury_amd.engine.batch import BatchError, SeqChunk, context_from_packed, host_ints
+from mercury_amd.hostcore import core
 from mercury_amd.parts import CacheSpec
 
 PS = 8
 FULL = CacheSpec(kv_heads=2, head_dim=16, window=None)
 WINDOW = CacheSpec(kv_heads=2, head_dim=16, window=20)
+
+
+def pack_step(chunks, manager, vocab_size, max_positions, pinned=False, table_width=-1):
+    """Pack on the host alone (no GPU here): pageable memory, no program, no tile lists."""
+    packer = core.StepPacker(manager, vocab_size, max_positions, pinned=pinned)
+    return packer.pack(chunks, None, table_width)
+
+
+def context(packed):
+    return context_from_packed(packed, host_ints(packed))
 
 
 def manager_with(requests: dict, slots=None) -> CacheManager:
@@ -27,7 +38,7 @@ def test_a_mixed_step_is_laid_out_by_sequence():
               SeqChunk("b", [9], 8, [0]),                # a decoded token
               SeqChunk("c", [1, 2, 3], 0, [])]           # a whole prompt, nothing wanted
     packed = pack_step(chunks, m, 100, 64, pinned=False)
-    step = context_from_packed(packed, packed.host)
+    step = context(packed)
     assert step.token_ids.tolist() == [5, 6, 7, 9, 1, 2, 3]
     assert step.positions.tolist() == [18, 19, 20, 8, 0, 1, 2]
     assert step.token_seq.tolist() == [0, 0, 0, 1, 2, 2, 2]
@@ -44,7 +55,7 @@ def test_a_mixed_step_is_laid_out_by_sequence():
     assert table[1].tolist() == m.table("b", 0) + [-1]
     assert table[2].tolist() == m.table("c", 0) + [-1, -1]
     wide = pack_step(chunks, m, 100, 64, pinned=False, table_width=6)
-    assert context_from_packed(wide, wide.host).block_tables[0].shape == (3, 6)
+    assert context(wide).block_tables[0].shape == (3, 6)
     assert packed.layout() != wide.layout()
 
 
@@ -52,7 +63,7 @@ def test_every_group_has_a_table_of_its_own():
     m = manager_with({"a": 40}, {0: FULL, 1: WINDOW})
     m.trim("a", 40)                                       # the window gives its first pages back
     packed = pack_step([SeqChunk("a", [1], 39, [0])], m, 100, 64, pinned=False)
-    step = context_from_packed(packed, packed.host)
+    step = context(packed)
     full, window = step.block_tables
     assert full[0].tolist() == m.table("a", 0) and min(full[0].tolist()) >= 0
     assert window[0].tolist() == m.table("a", 1) and window[0, 0] == -1
@@ -64,6 +75,7 @@ def test_every_group_has_a_table_of_its_own():
     ([SeqChunk("a", [100], 0, [])], "token id"),
     ([SeqChunk("a", [-1], 0, [])], "token id"),
     ([SeqChunk("a", [1, 2], 0, [2])], "wanted index"),
+    ([SeqChunk("a", [1, 2], 0, [1, 1])], "twice"),
     ([SeqChunk("a", [1], 64, [])], "limit"),
     ([SeqChunk("a", [1] * 30, 0, [])], "pages"),          # more tokens than the request holds pages for
 ])

@@ -456,3 +456,162 @@ def test_routed_feed_forward_and_other_position_encodings(tmp_path):
     assert torch.isfinite(got).all()
     error = (got[:safe] - want16[:safe]).abs().max()
     assert float(error) <= BF16_SLACK * cost, (float(error), cost, safe)
+
+
+# ------------------------------------------------------- position encodings from outside
+
+
+def register_position_toys():
+    from mercury_amd.config import Qwen2Config, register_architecture
+    from mercury_amd.parts import (Attention, DecoderModel, GatedMLP, PositionDescriptor,
+                                   PositionEncoding, PreNormBlock, RMSNorm, TensorSpec,
+                                   register_position)
+
+    @register_position("test_interleaved_rotary")
+    class InterleavedRotary(PositionEncoding):
+        """Rotary encoding that pairs dims (2j, 2j + 1) of a head: it only describes itself
+        (tables and layout); the kernels do the turning."""
+
+        def __init__(self, head_dim, theta):
+            self.head_dim, self.theta = head_dim, theta
+            self.cos = self.sin = None
+
+        def prepare(self, max_positions, device):
+            inv = 1.0 / (self.theta ** (torch.arange(0, self.head_dim, 2, dtype=torch.float32) / self.head_dim))
+            angles = torch.outer(torch.arange(max_positions, dtype=torch.float32), inv)
+            self.cos, self.sin = angles.cos().to(device), angles.sin().to(device)
+
+        def describe(self):
+            return PositionDescriptor(self.head_dim, self.cos, self.sin, interleaved=True)
+
+    @register_position("test_added_positions")
+    class AddedPositions(PositionEncoding):
+        """A stored vector per position added to every query and key head: nothing the
+        kernels know, so it describes nothing and applies itself."""
+
+        def __init__(self, head_dim, positions):
+            self.head_dim, self.positions = head_dim, positions
+            self.table = None
+
+        def param_specs(self):
+            return {"table": TensorSpec((self.positions, self.head_dim))}
+
+        def bind(self, params, dtype, device):
+            self.table = params["table"]
+
+        def describe(self):
+            return None
+
+        def apply(self, q, k, positions):
+            rows = self.table[positions.long()][:, None, :]
+            q += rows
+            if k is not None:
+                k += rows
+
+    class PositionedAttention(Attention):
+        """Attention whose position encoding brings tensors of its own."""
+
+        def param_specs(self):
+            specs = super().param_specs()
+            specs.update({"position." + n: s for n, s in self.position.param_specs().items()})
+            return specs
+
+        def bind(self, params, dtype, device):
+            super().bind(params, dtype, device)
+            self.position.bind({n[len("position."):]: t for n, t in params.items()
+                                if n.startswith("position.")}, dtype, device)
+
+    names = {"mixer": "mixer.", "ffn": "mlp.", "norm_mixer": "norm1.", "norm_ffn": "norm2."}
+
+    @register_architecture("TestPositionsLM", Qwen2Config)
+    def build(cfg):
+        h, eps, d = cfg.hidden_size, cfg.rms_norm_eps, cfg.head_dim
+        positions = [InterleavedRotary(d, cfg.rope_theta), AddedPositions(d, 128)]
+        layers = [PreNormBlock(PositionedAttention(h, cfg.num_attention_heads,
+                                                   cfg.num_key_value_heads, d, pos, qkv_bias=True),
+                               GatedMLP(h, cfg.intermediate_size), RMSNorm(h, eps), RMSNorm(h, eps),
+                               names) for pos in positions]
+        return DecoderModel(cfg.vocab_size, h, layers, RMSNorm(h, eps), tied_head=True,
+                            layer_prefix="layers.{}.", embed_name="embed.weight",
+                            norm_prefix="norm.", max_positions=128, config=cfg)
+
+    return build
+
+
+def plain_positions_logits(w, cfg, tokens):
+    eps, d = cfg["rms_norm_eps"], cfg["head_dim"]
+    n_q, n_kv = cfg["num_attention_heads"], cfg["num_key_value_heads"]
+    t = len(tokens)
+    h = w["embed.weight"][torch.tensor(tokens)]
+    inv = 1.0 / (cfg["rope_theta"] ** (torch.arange(0, d, 2, dtype=torch.float32) / d))
+    angles = torch.outer(torch.arange(t, dtype=torch.float32), inv)[:, None, :]
+
+    def interleaved(x):
+        even, odd = x[..., 0::2], x[..., 1::2]
+        out = torch.empty_like(x)
+        out[..., 0::2] = even * angles.cos() - odd * angles.sin()
+        out[..., 1::2] = odd * angles.cos() + even * angles.sin()
+        return out
+
+    for i in range(2):
+        p = f"layers.{i}."
+        x = plain.rms_norm(h, w[p + "norm1.weight"], eps)[0]
+        q = (x @ w[p + "mixer.q_proj.weight"].T + w[p + "mixer.q_proj.bias"]).view(t, n_q, d)
+        k = (x @ w[p + "mixer.k_proj.weight"].T + w[p + "mixer.k_proj.bias"]).view(t, n_kv, d)
+        v = (x @ w[p + "mixer.v_proj.weight"].T + w[p + "mixer.v_proj.bias"]).view(t, n_kv, d)
+        if i == 0:
+            q, k = interleaved(q), interleaved(k)
+        else:
+            rows = w[p + "mixer.position.table"][:t, None, :]
+            q, k = q + rows, k + rows
+        h = h + plain.causal_attention(q, k, v, d ** -0.5).reshape(t, -1) @ w[p + "mixer.o_proj.weight"].T
+        x = plain.rms_norm(h, w[p + "norm2.weight"], eps)[0]
+        h = h + plain.gated_mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                                w[p + "mlp.down_proj.weight"])
+    return plain.rms_norm(h, w["norm.weight"], eps)[0] @ w["embed.weight"].T
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_position_encodings_registered_from_outside(tmp_path, dtype):
+    """Two position encodings the package does not have, defined here: a rotary in the
+    interleaved pair layout, which only describes itself to the kernels (the host core runs
+    its layer), and a stored vector per position added to queries and keys, which applies
+    itself (its layer is run from Python between the host core's).  Whole, in portions and
+    token by token."""
+    from mercury_amd.engine.replay import ReplaySession
+    from mercury_amd.weights import write_random_model
+    from safetensors.torch import load_file
+    from tests.test_gpu_replay import BF16_SLACK
+
+    register_position_toys()
+    config = {**helpers.TINY_A, "architectures": ["TestPositionsLM"], "hidden_size": 64,
+              "head_dim": 32, "num_attention_heads": 4, "num_key_value_heads": 2,
+              "intermediate_size": 96, "max_position_embeddings": 128}
+    folder = write_random_model(tmp_path / "positions", config, seed=5, std=0.1, dtype=torch.bfloat16)
+    w = {k: v.float() for k, v in load_file(str(folder / "model.safetensors")).items()}
+    cfg = plain.read_config(folder)
+    tokens = helpers.random_tokens(512, 75, 9)
+    want = plain_positions_logits(w, cfg, tokens)
+    # the encodings matter: with neither, the logits are others
+    moved = plain_positions_logits(w, cfg, tokens[1:])
+    assert (moved[:-1] - want[1:-1]).abs().max() > 1e-2
+
+    s = ReplaySession(folder, dtype, 256)
+    kinds = s.runner.program.kinds
+    assert kinds.count("host") == 1 and kinds.count("attention") == 1
+    if dtype == "float32":
+        check = lambda got: torch.testing.assert_close(got, want, atol=2e-5, rtol=1e-4)
+    else:
+        w16 = {k: v.to(torch.bfloat16) for k, v in w.items()}
+        cost = float((plain_positions_logits(w16, cfg, tokens).float() - want).abs().max())
+        check = lambda got: float((got - want).abs().max()) <= BF16_SLACK * cost or pytest.fail(
+            f"bfloat16 error {float((got - want).abs().max()):.3e} against a cost of {cost:.3e}")
+    check(s.step([{"id": "w", "tokens": tokens, "want": list(range(75))}], ["w"]))
+    parts, at = [], 0
+    for size in (20, 2, 17, 1, 1, 30, 4):
+        part = tokens[at:at + size]
+        parts.append(s.step([{"id": "p", "tokens": part, "want": list(range(size))}],
+                            ["p"] if at + size == 75 else []))
+        at += size
+    check(torch.cat(parts))
+    assert s.manager.leaked_pages() == 0
