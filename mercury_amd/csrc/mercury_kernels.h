@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 10
+#define MK_ABI_VERSION 11
 
 #ifdef __cplusplus
 extern "C" {
@@ -158,6 +158,16 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
 // are searched by 64 workgroups per row.
 int mk_argmax(const float* logits, int rows, int vocab, long long row_stride, int* out,
               void* parts, hipStream_t stream);
+
+// mk_argmax without a buffer of the caller's, and without any allocation: the partial results
+// live in a device array inside the library (one per GPU, kept until the process ends), of
+// mk_argmax_static_max_rows() rows; more rows are refused.  This entry point has no
+// counterpart in the reference: it is for callers that cannot allocate (code under HIP graph
+// capture, serving loops and harnesses that forbid hipMalloc).  Calls that overlap on one GPU
+// share the array and race; calls on one stream, one after the other, are safe.
+int mk_argmax_static_max_rows(void);
+int mk_argmax_static(const float* logits, int rows, int vocab, long long row_stride, int* out,
+                     hipStream_t stream);
 
 // One token per row: the argmax where temperature <= 0, else an inverse-CDF draw with the
 // row's uniform number from softmax(logits / temperature) restricted to the nucleus top_p

@@ -101,6 +101,54 @@ extern "C" int mk_argmax(const float* logits, int rows, int vocab, long long row
   return 0;
 }
 
+// ------------------------------------------------------ argmax for callers that cannot allocate
+//
+// The two-stage search above needs rows * 64 partial results between its kernels.  Here they
+// live in a device array of the library's own instead of a buffer the caller brings, so that
+// a caller under graph capture, or one that may not allocate at all, has a variant that
+// allocates nothing.  The array's name is a host-side stand-in in host code: its device
+// address is asked for once per device (with that device current) and kept; only that address
+// is ever handed to a kernel.  Nothing in the array has to start at zero: each call's first
+// kernel writes every part that its second kernel reads.  Every call on a GPU uses that GPU's
+// one array, so two calls that overlap on one GPU (different streams) race.
+#define ARGMAX_STATIC_MAX_ROWS 256
+static __device__ __align__(256) unsigned char
+    argmax_static_scratch[ARGMAX_STATIC_MAX_ROWS * ARGMAX_PARTS * sizeof(MaxIdx)];
+
+#define ARGMAX_STATIC_MAX_DEVICES 64
+static void* g_argmax_scratch_of_device[ARGMAX_STATIC_MAX_DEVICES];
+
+extern "C" int mk_argmax_static_max_rows(void) { return ARGMAX_STATIC_MAX_ROWS; }
+
+extern "C" int mk_argmax_static(const float* logits, int rows, int vocab, long long row_stride,
+                                int* out, hipStream_t stream) {
+  MK_REQUIRE(rows >= 0 && vocab > 0 && row_stride >= vocab, "argmax_static: bad sizes");
+  MK_REQUIRE(rows <= ARGMAX_STATIC_MAX_ROWS,
+             "argmax_static: %d rows; the library's own scratch holds at most %d (use mk_argmax "
+             "with a buffer of the caller's)", rows, ARGMAX_STATIC_MAX_ROWS);
+  if (rows == 0) return 0;
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  MK_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+  MK_REQUIRE(device >= 0 && device < ARGMAX_STATIC_MAX_DEVICES, "argmax_static: device %d", device);
+  void* scratch = g_argmax_scratch_of_device[device];
+  if (scratch == nullptr) {
+    e = hipGetSymbolAddress(&scratch, HIP_SYMBOL(argmax_static_scratch));
+    MK_REQUIRE(e == hipSuccess && scratch != nullptr, "argmax_static: hipGetSymbolAddress: %s",
+               hipGetErrorString(e));
+    g_argmax_scratch_of_device[device] = scratch;
+  }
+  if (vocab >= 16384) {
+    argmax_part_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, stream>>>(logits, vocab, row_stride,
+                                                                      (MaxIdx*)scratch);
+    argmax_pick_kernel<<<rows, MK_WAVE, 0, stream>>>((const MaxIdx*)scratch, out);
+  } else {
+    argmax_kernel<<<rows, SP_THREADS, 0, stream>>>(logits, vocab, row_stride, out);
+  }
+  MK_LAUNCH_CHECK("argmax_static");
+  return 0;
+}
+
 // ------------------------------------------------------------- sampling without a nucleus
 //
 // When no row restricts the nucleus (top_p >= 1) the draw needs no threshold search, and the

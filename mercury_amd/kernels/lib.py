@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 from . import build
 
-ABI_VERSION = 10
+ABI_VERSION = 11
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -26,6 +26,8 @@ _SIGNATURES = {
         "mk_attention_generic": [P, I, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
         "mk_qkv_finish": [P, I, L, P, I, P, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
         "mk_argmax": [P, I, I, L, P, P, P],
+        "mk_argmax_static_max_rows": [],
+        "mk_argmax_static": [P, I, I, L, P, P],
         "mk_sample_scratch_bytes": [I, I],
         "mk_sample": [P, I, I, L, P, P, P, P, P, P],
         "mk_fill_normal": [P, I, L, c_ulonglong, F, F, P],
