@@ -8,7 +8,10 @@ random token ids, a batch of 8 and a context that reaches 4,096 tokens at the la
 One JSON line is printed: `value` is decoded tokens per second; `prefill` times one 2,048-token
 prompt as one step; `roofline` divides the bytes a decode step has to read (every weight it
 uses once, and the cache of the live requests) by its time and by the HBM peak; `points`
-holds decode throughput at batch 1 and 64.
+holds decode throughput at batch 1 and 64 and, at the default batch, at half the context.
+Beside the published peaks both fractions are also given against what this machine reaches in
+the same run: a streaming read of a 2 GiB matrix by the engine's one-row projection, and a
+8192 x 8192 x 8192 bfloat16 product by its tiled matrix-core kernel (`measured`).
 
     python bench.py --shape 32b --serve
 
@@ -166,8 +169,46 @@ class Bench:
         self.engine._drain_commands()
         assert self.engine.leaked_blocks() == 0
         ms = 1e3 * elapsed / steps
-        return {"tok_s": batch * steps / elapsed, "ms": ms, "fill_s": fill_s,
+        timed = self.engine.metrics.step_records()[-steps:]
+        device_ms = 1e3 * sum(r.device_s for r in timed) / steps
+        return {"tok_s": batch * steps / elapsed, "ms": ms, "fill_s": fill_s, "device_ms": device_ms,
                 "prompt_len": prompt_len, "bytes": self.model.decode_weight_bytes() + kv_bytes}
+
+    def measured_peaks(self) -> dict:
+        """What this machine reaches, by the engine's own kernels: GB/s of a streaming read
+        (a 2 GiB matrix times one row, the projection every decode step is made of) and
+        FLOP/s of a large bfloat16 product (8192 x 8192 x 8192 through the tiled matrix-core
+        kernel)."""
+        torch = self.torch
+        from mercury_amd.kernels import ops
+
+        def best(fn, repeats=5):
+            fn()
+            times = []
+            for _ in range(repeats):
+                start, stop = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                start.record()
+                fn()
+                stop.record()
+                stop.synchronize()
+                times.append(1e-3 * start.elapsed_time(stop))
+            return min(times)
+
+        dtype = torch.bfloat16 if self.engine_cfg.dtype == "bfloat16" else torch.float32
+        rows = (1 << 31) // (4096 * torch.empty((), dtype=dtype).element_size())
+        big = torch.empty((rows, 4096), dtype=dtype, device="cuda:0").normal_()
+        one = torch.empty((1, 4096), dtype=dtype, device="cuda:0").normal_()
+        read_s = best(lambda: ops.linear(one, big, out_dtype=torch.float32))
+        gbs = big.numel() * big.element_size() / read_s / 1e9
+        del big
+        out = {"hbm_read_gbs": round(gbs, 1)}
+        if self.engine_cfg.dtype == "bfloat16":
+            n = 8192
+            a = torch.empty((n, n), dtype=torch.bfloat16, device="cuda:0").normal_()
+            b = torch.empty((n, n), dtype=torch.bfloat16, device="cuda:0").normal_()
+            gemm_s = best(lambda: ops.linear(a, b))
+            out["gemm_flops"] = round(2.0 * n ** 3 / gemm_s, -9)
+        return out
 
     def prefill(self, tokens: int, repeats: int = 5) -> dict:
         from mercury_amd import SamplingParams
@@ -284,6 +325,10 @@ def main(argv=None) -> int:
     print(f"[bench] prefill {PREFILL_TOKENS}: {pre['ms']:.2f} ms", file=sys.stderr, flush=True)
     points = {}
     if not args.no_points:
+        half = bench.decode(args.batch, args.context // 2, max(8, args.steps // 2), min(args.warmup, 4))
+        points[f"decode_b{args.batch}_ctx{args.context // 2}"] = round(half["tok_s"], 1)
+        print(f"[bench] decode b{args.batch} at context {args.context // 2}: {half['ms']:.3f} ms/step",
+              file=sys.stderr, flush=True)
         for b in (1, 64):
             steps = max(8, args.steps // 2)
             run = bench.decode(b, args.context, steps, min(args.warmup, 4))
@@ -292,6 +337,9 @@ def main(argv=None) -> int:
 
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     achieved = main_run["bytes"] / (main_run["ms"] * 1e-3) / 1e9
+    peaks = bench.measured_peaks()
+    print(f"[bench] this machine: {peaks}", file=sys.stderr, flush=True)
+    prefill_rate = prefill_flops(cfg, PREFILL_TOKENS) / (pre["ms"] * 1e-3)
     line = {
         "metric": f"decode tok/s at batch {args.batch}, context {args.context} ({model_name} shapes)",
         "value": round(main_run["tok_s"], 1),
@@ -300,6 +348,7 @@ def main(argv=None) -> int:
         "steps": args.steps,
         "warmup": args.warmup,
         "ms_per_step": round(main_run["ms"], 4),
+        "device_ms_per_step": round(main_run["device_ms"], 4),
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
@@ -317,10 +366,14 @@ def main(argv=None) -> int:
         },
         "prefill": {"value": round(pre["tok_s"], 1), "tokens": PREFILL_TOKENS,
                     "ms": round(pre["ms"], 3),
-                    "frac": round(prefill_flops(cfg, PREFILL_TOKENS) / (pre["ms"] * 1e-3)
-                                  / PEAK_FLOPS[short], 5)},
+                    "frac": round(prefill_rate / PEAK_FLOPS[short], 5),
+                    "measured_peak": peaks.get("gemm_flops"),
+                    "frac_of_measured": (round(prefill_rate / peaks["gemm_flops"], 5)
+                                         if peaks.get("gemm_flops") else None)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": PEAK_HBM_GBS,
-                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 5)},
+                     "unit": "GB/s", "frac": round(achieved / PEAK_HBM_GBS, 5),
+                     "measured_peak": peaks["hbm_read_gbs"],
+                     "frac_of_measured": round(achieved / peaks["hbm_read_gbs"], 5)},
         "points": points,
     }
     print(json.dumps(line), flush=True)
