@@ -598,6 +598,370 @@ __global__ __launch_bounds__(64 * ATTN_WAVES * KG, (RT == 1 ? (KG > 2 ? KG : 2) 
   }
 }
 
+// ------------------------------------------------------- prompts in tiles of 32 rows by 64 keys
+//
+// The same work as the kernel above with the products v_mfma_f32_32x32x16_bf16: a wavefront
+// owns 32 rows, four wavefronts 128 consecutive rows of one sequence and one kv head, and a
+// block is 64 keys.  With a query per lane (lane l: row l % 32; the two halves of the
+// wavefront hold different keys of it) the maximum and the sum over a block's keys are
+// sixteen values deep in a lane's own registers per sub-block of 32 keys, one exchange
+// between the halves apart; per score there is the least left to do beside the products: one
+// maximum, one fused multiply-add, one exponential, one addition, half a conversion.
+//
+//   S^T[key, row]  = K[key, :] . Q[row, :]     A = K (32 keys x 16 dims), B = Q^T (16 x 32 rows)
+//   O^T[dim, row] += V^T[dim, key] P^T[key, row]   A = V^T (32 dims x 16 keys), B = P^T
+//
+// A lane's sixteen scores of a sub-block are keys 8 (i / 4) + 4 (l / 32) + i % 4; the second
+// product's step s takes its registers 8 s .. 8 s + 7, which are keys 16 s + 4 (l / 32) +
+// {0..3, 8..11}: the lane's operand of values is two 8-byte pieces of a dim's row of keys.
+//
+// Keys and values travel from the cache straight into LDS (global_load_lds_dwordx4: a
+// wavefront's 64 x 16 bytes land side by side, no register in between), into a ring of
+// buffers filled several blocks ahead of their use; a workgroup whose rows see few blocks has
+// them all in flight at once, one whose rows see many never waits for the cache's latency.
+// Per buffer: keys [64][D], the 16-byte chunks of a key's row permuted by the key's number
+// against bank conflicts (by permuting which chunk each lane fetches); values [8 pieces of 8
+// keys][D dims][8 keys], which the operand reads cover without conflicts as they lie.
+//
+// KG groups of four wavefronts may share a workgroup's rows, taking the key blocks in turn
+// with rings of their own; their running maxima, sums and weighted values are combined
+// through LDS in group order at the end (a short prompt's longest chain of blocks is cut
+// into KG chains side by side).
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
+
+template <int D>
+__device__ __forceinline__ int wide_key_offset(int key, int chunk) {   // in 16-byte units
+  constexpr int CH = D / 8;
+  return key * CH + (chunk & ~7) + ((chunk ^ key) & 7);
+}
+
+// The loads of one block by one wavefront (D / 16 instructions), into the ring buffer at
+// LDS byte address `dst`.  Instruction j < D / 32 brings keys: 1024 bytes are 1024 / (2 D)
+// keys' rows; instruction j >= D / 32 brings values: 64 dims of one piece of 8 keys.  Keys
+// outside what the workgroup's rows see (or past the group's last block) are fetched from
+// page 0, which always exists, and masked in the scores.
+// What a lane adds to the wavefront's address of a load, the same for every block.
+struct WideLane {
+  uint32_t k_at, v_at;   // bytes
+};
+
+template <int D>
+__device__ __forceinline__ WideLane wide_lane(int page_size, int lane, int wave) {
+  constexpr int KEYS_PER_LOAD = 512 / D, CH = D / 8;
+  const int key = wave * KEYS_PER_LOAD + lane / CH;      // of load j = 0; load j is 4 j loads on
+  const int slot = lane % CH;
+  const int chunk = (slot & ~7) | ((slot ^ key) & 7);    // the chunk that lies at the lane's slot
+  const int dim = ((wave % (D / 64)) * 64 + lane) % D;
+  WideLane out;
+  out.k_at = (uint32_t)(key & 15) * (uint32_t)(D * 2) + (uint32_t)chunk * 16u;
+  out.v_at = (uint32_t)dim * (uint32_t)(page_size * 2);
+  return out;
+}
+
+// The loads of one block by one wavefront, D / 32 of keys and as many of values, into the
+// ring buffer at LDS byte address `dst`.  Load j of the keys brings 1024 bytes of rows
+// (8 keys at D = 64, 4 at D = 128), load j of the values 64 dims of one piece of 8 keys; both
+// lie in the stretch of 16 keys number (wave / 2) + 2 j (D = 64) or j (D = 128) of the
+// block, so the page is looked up once for the pair, everything but the lane's own offset is
+// the wavefront's (scalar) arithmetic, and the load takes that base and a 32-bit offset.
+// Keys outside what the workgroup's rows see (or past the group's last block) are fetched
+// from page 0, which always exists, and masked in the scores.
+template <int D>
+__device__ __forceinline__ void wide_fetch(const AttnParams& p, TableWindow& tw, int b, int b_end,
+                                           int kmin, int kmax, int kvh, int lane, int wave,
+                                           unsigned int dst, const WideLane& mine) {
+  constexpr int KEYS_PER_LOAD = 512 / D;
+  const int ps = 1 << p.page_shift;
+  const uint32_t head_bytes = (uint32_t)ps * D * 2;
+  const uint32_t page_bytes = head_bytes * (uint32_t)p.n_kv;
+  const uint32_t head_at = (uint32_t)kvh * head_bytes;
+  auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+#pragma unroll
+  for (int j = 0; j < D / 32; ++j) {
+    const int load = wave + 4 * j;
+    const int stretch = (load * KEYS_PER_LOAD) >> 4;       // 16 keys, within one page
+    const int piece = load / (D / 64);                      // the values' piece of 8 keys
+    const int kh = uniform((b << 6) + stretch * 16);
+    const int live = uniform(b < b_end && kh <= kmax && kh + 15 >= kmin);
+    const int index = kh >> p.page_shift;
+    if (live && uniform(index >= tw.base + 64)) {           // once in 64 pages
+      tw.base = index;
+      tw.mine = index + lane < tw.width ? tw.table[index + lane] : 0;
+      __builtin_amdgcn_s_waitcnt(0x0F70);                    // vmcnt(0): before the readlane below
+    }
+    const int page = live ? __builtin_amdgcn_readlane(tw.mine, uniform(index - tw.base)) : 0;
+    const uint64_t page_at = (uint64_t)(uint32_t)page * page_bytes + head_at;
+    const uint32_t off = (uint32_t)(kh & (ps - 1));
+    const char* k_from = (const char*)p.k_cache + page_at + off * (uint32_t)(D * 2);
+    const char* v_from = (const char*)p.v_cache + page_at + (off + (uint32_t)(piece & 1) * 8u) * 2u;
+    const unsigned int k_to = dst + (unsigned int)load * 1024u;
+    const unsigned int v_to = dst + (unsigned int)(64 * D * 2) + (unsigned int)load * 1024u;
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 : : "s"(k_to), "v"(mine.k_at), "s"(k_from) : "memory");
+    asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
+                 : : "s"(v_to), "v"(mine.v_at), "s"(v_from) : "memory");
+  }
+}
+
+// NSUB sub-blocks of 32 keys (from `sub0` of the block in LDS) against a wavefront's 32
+// rows: scores, one round of the online softmax over all of them, weighted values.
+template <int D, int NSUB, bool MASKED>
+__device__ __forceinline__ void wide_block(const Frag (&qf)[D / 16], f32x16 (&acc)[D / 32], float& m,
+                                           float& lsum, const uint4* lds_k, const uint2* lds_v,
+                                           int key0, int sub0, float c, int n, int hh, bool row_ok,
+                                           int pos, int lo) {
+  // All of the keys' operands are asked for before the first product, and the values'
+  // before the softmax, whose arithmetic then hides their way out of LDS.
+  Frag kf[NSUB][D / 16];
+#pragma unroll
+  for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+    for (int k = 0; k < D / 16; ++k)
+      kf[u][k].u = lds_k[wide_key_offset<D>((sub0 + u) * 32 + n, k * 2 + hh)];
+  f32x16 sc[NSUB];
+#pragma unroll
+  for (int u = 0; u < NSUB; ++u) {
+#pragma unroll
+    for (int i = 0; i < 16; ++i) sc[u][i] = 0.f;
+#pragma unroll
+    for (int k = 0; k < D / 16; ++k)
+      sc[u] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(kf[u][k].v, qf[k].v, sc[u], 0, 0, 0);
+  }
+  // values [piece][dim][8 keys]: the lane's two pieces of four keys for step s of sub-block u
+  // are bytes 8 hh .. + 8 of pieces 4 u + 2 s and 4 u + 2 s + 1 of its dim.
+  Frag vf[D / 32][NSUB][2];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+      for (int s2 = 0; s2 < 2; ++s2) {
+        const int piece = (sub0 + u) * 4 + s2 * 2;
+        vf[db][u][s2].u2[0] = lds_v[((piece * D) + db * 32 + n) * 2 + hh];
+        vf[db][u][s2].u2[1] = lds_v[(((piece + 1) * D) + db * 32 + n) * 2 + hh];
+      }
+  if (MASKED) {
+#pragma unroll
+    for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) {
+        const int key = key0 + (sub0 + u) * 32 + 8 * (i >> 2) + 4 * hh + (i & 3);
+        const bool ok = row_ok && key <= pos && key >= lo;
+        sc[u][i] = ok ? sc[u][i] : -INFINITY;
+      }
+  }
+  float bm = sc[0][0];
+#pragma unroll
+  for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+    for (int i = (u == 0 ? 1 : 0); i < 16; ++i) bm = fmaxf(bm, sc[u][i]);
+  bm *= c;     // the largest raw score is the largest scaled one (c > 0)
+  // The two lanes of a row exchange their maxima and the row's maximum moves only when some
+  // lane of the wavefront saw a score above its row's; what is accumulated is multiplied
+  // either way (by one when nothing moved): a multiplication under a branch would have the
+  // accumulators copied around it, which costs more than the multiplications.
+  float corr = 1.f;
+  if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+    bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
+    const float m_new = fmaxf(m, bm);
+    corr = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
+    m = m_new;
+  }
+  lsum *= corr;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] *= corr;
+  const float m_use = (MASKED && m == -INFINITY) ? 0.f : m;
+  Frag pf[NSUB][2];
+  float part = 0.f;
+#pragma unroll
+  for (int u = 0; u < NSUB; ++u) {
+    float e[16];
+#pragma unroll
+    for (int i = 0; i < 16; ++i) e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[u][i], c, -m_use));
+    part += (((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]))) +
+            (((e[8] + e[9]) + (e[10] + e[11])) + ((e[12] + e[13]) + (e[14] + e[15])));
+#pragma unroll
+    for (int s = 0; s < 2; ++s)
+      pf[u][s].u = make_uint4(pack_bf16x2(e[8 * s], e[8 * s + 1]), pack_bf16x2(e[8 * s + 2], e[8 * s + 3]),
+                              pack_bf16x2(e[8 * s + 4], e[8 * s + 5]), pack_bf16x2(e[8 * s + 6], e[8 * s + 7]));
+  }
+  lsum += part;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+      for (int s = 0; s < 2; ++s)
+        acc[db] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(vf[db][u][s].v, pf[u][s].v, acc[db], 0, 0, 0);
+}
+
+// s_waitcnt immediate: at most `loads` vector-memory loads outstanding (vmcnt is split over
+// bits 3:0 and 15:14; the other counters are left alone).
+#define WIDE_WAIT(loads) (((loads) & 15) | (((loads) >> 4) << 14) | (7 << 4) | (15 << 8))
+
+template <int D, int KG, int NB>
+__global__ __launch_bounds__(256 * KG, (KG == 1 && NB * D <= 256) ? 2 : 1) void attn_wide_kernel(AttnParams p) {
+  constexpr int BUFFER = 2 * 64 * D * 2;                   // bytes of a block's keys and values
+  constexpr int LOADS = D / 16;                            // load instructions per wavefront and block
+  constexpr int MERGE = D / 2 + 2;                         // floats a thread hands over
+  static_assert(KG == 1 || (KG - 1) * MERGE * 256 * 4 <= KG * NB * BUFFER, "merge space fits the rings");
+  static_assert((NB - 1) * LOADS < 64, "the loads in flight fit the counter");
+  __shared__ __attribute__((aligned(1024))) unsigned char lds[KG * NB * BUFFER];
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3;
+  const int kgroup = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
+  const int wave_u = __builtin_amdgcn_readfirstlane(wave);
+  unsigned char* const ring = lds + kgroup * (NB * BUFFER);
+  const unsigned int ring_at = (unsigned int)(uintptr_t)(__attribute__((address_space(3))) void*)ring;
+  const int n = lane & 31, hh = lane >> 5;
+  const int tile = p.num_tiles - 1 - (int)blockIdx.x;     // the longest work first
+  const int kvh = blockIdx.y;
+  const int seq = p.tile_seq[tile];
+  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  const int pos0 = p.kv_len[seq] - q_len;
+  const int G = p.group;
+  const int rows_total = q_len * G;
+  const int wg_row0 = p.tile_row0[tile];
+  const int row0 = wg_row0 + wave * 32;
+  const bool wave_has_rows = row0 < rows_total;
+
+  const int flat = row0 + n;
+  const bool row_ok = flat < rows_total;
+  const int tok = row_ok ? flat / G : 0;
+  const int head = kvh * G + (row_ok ? flat % G : 0);
+  const int pos = pos0 + tok;
+  const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
+
+  const int wg_last = min(wg_row0 + 127, rows_total - 1);
+  const int wg_kmax = pos0 + wg_last / G;
+  const int wg_kmin = p.window > 0 ? max(0, pos0 + wg_row0 / G - p.window + 1) : 0;
+  const int b0 = wg_kmin >> 6, b1 = (wg_kmax >> 6) + 1;
+  const int first = __builtin_amdgcn_readfirstlane(b0 + kgroup);   // this group's blocks: first, first + KG, ...
+  const int iterations = __builtin_amdgcn_readfirstlane((b1 - b0 + KG - 1) / KG);   // the same for every group
+
+  // The ring starts to fill before anything else is asked of memory.
+  const WideLane mine = wide_lane<D>(1 << p.page_shift, lane, wave_u);
+  TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
+#pragma unroll
+  for (int i = 0; i < NB - 1; ++i)
+    wide_fetch<D>(p, tw, first + i * KG, b1, wg_kmin, wg_kmax, kvh, lane, wave_u,
+                  ring_at + (unsigned int)(i * BUFFER), mine);
+
+  Frag qf[D / 16];
+  {
+    const bf16_t* qrow = p.q + (size_t)(q0 + tok) * p.q_stride + head * D + hh * 8;
+#pragma unroll
+    for (int k = 0; k < D / 16; ++k)
+      qf[k].u = row_ok ? *(const uint4*)(qrow + k * 16) : make_uint4(0, 0, 0, 0);
+  }
+  f32x16 acc[D / 32];
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
+  float m = -INFINITY, lsum = 0.f;
+
+  auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  const int last_flat = min(row0 + 31, rows_total - 1);
+  const int kmax = uniform(wave_has_rows ? pos0 + last_flat / G : -1);
+  const int kmin = uniform(p.window > 0 ? max(0, pos0 + row0 / G - p.window + 1) : 0);
+  const int see_upto = uniform(pos0 + row0 / G);       // every valid row of the wavefront sees up to here
+  const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
+  const float c = p.scale * 1.44269504088896340736f;
+  // the queries were asked for after the ring's first loads: all of them have to be there
+  // before the counting below starts
+  __builtin_amdgcn_s_waitcnt(WIDE_WAIT(0));
+
+  // One block: block i's loads of this wavefront have landed once at most the NB - 2 later
+  // blocks' are outstanding (in the first iteration the queries' loads were waited for
+  // above, which covered everything); after the barrier every wavefront's have, and
+  // everybody is done with block i - 1, whose buffer the block NB - 1 ahead now takes.
+  // Heads of 64: one softmax round over the block's 64 keys; heads of 128 (twice the
+  // accumulators): one per 32 keys, or the scores would not fit the registers.
+  constexpr int NSUB = D <= 64 ? 2 : 1;
+#define WIDE_ITERATION(MASKED)                                                                   \
+  do {                                                                                           \
+    const int b = first + i * KG;                                                                \
+    __builtin_amdgcn_s_waitcnt(WIDE_WAIT((NB - 2) * LOADS));                                     \
+    __syncthreads();                                                                             \
+    wide_fetch<D>(p, tw, b + (NB - 1) * KG, b1, wg_kmin, wg_kmax, kvh, lane, wave_u,             \
+                  ring_at + (unsigned int)(((i + NB - 1) % NB) * BUFFER), mine);                 \
+    const uint4* lds_k = (const uint4*)(ring + (i % NB) * BUFFER);                               \
+    const uint2* lds_v = (const uint2*)(ring + (i % NB) * BUFFER + 64 * D * 2);                  \
+    const int key0 = b << 6;                                                                     \
+    _Pragma("unroll") for (int sub0 = 0; sub0 < 2; sub0 += NSUB) {                               \
+      const int lo_key = key0 + sub0 * 32, hi_key = lo_key + NSUB * 32 - 1;                      \
+      if (MASKED && (b >= b1 || lo_key > kmax || hi_key < kmin)) continue;                       \
+      wide_block<D, NSUB, MASKED>(qf, acc, m, lsum, lds_k, lds_v, key0, sub0, c, n, hh, row_ok,  \
+                                  pos, lo);                                                      \
+    }                                                                                            \
+  } while (0)
+  // The blocks every valid row of the wavefront sees in full, [see_from, see_upto], take a
+  // loop of their own in which nothing is tested; the blocks before (a window's edge) and
+  // after (the causal edge, the sequence's end, blocks only other wavefronts see) are masked
+  // key by key.  Every wavefront meets the same number of barriers, in whichever loop.
+  const int full_from = uniform(max(0, ((see_from + 63) >> 6) - first + KG - 1) / KG);
+  const int last_full = (see_upto - 63) >> 6;             // the last block seen in full, if any
+  const int full_upto = uniform(see_upto >= 63 && last_full >= first
+                                    ? min(iterations, (last_full - first) / KG + 1) : 0);
+  int i = 0;
+  for (; i < min(full_from, iterations); ++i) WIDE_ITERATION(true);
+  for (; i < full_upto; ++i) WIDE_ITERATION(false);
+  for (; i < iterations; ++i) WIDE_ITERATION(true);
+#undef WIDE_ITERATION
+  // nothing may still be on its way into LDS when the workgroup's memory is given up or reused
+  __builtin_amdgcn_s_waitcnt(WIDE_WAIT(0));
+
+  if constexpr (KG > 1) {
+    // Groups 1.. hand their state to group 0, element by element: the same lane of the same
+    // wavefront-in-group holds the same rows and dims in every group.
+    __syncthreads();                                    // the rings are free now
+    float* const merge = (float*)lds;
+    const int slot = threadIdx.x & 255;
+    if (kgroup > 0) {
+      float* mine = merge + (size_t)(kgroup - 1) * MERGE * 256 + slot;
+      int e = 0;
+      mine[256 * e++] = m;
+      mine[256 * e++] = lsum;
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) mine[256 * e++] = acc[db][i];
+    }
+    __syncthreads();
+    if (kgroup > 0) return;
+#pragma unroll
+    for (int g = 1; g < KG; ++g) {
+      const float* theirs = merge + (size_t)(g - 1) * MERGE * 256 + slot;
+      int e = 0;
+      const float m_g = theirs[256 * e++], l_g = theirs[256 * e++];
+      const float m_new = fmaxf(m, m_g);
+      const float c_own = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+      const float c_g = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_g - m_new);
+      m = m_new;
+      lsum = lsum * c_own + l_g * c_g;
+#pragma unroll
+      for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) acc[db][i] = acc[db][i] * c_own + theirs[256 * e++] * c_g;
+    }
+  }
+
+  if (!row_ok) return;
+  float l = lsum + __shfl_xor(lsum, 32, 64);
+  const float inv = 1.f / l;
+  // acc[db][i] is O^T[dim = db * 32 + 8 (i / 4) + 4 hh + i % 4][row n].
+  bf16_t* dst = p.out + (size_t)(q0 + tok) * p.out_stride + head * D + 4 * hh;
+#pragma unroll
+  for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+    for (int q4 = 0; q4 < 4; ++q4)
+      *(uint2*)(dst + db * 32 + 8 * q4) =
+          make_uint2(pack_bf16x2(acc[db][4 * q4] * inv, acc[db][4 * q4 + 1] * inv),
+                     pack_bf16x2(acc[db][4 * q4 + 2] * inv, acc[db][4 * q4 + 3] * inv));
+}
+
 // Merge the key splits of one (tile, kv head, row) per workgroup: the maximum of the running
 // maxima, then the sums and the partial results rescaled to it.  Thread (g, dim) adds the
 // splits g, g + 4, ... of its dim, four loads in flight at a time; the four groups are then
@@ -711,6 +1075,21 @@ static void launch_staged(const AttnParams& p, int rows_per_tile, int key_groups
   }
 }
 
+// Ring depths by measurement: 64-wide heads run three workgroups a compute unit with three
+// buffers (2,048 x 4 tokens, 14 heads: 73 us against 83 with four buffers and two workgroups);
+// 128-wide heads two workgroups with two buffers (8,192 tokens, 28 heads: 752 us against 1256
+// with three buffers and one workgroup).
+template <int D>
+static void launch_wide(const AttnParams& p, int key_groups, hipStream_t stream) {
+  const dim3 grid(p.num_tiles, p.n_kv);
+  if constexpr (D == 64) {
+    attn_wide_kernel<D, 1, 3><<<grid, 256, 0, stream>>>(p);
+  } else {
+    if (key_groups == 2) attn_wide_kernel<D, 2, 2><<<grid, 512, 0, stream>>>(p);
+    else attn_wide_kernel<D, 1, 2><<<grid, 256, 0, stream>>>(p);
+  }
+}
+
 template <int D>
 static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stream) {
   const int per = ATTN_WAVES / p.kv_fold;   // tiles per workgroup
@@ -745,6 +1124,13 @@ extern "C" int mk_attention_mfma_staged(int head_dim, int rows_per_tile) {
   return rows_per_tile == 16 ? (head_dim == 64 ? 4 : 2) : (rows_per_tile == 32 ? 1 : 0);
 }
 
+// Into how many chains the prompt kernel of 32-row wavefronts and 64-key blocks (`staged` = 8
+// for one chain, 16 for two; 32 rows per wavefront, tile list in steps of 128 rows) can cut a
+// workgroup's keys at this head size; 0 if it does not take the size.
+extern "C" int mk_attention_mfma_wide(int head_dim) {
+  return head_dim == 64 ? 1 : (head_dim == 128 ? 2 : 0);
+}
+
 extern "C" int mk_attention_mfma_supported(int head_dim, int page_size) {
   const bool d_ok = head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 ||
                     head_dim == 192 || head_dim == 256;
@@ -776,9 +1162,15 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   MK_REQUIRE(rows_per_tile <= mk_attention_mfma_max_rows(d),
              "attention: %d rows per tile are too many for head size %d", rows_per_tile, d);
   MK_REQUIRE(split_blocks >= 0, "attention: negative split size");
-  MK_REQUIRE(staged == 0 || staged == 1 || staged == 2 || staged == 4,
-             "attention: %d key groups (0, 1, 2 or 4)", staged);
-  MK_REQUIRE(!staged || (num_splits == 1 && staged <= mk_attention_mfma_staged(d, rows_per_tile)),
+  MK_REQUIRE(staged == 0 || staged == 1 || staged == 2 || staged == 4 || staged == 8 || staged == 16,
+             "attention: %d key groups (0, 1, 2 or 4; 8 and 16 for the kernel of 32-row "
+             "wavefronts with one and two)", staged);
+  MK_REQUIRE(staged < 8 || (num_splits == 1 && rows_per_tile == 32 &&
+                            staged / 8 <= mk_attention_mfma_wide(d)),
+             "attention: the kernel of 32-row wavefronts takes unsplit keys, head sizes 64 and "
+             "128 (two key groups with 128 only) and 32 rows per wavefront");
+  MK_REQUIRE(!staged || staged >= 8 ||
+                 (num_splits == 1 && staged <= mk_attention_mfma_staged(d, rows_per_tile)),
              "attention: staging in LDS takes unsplit keys, head sizes 64 and 128 and 16 or 32 "
              "rows per wavefront (one key group with 32)");
   if (num_tiles == 0) return 0;
@@ -809,6 +1201,11 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   // with few tiles the wavefronts are better spread over more workgroups (one decoded token
   // of 8 key/value heads: 10 us unfolded, 16 folded; 64 tokens: 194 and 186)
   p.kv_fold = num_tiles < 32 ? 1 : (n_kv % 4 == 0 ? 4 : (n_kv % 2 == 0 ? 2 : 1));
+  if (staged >= 8) {
+    if (d == 64) launch_wide<64>(p, staged / 8, stream); else launch_wide<128>(p, staged / 8, stream);
+    MK_LAUNCH_CHECK("attention_mfma");
+    return 0;
+  }
   switch (d) {
     case 32: staged ? launch_staged<32>(p, rows_per_tile, staged, stream) : launch_attn<32>(p, rows_per_tile, stream); break;
     case 64: staged ? launch_staged<64>(p, rows_per_tile, staged, stream) : launch_attn<64>(p, rows_per_tile, stream); break;

@@ -27,6 +27,14 @@ constexpr int kFusedQkvMinWorkgroups = 128;
 
 constexpr int kAttentionTargetWaves = 1024;
 constexpr int kAttentionStagedWorkgroups = 64;
+// workgroups of 128 rows from which the kernel of 32-row wavefronts wins over the 16-row one
+// (14 heads of 64 in 2 groups: 2,048 tokens, 224 workgroups, 34 us against 30; 4 x 2,048, 896:
+// 73 against 90; 8,192: 202 against 288.  28 heads of 128 in 4 groups: 2,048 tokens, 448: 85
+// against 96; 8,192: 752 against 969; 512 tokens over 1,536, 112: 54 against 41; 40 heads in 8
+// groups there, 160: 54 with two key groups against 67)
+constexpr int kAttentionWideWorkgroups64 = 512;
+constexpr int kAttentionWideWorkgroups128 = 256;
+constexpr int kAttentionWideSplitWorkgroups128 = 128;
 constexpr int kAttentionStagedMaxWaves = 8192;
 constexpr int kAttentionWideTileWaves = 400;
 constexpr int kAttentionMinBlocksPerSplit = 2;
@@ -150,6 +158,21 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   if (tile_rows > 0) rows = tile_rows;
   int staged = staged_in;
   const bool split_forced = splits_in > 0;
+  if (staged >= 8) rows = 32;
+  // Long prompts of a head size it takes go to the kernel of 32-row wavefronts and 64-key
+  // blocks (`staged` 8, or 16 with the keys in two chains): workgroups of 128 rows of one
+  // sequence, chosen from the number of such workgroups at which it measured faster.
+  if (staged < 0 && !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 128) {
+    const int chains = t.mk_attention_mfma_wide(head_dim);
+    const long long workgroups = (total_rows / 128) * n_kv;
+    const long long full = head_dim == 64 ? kAttentionWideWorkgroups64 : kAttentionWideWorkgroups128;
+    if (chains >= 1 && workgroups >= full) {
+      staged = 8;
+    } else if (chains >= 2 && workgroups >= kAttentionWideSplitWorkgroups128 && blocks >= 16) {
+      staged = 16;
+    }
+    if (staged >= 8) rows = 32;
+  }
   if (staged < 0) {
     // prompts: plenty of rows per sequence, enough workgroups of 64 of them; 16 rows a
     // wavefront measured faster than 32 there
@@ -174,6 +197,7 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
     }
   }
   plan.staged = staged;
+  if (staged >= 8) return plan;
   const long long waves = std::max<long long>(1, (long long)plan.num_tiles * n_kv);
   if (!staged && waves < kAttentionTargetWaves) {
     // decoding, and short prompt portions over a long prefix (16 tokens over 2,032: 47 us as

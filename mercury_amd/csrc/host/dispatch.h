@@ -53,7 +53,8 @@ bool qkv_fusable(int x_dtype, int w_dtype, int m, int k, int head_dim, int rotar
 struct AttentionPlan {
   bool mfma = false;
   int rows = 16;          // rows per wavefront tile
-  int staged = 0;         // 0, or how many groups of four wavefronts share a workgroup's keys
+  int staged = 0;         // 0, or how many groups of four wavefronts share a workgroup's keys;
+                          // 8 and 16: the kernel of 32-row wavefronts with one and two groups
   int splits = 1;
   int split_blocks = 0;
   int tile_rows = 16;     // rows per entry of the tile list: rows, or 4 * rows when staged

@@ -26,6 +26,7 @@ class KernelError : public std::runtime_error {
   X(mk_linear_skinny_acc) X(mk_gated_skinny) X(mk_qkv_skinny) X(mk_qkv_tiled)                \
   X(mk_gated_tiled) X(mk_linear_tiled_slices) X(mk_linear_tiled_partials) X(mk_linear_tiled) \
   X(mk_attention_mfma_supported) X(mk_attention_mfma_max_rows) X(mk_attention_mfma_staged)   \
+  X(mk_attention_mfma_wide)                                                                  \
   X(mk_attention_mfma)
 
 struct KernelTable {

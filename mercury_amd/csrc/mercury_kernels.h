@@ -6,7 +6,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 11
+#define MK_ABI_VERSION 12
 
 #ifdef __cplusplus
 extern "C" {
@@ -143,7 +143,10 @@ int mk_attention_mfma_max_rows(int head_dim);
 // 4 * rows_per_tile rows, one per workgroup, whose wavefronts share the keys and values
 // through LDS, `staged` (1, 2 or 4, at most what mk_attention_mfma_staged returns) groups of
 // four wavefronts taking the key blocks in turn; for many rows per sequence, keys unsplit.
+// staged = 8: the prompt kernel built on 32 x 32 x 16 products (wavefronts of 32 rows, blocks
+// of 64 keys; tiles of 128 rows, rows_per_tile = 32), where mk_attention_mfma_wide says so.
 int mk_attention_mfma_staged(int head_dim, int rows_per_tile);
+int mk_attention_mfma_wide(int head_dim);
 int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       const void* k_cache, const void* v_cache, const int* tile_seq,
                       const int* tile_row0, int num_tiles, const int* cu_q, const int* kv_len,

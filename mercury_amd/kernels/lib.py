@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 from . import build
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 P, I, F, L = c_void_p, c_int, c_float, c_longlong
 
@@ -50,6 +50,7 @@ _SIGNATURES = {
         "mk_attention_mfma_supported": [I, I],
         "mk_attention_mfma_max_rows": [I],
         "mk_attention_mfma_staged": [I, I],
+        "mk_attention_mfma_wide": [I],
         "mk_attention_mfma": [P, I, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, P, P, P],
     },
 }

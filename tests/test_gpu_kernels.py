@@ -747,7 +747,10 @@ def test_attention_wide_tiles_for_prompts(tile_rows, d, n_q, n_kv, window, split
 @pytest.mark.parametrize("tile_rows,d,n_q,n_kv,page,groups", [
     (16, 64, 14, 2, 16, 1), (32, 64, 14, 2, 16, 1), (16, 128, 8, 2, 32, 1), (32, 128, 4, 4, 16, 1),
     (32, 64, 3, 1, 64, 1), (16, 64, 14, 2, 16, 2), (16, 64, 14, 2, 16, 4), (16, 128, 8, 2, 32, 2),
-    (16, 64, 3, 1, 64, 4)])
+    (16, 64, 3, 1, 64, 4),
+    # the kernel of 32-row wavefronts and 64-key blocks (32 x 32 x 16 products)
+    (32, 64, 14, 2, 16, 8), (32, 64, 3, 1, 64, 8), (32, 64, 8, 8, 32, 8), (32, 64, 16, 1, 128, 8),
+    (32, 128, 8, 2, 32, 8), (32, 128, 3, 1, 16, 8), (32, 128, 4, 4, 16, 16), (32, 128, 14, 2, 64, 16)])
 @pytest.mark.parametrize("window", [None, 40])
 def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, groups, window):
     """Workgroups whose wavefronts share the keys and values of one sequence through LDS, in
@@ -775,6 +778,40 @@ def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, groups
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("d,n_q,n_kv,page,groups", [
+    (64, 14, 2, 16, 8), (128, 6, 2, 16, 8), (128, 6, 2, 64, 16)])
+@pytest.mark.parametrize("window", [None, 200, 700])
+def test_attention_of_32_row_wavefronts_over_long_prompts(d, n_q, n_kv, page, groups, window):
+    """The prompt kernel of 32-row wavefronts walks its key blocks in three stretches: blocks
+    that a window's far edge cuts, blocks that every row sees whole, blocks that the diagonal
+    cuts.  Long sequences give each stretch several blocks, with one and with two chains of
+    blocks side by side; in each sequence one far key carries a score that stands out for the
+    rows that may see it, so a block dropped or taken twice shows."""
+    lens, q_lens = [1500, 700, 260], [1500, 300, 129]
+    qs, ks, vs = [], [], []
+    for i, s in enumerate(lens):
+        k = rnd(s, n_kv, d, seed=900 + i)
+        q = rnd(s, n_q, d, seed=920 + i)
+        far = s // 3 + 5
+        k[far] *= 3.0
+        q[far + 150:] += 6.0 / (9 * d ** 0.5) * k[far].repeat_interleave(n_q // n_kv, 0)
+        ks.append(rounded(k, torch.bfloat16))
+        vs.append(rounded(rnd(s, n_kv, d, seed=910 + i), torch.bfloat16))
+        qs.append(rounded(q, torch.bfloat16))
+    per = [-(-s // page) for s in lens]
+    order = torch.randperm(sum(per) + 3, generator=torch.Generator().manual_seed(11)).tolist()
+    pages, at = [], 0
+    for n in per:
+        pages.append(order[at:at + n])
+        at += n
+    got = run_attention([q[-ql:] for q, ql in zip(qs, q_lens)], ks, vs, torch.bfloat16, pages, page,
+                        sum(per) + 3, lens, q_lens, d ** -0.5, window=window, poison=1e4,
+                        kernel="mfma", tile_rows=32, staged=groups)
+    want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, 0, window)[-ql:]
+                      for q, k, v, ql in zip(qs, ks, vs, q_lens)])
+    torch.testing.assert_close(got, want, **tol(torch.bfloat16))
+
+
 def test_attention_through_lds_is_refused_where_it_does_not_fit():
     from mercury_amd.kernels.ops import KernelArgumentError
 
@@ -782,6 +819,11 @@ def test_attention_through_lds_is_refused_where_it_does_not_fit():
     with pytest.raises((KernelArgumentError, RuntimeError)):
         run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
                       kernel="mfma", staged=True)
+    # two chains of key blocks exist for 128-wide heads only
+    q = rounded(rnd(40, 2, 64, seed=1), torch.bfloat16)
+    with pytest.raises((KernelArgumentError, RuntimeError)):
+        run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
+                      kernel="mfma", tile_rows=32, staged=16)
 
 
 @pytest.mark.parametrize("batch,context", [(1, 4096), (3, 1500), (64, 300)])
