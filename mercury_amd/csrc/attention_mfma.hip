@@ -217,18 +217,27 @@ __device__ __forceinline__ void attend(TileState<D, RT>& st, const KeyBlock<D>& 
 // keys may be split); a prompt portion may give each wavefront RT consecutive tiles, which
 // share every key and value fragment the wavefront loads.  AHEAD: how many blocks of keys
 // are in flight beyond the one in the matrix cores (0, 1 or 2).
-template <int D, int RT, int AHEAD>
+//
+// GROUPED (one tile of 16 rows, keys split): the four wavefronts of a workgroup take four
+// consecutive parts of one tile's keys for one kv head, and add their results up through LDS
+// before anything is written: a quarter of the partial results for the merge, or none at all
+// when the workgroup has the tile's whole range.  p.num_splits then counts workgroups per
+// tile, each of ATTN_WAVES parts.
+template <int D, int RT, int AHEAD, bool GROUPED = false>
 __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) void attn_mfma_kernel(AttnParams p) {
+  static_assert(!GROUPED || (RT == 1 && D <= 128), "grouped parts: one tile, heads up to 128");
   const int lane = threadIdx.x & 63;
   // Tiles are taken from the last: under a causal mask the later tiles of a prompt read the
   // most keys, and the longest work should start first.
   // The wavefronts of a workgroup take `kv_fold` key/value heads of the same tiles: a page
   // holds its heads' keys side by side, and wavefronts that read them at the same time read
   // a longer stretch of memory between them.
-  const int wave = threadIdx.x >> 6, fold = p.kv_fold;
+  const int wave = threadIdx.x >> 6, fold = GROUPED ? ATTN_WAVES : p.kv_fold;
   const int tile = p.num_tiles - 1 - (blockIdx.x * (ATTN_WAVES / fold) + wave / fold);
-  if (tile < 0) return;
-  const int kvh = blockIdx.y * fold + wave % fold, split = blockIdx.z;
+  if (tile < 0) return;   // never in a grouped launch: one tile per workgroup
+  const int kvh = GROUPED ? blockIdx.y : blockIdx.y * fold + wave % fold;
+  const int split = GROUPED ? blockIdx.z * ATTN_WAVES + wave : blockIdx.z;
+  const int splits = GROUPED ? p.num_splits * ATTN_WAVES : p.num_splits;
   const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
   const int pos0 = p.kv_len[seq] - q_len;  // position of the step's first token of the sequence
@@ -262,8 +271,7 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
   const int kmax = pos0 + last_flat / G;
   const int kmin = p.window > 0 ? max(0, pos0 + row0 / G - p.window + 1) : 0;
   const int blk_lo = kmin >> 5, blk_hi = (kmax >> 5) + 1;
-  const int per = p.split_blocks > 0 ? p.split_blocks
-                                     : (blk_hi - blk_lo + p.num_splits - 1) / p.num_splits;
+  const int per = p.split_blocks > 0 ? p.split_blocks : (blk_hi - blk_lo + splits - 1) / splits;
   const int b0 = blk_lo + split * per, b1 = min(blk_hi, b0 + per);
   // Keys [see_from, see_upto] are visible to every valid row of the tiles.
   const int see_upto = pos0 + row0 / G;
@@ -304,6 +312,62 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
         attend<D, RT>(st, z, (b + 2) << 5, c, g4, see_upto, see_from);
       }
     }
+  }
+
+  if constexpr (GROUPED) {
+    // Rows padded by four floats: the 16 rows a store instruction touches then start on
+    // different banks.
+    constexpr int PITCH = D + 4;
+    __shared__ float part[ATTN_WAVES][16][PITCH];
+    __shared__ float part_m[ATTN_WAVES][16], part_l[ATTN_WAVES][16];
+    float l = st.lsum[0];
+    l += __shfl_xor(l, 16, 64);
+    l += __shfl_xor(l, 32, 64);
+#pragma unroll
+    for (int dt = 0; dt < D / 16; ++dt)
+      *(float4*)&part[wave][r][dt * 16 + g4 * 4] = make_float4(
+          st.acc[0][dt][0], st.acc[0][dt][1], st.acc[0][dt][2], st.acc[0][dt][3]);
+    if (g4 == 0) {
+      part_m[wave][r] = st.m[0];
+      part_l[wave][r] = l;
+    }
+    __syncthreads();
+    // Each thread adds the four parts of four dims of a row, in the parts' order.
+    constexpr int CHUNKS = D / 4;
+    for (int e = threadIdx.x; e < 16 * CHUNKS; e += 64 * ATTN_WAVES) {
+      const int row = e / CHUNKS, dim = (e % CHUNKS) * 4;
+      const int flat = row0 + row;
+      if (flat >= rows_total) continue;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int w = 0; w < ATTN_WAVES; ++w) mx = fmaxf(mx, part_m[w][row]);
+      float total = 0.f;
+      float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+      for (int w = 0; w < ATTN_WAVES; ++w) {
+        const float mw = part_m[w][row];
+        const float wt = mw == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(mw - mx);
+        total += part_l[w][row] * wt;
+        const float4 v = *(const float4*)&part[w][row][dim];
+        o.x += v.x * wt;
+        o.y += v.y * wt;
+        o.z += v.z * wt;
+        o.w += v.w * wt;
+      }
+      if (p.num_splits == 1) {
+        const float inv = total > 0.f ? 1.f / total : 0.f;
+        bf16_t* dst = p.out + (size_t)(q0 + flat / G) * p.out_stride + (kvh * G + flat % G) * D + dim;
+        *(uint2*)dst = make_uint2(pack_bf16x2(o.x * inv, o.y * inv), pack_bf16x2(o.z * inv, o.w * inv));
+      } else {
+        const size_t slot = (((size_t)tile * p.n_kv + kvh) * p.num_splits + blockIdx.z) * 16 + row;
+        *(float4*)(p.part_o + slot * D + dim) = o;
+        if (dim == 0) {
+          p.part_ml[slot * 2] = mx;
+          p.part_ml[slot * 2 + 1] = total;
+        }
+      }
+    }
+    return;
   }
 
 #pragma unroll
@@ -1090,8 +1154,34 @@ static void launch_wide(const AttnParams& p, int key_groups, hipStream_t stream)
   }
 }
 
+// Whether a split of one 16-row tile's keys goes to workgroups of ATTN_WAVES consecutive
+// parts each (the GROUPED kernel).
+static bool attn_grouped(int rows_per_tile, int num_splits) {
+  return rows_per_tile == 16 && num_splits >= ATTN_WAVES && num_splits % ATTN_WAVES == 0;
+}
+
+template <int D>
+static void launch_merge(const AttnParams& p, hipStream_t stream) {
+  if (p.num_splits > 1 && p.num_splits <= ATTN_MERGE_ROWS_MAX_SPLITS) {
+    attn_merge_rows_kernel<D><<<dim3(p.num_tiles, p.n_kv), 256, 0, stream>>>(p);
+  } else if (p.num_splits > 1) {
+    dim3 mgrid(p.num_tiles, p.n_kv, p.tile_rows);
+    attn_merge_kernel<D><<<mgrid, 256, 0, stream>>>(p);
+  }
+}
+
 template <int D>
 static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stream) {
+  if constexpr (D <= 128) {
+    if (attn_grouped(rows_per_tile, p.num_splits)) {
+      AttnParams g = p;
+      g.num_splits = p.num_splits / ATTN_WAVES;
+      const dim3 grid(g.num_tiles, g.n_kv, g.num_splits);
+      attn_mfma_kernel<D, 1, ATTN_AHEAD_16, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(g);
+      launch_merge<D>(g, stream);
+      return;
+    }
+  }
   const int per = ATTN_WAVES / p.kv_fold;   // tiles per workgroup
   dim3 grid((p.num_tiles + per - 1) / per, p.n_kv / p.kv_fold, p.num_splits);
   const int threads = 64 * ATTN_WAVES;
@@ -1103,12 +1193,7 @@ static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stre
     // 64 rows: only instantiated where the accumulators fit the register file
     if constexpr (D <= 64) attn_mfma_kernel<D, 4, ATTN_AHEAD_64><<<grid, threads, 0, stream>>>(p);
   }
-  if (p.num_splits > 1 && p.num_splits <= ATTN_MERGE_ROWS_MAX_SPLITS) {
-    attn_merge_rows_kernel<D><<<dim3(p.num_tiles, p.n_kv), 256, 0, stream>>>(p);
-  } else if (p.num_splits > 1) {
-    dim3 mgrid(p.num_tiles, p.n_kv, p.tile_rows);
-    attn_merge_kernel<D><<<mgrid, 256, 0, stream>>>(p);
-  }
+  launch_merge<D>(p, stream);
 }
 
 // The most rows (16, 32 or 64) one wavefront can take for this head size.

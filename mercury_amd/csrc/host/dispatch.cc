@@ -206,6 +206,9 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
     const int by_blocks = std::max(1, blocks / kAttentionMinBlocksPerSplit);
     const int by_waves = (int)((kAttentionTargetWaves + waves - 1) / waves);
     plan.splits = std::max(1, std::min({by_blocks, by_waves, kAttentionMaxSplits}));
+    // in fours, a workgroup's wavefronts take consecutive parts of one tile and add them up
+    // through LDS before they write
+    if (plan.splits >= 4) plan.splits = plan.splits / 4 * 4;
   }
   if (split_forced) {
     plan.splits = splits_in;
