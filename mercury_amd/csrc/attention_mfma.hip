@@ -767,11 +767,14 @@ __device__ __forceinline__ void wide_fetch(const AttnParams& p, TableWindow& tw,
   }
 }
 
+#define WIDE_SLACK 8.f
+
 // NSUB sub-blocks of 32 keys (from `sub0` of the block in LDS) against a wavefront's 32
 // rows: scores, one round of the online softmax over all of them, weighted values.
 template <int D, int NSUB, bool MASKED>
 __device__ __forceinline__ void wide_block(const Frag (&qf)[D / 16], f32x16 (&acc)[D / 32], float& m,
-                                           float& lsum, const uint4* lds_k, const uint2* lds_v,
+                                           f32x4 (&rowsum)[2], const Frag (&ones)[2],
+                                           const uint4* lds_k, const uint2* lds_v,
                                            int key0, int sub0, float c, int n, int hh, bool row_ok,
                                            int pos, int lo) {
   // All of the keys' operands are asked for before the first product, and the values'
@@ -820,38 +823,48 @@ __device__ __forceinline__ void wide_block(const Frag (&qf)[D / 16], f32x16 (&ac
 #pragma unroll
     for (int i = (u == 0 ? 1 : 0); i < 16; ++i) bm = fmaxf(bm, sc[u][i]);
   bm *= c;     // the largest raw score is the largest scaled one (c > 0)
-  // The two lanes of a row exchange their maxima and the row's maximum moves only when some
-  // lane of the wavefront saw a score above its row's; what is accumulated is multiplied
-  // either way (by one when nothing moved): a multiplication under a branch would have the
-  // accumulators copied around it, which costs more than the multiplications.
-  float corr = 1.f;
-  if (__builtin_amdgcn_ballot_w64(bm > m) != 0) {
+  // The row's reference maximum moves, and what is accumulated is rescaled, only when some
+  // lane of the wavefront saw a score more than WIDE_SLACK (in powers of two) above its
+  // row's: until then the exponentials may reach 2^WIDE_SLACK instead of 1, which float32
+  // sums and bfloat16 weights hold as well, and the result is a quotient in which the
+  // reference cancels.  The two lanes of a row exchange their maxima first, so that both
+  // always hold the same reference.
+  if (__builtin_expect(__builtin_amdgcn_ballot_w64(bm > m + WIDE_SLACK) != 0, 0)) {
     bm = fmaxf(bm, __shfl_xor(bm, 32, 64));
     const float m_new = fmaxf(m, bm);
-    corr = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
+    const float corr = __builtin_amdgcn_exp2f(m - (m_new == -INFINITY ? 0.f : m_new));
     m = m_new;
+    rowsum[0] *= corr;
+    rowsum[1] *= corr;
+#pragma unroll
+    for (int db = 0; db < D / 32; ++db)
+#pragma unroll
+      for (int i = 0; i < 16; ++i) acc[db][i] *= corr;
   }
-  lsum *= corr;
-#pragma unroll
-  for (int db = 0; db < D / 32; ++db)
-#pragma unroll
-    for (int i = 0; i < 16; ++i) acc[db][i] *= corr;
   const float m_use = (MASKED && m == -INFINITY) ? 0.f : m;
   Frag pf[NSUB][2];
-  float part = 0.f;
 #pragma unroll
   for (int u = 0; u < NSUB; ++u) {
     float e[16];
 #pragma unroll
     for (int i = 0; i < 16; ++i) e[i] = __builtin_amdgcn_exp2f(__builtin_fmaf(sc[u][i], c, -m_use));
-    part += (((e[0] + e[1]) + (e[2] + e[3])) + ((e[4] + e[5]) + (e[6] + e[7]))) +
-            (((e[8] + e[9]) + (e[10] + e[11])) + ((e[12] + e[13]) + (e[14] + e[15])));
 #pragma unroll
     for (int s = 0; s < 2; ++s)
       pf[u][s].u = make_uint4(pack_bf16x2(e[8 * s], e[8 * s + 1]), pack_bf16x2(e[8 * s + 2], e[8 * s + 3]),
                               pack_bf16x2(e[8 * s + 4], e[8 * s + 5]), pack_bf16x2(e[8 * s + 6], e[8 * s + 7]));
   }
-  lsum += part;
+  // The rows' sums of weights come out of the matrix cores as well, which have time to
+  // spare while the vector unit does not: the weights against ones.  As the operand of a
+  // 16 x 16 x 32 product a lane's eight weights are column lane % 16, keys' group lane / 16:
+  // groups 0 and 2 are the two halves of row lane % 16, groups 1 and 3 those of row
+  // 16 + lane % 16, and ones in the matching groups (`ones[0]`, `ones[1]`) pick each.
+#pragma unroll
+  for (int u = 0; u < NSUB; ++u)
+#pragma unroll
+    for (int s = 0; s < 2; ++s) {
+      rowsum[0] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones[0].v, pf[u][s].v, rowsum[0], 0, 0, 0);
+      rowsum[1] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ones[1].v, pf[u][s].v, rowsum[1], 0, 0, 0);
+    }
 #pragma unroll
   for (int db = 0; db < D / 32; ++db)
 #pragma unroll
@@ -866,7 +879,7 @@ __device__ __forceinline__ void wide_block(const Frag (&qf)[D / 16], f32x16 (&ac
 #define WIDE_WAIT(loads) (((loads) & 15) | (((loads) >> 4) << 14) | (7 << 4) | (15 << 8))
 
 template <int D, int KG, int NB>
-__global__ __launch_bounds__(256 * KG, (KG == 1 && NB * D <= 256) ? 2 : 1) void attn_wide_kernel(AttnParams p) {
+__global__ __launch_bounds__(256 * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D <= 256 ? 2 : 1))) void attn_wide_kernel(AttnParams p) {
   constexpr int BUFFER = 2 * 64 * D * 2;                   // bytes of a block's keys and values
   constexpr int LOADS = D / 16;                            // load instructions per wavefront and block
   constexpr int MERGE = D / 2 + 2;                         // floats a thread hands over
@@ -924,7 +937,17 @@ __global__ __launch_bounds__(256 * KG, (KG == 1 && NB * D <= 256) ? 2 : 1) void 
   for (int db = 0; db < D / 32; ++db)
 #pragma unroll
     for (int i = 0; i < 16; ++i) acc[db][i] = 0.f;
-  float m = -INFINITY, lsum = 0.f;
+  float m = -INFINITY;
+  // Sums of weights per row, kept by the matrix cores (see wide_block): rowsum[h][.] on lane l
+  // is the sum of row 16 h + l % 16, both halves' keys included.
+  f32x4 rowsum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+  Frag ones[2];
+  {
+    const uint32_t pair = 0x3F803F80u;                    // two bfloat16 ones
+    const uint32_t even = (lane & 16) ? 0u : pair, odd = (lane & 16) ? pair : 0u;
+    ones[0].u = make_uint4(even, even, even, even);
+    ones[1].u = make_uint4(odd, odd, odd, odd);
+  }
 
   auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
   const int last_flat = min(row0 + 31, rows_total - 1);
@@ -957,8 +980,8 @@ __global__ __launch_bounds__(256 * KG, (KG == 1 && NB * D <= 256) ? 2 : 1) void 
     _Pragma("unroll") for (int sub0 = 0; sub0 < 2; sub0 += NSUB) {                               \
       const int lo_key = key0 + sub0 * 32, hi_key = lo_key + NSUB * 32 - 1;                      \
       if (MASKED && (b >= b1 || lo_key > kmax || hi_key < kmin)) continue;                       \
-      wide_block<D, NSUB, MASKED>(qf, acc, m, lsum, lds_k, lds_v, key0, sub0, c, n, hh, row_ok,  \
-                                  pos, lo);                                                      \
+      wide_block<D, NSUB, MASKED>(qf, acc, m, rowsum, ones, lds_k, lds_v, key0, sub0, c, n, hh,  \
+                                  row_ok, pos, lo);                                              \
     }                                                                                            \
   } while (0)
   // The blocks every valid row of the wavefront sees in full, [see_from, see_upto], take a
@@ -977,6 +1000,8 @@ __global__ __launch_bounds__(256 * KG, (KG == 1 && NB * D <= 256) ? 2 : 1) void 
   // nothing may still be on its way into LDS when the workgroup's memory is given up or reused
   __builtin_amdgcn_s_waitcnt(WIDE_WAIT(0));
 
+  // this lane's row's sum of weights, both halves' keys included
+  float lsum = (lane & 16) ? rowsum[1][0] : rowsum[0][0];
   if constexpr (KG > 1) {
     // Groups 1.. hand their state to group 0, element by element: the same lane of the same
     // wavefront-in-group holds the same rows and dims in every group.
@@ -1013,8 +1038,7 @@ __global__ __launch_bounds__(256 * KG, (KG == 1 && NB * D <= 256) ? 2 : 1) void 
   }
 
   if (!row_ok) return;
-  float l = lsum + __shfl_xor(lsum, 32, 64);
-  const float inv = 1.f / l;
+  const float inv = 1.f / lsum;
   // acc[db][i] is O^T[dim = db * 32 + 8 (i / 4) + 4 hh + i % 4][row n].
   bf16_t* dst = p.out + (size_t)(q0 + tok) * p.out_stride + head * D + 4 * hh;
 #pragma unroll

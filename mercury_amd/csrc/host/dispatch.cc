@@ -31,11 +31,12 @@ constexpr int kAttentionStagedWorkgroups = 64;
 // (14 heads of 64 in 2 groups: 2,048 tokens, 224 workgroups, 34 us against 30; 4 x 2,048, 896:
 // 73 against 90; 8,192: 202 against 288.  28 heads of 128 in 4 groups: 2,048 tokens, 448: 85
 // against 96; 8,192: 752 against 969; 512 tokens over 1,536, 112: 54 against 41; 40 heads in 8
-// groups there, 160: 54 with two key groups against 67)
+// groups there, 160: 54 with two key groups against 67; 14 heads of 64 at 4,096 tokens, 448
+// workgroups: 97 against 91 with four key groups)
 constexpr int kAttentionWideWorkgroups64 = 512;
 constexpr int kAttentionWideWorkgroups128 = 256;
 constexpr int kAttentionWideSplitWorkgroups128 = 128;
-constexpr int kAttentionStagedMaxWaves = 8192;
+constexpr int kAttentionStagedMaxWaves = 16384;
 constexpr int kAttentionWideTileWaves = 400;
 constexpr int kAttentionMinBlocksPerSplit = 2;
 // Beyond this the merge of the parts costs more than the shorter chains save (one sequence
@@ -188,7 +189,8 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   if (staged == -1) {
     // A workgroup's chain of key blocks is cut into 2 or 4 chains side by side while that
     // leaves the chip short of wavefronts and every chain a few blocks (measured at 2,048
-    // tokens, 14 heads of 64: 45, 35, 32 us with 1, 2, 4 groups; at 8,192: 264, 349, 284;
+    // tokens, 14 heads of 64: 45, 35, 32 us with 1, 2, 4 groups; at 4,096: 95, 106, 91; at
+    // 8,192: 264, 349, 284;
     // 28 heads of 128 at 2,048: 100, 91 with 1, 2; at 8,192: 878, 1055).
     staged = t.mk_attention_mfma_staged(head_dim, 16);
     while (staged > 1 && ((long long)plan.num_tiles * n_kv * 4 * staged > kAttentionStagedMaxWaves ||
