@@ -8,7 +8,8 @@ random token ids, a batch of 8 and a context that reaches 4,096 tokens at the la
 One JSON line is printed: `value` is decoded tokens per second; `prefill` times one 2,048-token
 prompt as one step; `roofline` divides the bytes a decode step has to read (every weight it
 uses once, and the cache of the live requests) by its time and by the HBM peak; `points`
-holds decode throughput at batch 1 and 64 and, at the default batch, at half the context.
+holds decode throughput at batch 1 and 64 and, at the default batch, at half the context, and
+the tokens a second of one 8,192-token prompt as one step.
 Beside the published peaks both fractions are also given against what this machine reaches in
 the same run: a streaming read of a 2 GiB matrix by the engine's one-row projection, and a
 8192 x 8192 x 8192 bfloat16 product by its tiled matrix-core kernel (`measured`).
@@ -52,6 +53,7 @@ SHAPES = {"0.5b": ("Qwen2.5-0.5B", QWEN25_05B), "7b": ("Qwen2.5-7B", QWEN25_7B),
           "32b": ("Qwen2.5-32B", QWEN25_32B)}
 CONTEXT = 4096
 PREFILL_TOKENS = 2048
+LONG_PREFILL_TOKENS = 8192   # a second prompt length, in `points`
 BLOCK_SIZE = 16
 PEAK_HBM_GBS = 8000.0          # MI355X HBM3E
 PEAK_FLOPS = {"bf16": 2.5e15, "fp32": 157.3e12}
@@ -103,12 +105,12 @@ class Bench:
         self.torch = torch
         self.cfg = cfg
         t0 = time.time()
-        pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + PREFILL_TOKENS // BLOCK_SIZE + 8
+        pages = max_batch * (-(-(context + 128) // BLOCK_SIZE) + 1) + LONG_PREFILL_TOKENS // BLOCK_SIZE + 8
         self.engine_cfg = EngineConfig(
             model="random", random_weights=True, weight_seed=seed, weight_std=0.02,
             device="cuda:0", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
             max_running=max_batch + 1, prefill_budget=prefill_budget,
-            max_model_len=max(context, PREFILL_TOKENS) + 128, seed=seed,
+            max_model_len=max(context, LONG_PREFILL_TOKENS) + 128, seed=seed,
             lookahead=lookahead)
         self.engine = Engine(self.engine_cfg, model_config=cfg, eos_token_ids=())
         self.runner, self.manager = self.engine.executor.runner, self.engine.manager
@@ -334,6 +336,11 @@ def main(argv=None) -> int:
             run = bench.decode(b, args.context, steps, min(args.warmup, 4))
             points[f"decode_b{b}"] = round(run["tok_s"], 1)
             print(f"[bench] decode b{b}: {run['ms']:.3f} ms/step", file=sys.stderr, flush=True)
+        long = bench.prefill(LONG_PREFILL_TOKENS, repeats=3)
+        points[f"prefill_{LONG_PREFILL_TOKENS}"] = round(long["tok_s"], 1)
+        long_rate = prefill_flops(cfg, LONG_PREFILL_TOKENS) / (long["ms"] * 1e-3)
+        print(f"[bench] prefill {LONG_PREFILL_TOKENS}: {long['ms']:.2f} ms "
+              f"({long_rate / 1e15:.3f} PFLOP/s)", file=sys.stderr, flush=True)
 
     short = "bf16" if args.dtype == "bfloat16" else "fp32"
     achieved = main_run["bytes"] / (main_run["ms"] * 1e-3) / 1e9

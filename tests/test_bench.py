@@ -47,7 +47,7 @@ def test_the_line_of_one_gpu_keeps_the_contract():
     assert roof["bound"] == "hbm" and roof["peak"] == 8000.0 and roof["unit"] == "GB/s"
     assert roof["frac"] == pytest.approx(roof["achieved"] / roof["peak"], rel=1e-3) and 0 < roof["frac"] < 1
     assert 0 < line["prefill"]["frac"] < 1
-    assert set(line["points"]) == {"decode_b1", "decode_b64", "decode_b8_ctx256"}
+    assert set(line["points"]) == {"decode_b1", "decode_b64", "decode_b8_ctx256", "prefill_8192"}
     assert line["points"]["decode_b64"] > line["points"]["decode_b1"] > 0
     # against what the machine itself reaches: a streaming read between 2 and 8 TB/s, a large
     # product between 0.3 and 2.5 PFLOP/s; the step's device time (between two events, so with
