@@ -81,11 +81,6 @@ __device__ __forceinline__ float load_scalar(const void* p, int is_bf16, int i) 
   return is_bf16 ? bf16_to_f32(((const bf16_t*)p)[i]) : ((const float*)p)[i];
 }
 
-// Token m's values (bias added) at dims dd .. dd + 4 (`lo`) and dd + d/2 .. (`hi`) of head
-// `head` of [q heads | k heads | v heads]: rounded to bfloat16 as a stored projection would
-// be, q and k rotated by the token's position (the four lanes' dims are 4 rotation pairs), q
-// written to q_out, k and v into the paged cache.
-// Formulas: reference mercury/model/qwen2.py:57-64, mercury/model/rope.py:19-29.
 // Where token m's keys and values go: its position and the page that holds it (-1: none).
 // Looked up once per token, before any store: the stores might alias the tables for all the
 // compiler knows, and it would fetch them again after each.
@@ -102,8 +97,34 @@ __device__ __forceinline__ QkvPlace qkv_place(const QkvTarget& p, int m) {
   return place;
 }
 
-__device__ __forceinline__ void qkv_store(const QkvTarget& p, const QkvPlace& place, int m,
-                                          int head, int dd, float* lo, float* hi) {
+// The rotation of the 4 pairs (dims dd .. dd + 4 and their partners) of a token at the place's
+// position: asked for apart from the store, so that a kernel can have the angles on their way
+// while it still multiplies.  Heads of values, and models without rotation, turn by nothing.
+struct QkvAngles {
+  float4 c, s;
+};
+
+__device__ __forceinline__ QkvAngles qkv_angles(const QkvTarget& p, const QkvPlace& place, int head,
+                                                int dd) {
+  QkvAngles a;
+  a.c = make_float4(1.f, 1.f, 1.f, 1.f);
+  a.s = make_float4(0.f, 0.f, 0.f, 0.f);
+  if (p.rotate && head < p.n_q + p.n_kv) {
+    const int half = p.d / 2;
+    a.c = *(const float4*)(p.cos_table + (size_t)place.pos * half + dd);
+    a.s = *(const float4*)(p.sin_table + (size_t)place.pos * half + dd);
+  }
+  return a;
+}
+
+// Token m's values (bias added) at dims dd .. dd + 4 (`lo`) and dd + d/2 .. (`hi`) of head
+// `head` of [q heads | k heads | v heads]: rounded to bfloat16 as a stored projection would
+// be, q and k rotated by the token's position (the four lanes' dims are 4 rotation pairs), q
+// written to q_out, k and v into the paged cache.
+// Formulas: reference mercury/model/qwen2.py:57-64, mercury/model/rope.py:19-29.
+__device__ __forceinline__ void qkv_store(const QkvTarget& p, const QkvPlace& place,
+                                          const QkvAngles& angles, int m, int head, int dd,
+                                          float* lo, float* hi) {
   const int d = p.d, half = d / 2;
   const int pos = place.pos;
 #pragma unroll
@@ -113,9 +134,8 @@ __device__ __forceinline__ void qkv_store(const QkvTarget& p, const QkvPlace& pl
   }
   const bool is_v = head >= p.n_q + p.n_kv;
   if (p.rotate && !is_v) {
-    const float4 c = *(const float4*)(p.cos_table + (size_t)pos * half + dd);
-    const float4 s = *(const float4*)(p.sin_table + (size_t)pos * half + dd);
-    const float cs[4] = {c.x, c.y, c.z, c.w}, sn[4] = {s.x, s.y, s.z, s.w};
+    const float cs[4] = {angles.c.x, angles.c.y, angles.c.z, angles.c.w};
+    const float sn[4] = {angles.s.x, angles.s.y, angles.s.z, angles.s.w};
 #pragma unroll
     for (int i = 0; i < 4; ++i) {
       const float u = lo[i], v = hi[i];
@@ -212,6 +232,22 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
 
   int step = step_begin + wave;
   if (step < step_end) load_w(0, step);
+
+  // SK_QKV: where the tokens' keys and values go and by what their pairs turn is asked for
+  // now, by the wavefront that will write them: three trips to memory, each waiting for the
+  // one before, that would otherwise follow the products.
+  constexpr bool EARLY_PLACE = EPI == SK_QKV && MT <= 2;
+  QkvPlace place[MT];
+  QkvAngles angles[MT];
+  if constexpr (EARLY_PLACE) {
+    if (wave == 0) {
+#pragma unroll
+      for (int tb = 0; tb < MT; ++tb) {
+        place[tb] = qkv_place(p, min(tb * 16 + r, M - 1));
+        angles[tb] = qkv_angles(p, place[tb], head, dd0 + g4 * 4);
+      }
+    }
+  }
 
   // SK_ACC: the values the result is added to are asked for now, by the wavefront that will
   // write them, so that the epilogue does not wait for them.
@@ -335,7 +371,11 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
           hi[i] += load_scalar(p.bias, p.bias_bf16, n0 + half + g4 * 4 + i);
         }
       }
-      qkv_store(p, qkv_place(p, m), m, head, dd, lo, hi);
+      if constexpr (!EARLY_PLACE) {
+        place[tb] = qkv_place(p, m);
+        angles[tb] = qkv_angles(p, place[tb], head, dd);
+      }
+      qkv_store(p, place[tb], angles[tb], m, head, dd, lo, hi);
     } else {
       float* dst = (float*)p.out + ((size_t)(EPI == SK_PARTIAL ? slice : 0) * M + m) * N;
 #pragma unroll
@@ -759,7 +799,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
             hi[i] += Elem<TBIAS>::load(bias + head * target.d + half + dd + i);
           }
         }
-        qkv_store(target, place, m, head, dd, lo, hi);
+        qkv_store(target, place, qkv_angles(target, place, head, dd), m, head, dd, lo, hi);
       }
       continue;
     }
