@@ -1166,12 +1166,14 @@ static void launch_staged(const AttnParams& p, int rows_per_tile, int key_groups
 // Ring depths by measurement: 64-wide heads run three workgroups a compute unit with three
 // buffers (2,048 x 4 tokens, 14 heads: 73 us against 83 with four buffers and two workgroups);
 // 128-wide heads two workgroups with two buffers (8,192 tokens, 28 heads: 752 us against 1256
-// with three buffers and one workgroup).
+// with three buffers and one workgroup).  Key groups: as many as keep three (64) or two (128)
+// wavefronts a SIMD in one workgroup, for launches of fewer workgroups than fill the chip.
 template <int D>
 static void launch_wide(const AttnParams& p, int key_groups, hipStream_t stream) {
   const dim3 grid(p.num_tiles, p.n_kv);
   if constexpr (D == 64) {
-    attn_wide_kernel<D, 1, 3><<<grid, 256, 0, stream>>>(p);
+    if (key_groups == 3) attn_wide_kernel<D, 3, 3><<<grid, 768, 0, stream>>>(p);
+    else attn_wide_kernel<D, 1, 3><<<grid, 256, 0, stream>>>(p);
   } else {
     if (key_groups == 2) attn_wide_kernel<D, 2, 2><<<grid, 512, 0, stream>>>(p);
     else attn_wide_kernel<D, 1, 2><<<grid, 256, 0, stream>>>(p);
@@ -1233,11 +1235,12 @@ extern "C" int mk_attention_mfma_staged(int head_dim, int rows_per_tile) {
   return rows_per_tile == 16 ? (head_dim == 64 ? 4 : 2) : (rows_per_tile == 32 ? 1 : 0);
 }
 
-// Into how many chains the prompt kernel of 32-row wavefronts and 64-key blocks (`staged` = 8
-// for one chain, 16 for two; 32 rows per wavefront, tile list in steps of 128 rows) can cut a
-// workgroup's keys at this head size; 0 if it does not take the size.
+// Into how many chains the prompt kernel of 32-row wavefronts and 64-key blocks (`staged` =
+// 8 times the number of chains; 32 rows per wavefront, tile list in steps of 128 rows) can cut
+// a workgroup's keys at this head size: bit n - 1 is set when n chains exist (64: one or
+// three, 128: one or two); 0 if it does not take the size.
 extern "C" int mk_attention_mfma_wide(int head_dim) {
-  return head_dim == 64 ? 1 : (head_dim == 128 ? 2 : 0);
+  return head_dim == 64 ? 0b101 : (head_dim == 128 ? 0b011 : 0);
 }
 
 extern "C" int mk_attention_mfma_supported(int head_dim, int page_size) {
@@ -1271,13 +1274,14 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
   MK_REQUIRE(rows_per_tile <= mk_attention_mfma_max_rows(d),
              "attention: %d rows per tile are too many for head size %d", rows_per_tile, d);
   MK_REQUIRE(split_blocks >= 0, "attention: negative split size");
-  MK_REQUIRE(staged == 0 || staged == 1 || staged == 2 || staged == 4 || staged == 8 || staged == 16,
-             "attention: %d key groups (0, 1, 2 or 4; 8 and 16 for the kernel of 32-row "
-             "wavefronts with one and two)", staged);
+  MK_REQUIRE(staged == 0 || staged == 1 || staged == 2 || staged == 4 || staged == 8 ||
+                 staged == 16 || staged == 24,
+             "attention: %d key groups (0, 1, 2 or 4; 8, 16 and 24 for the kernel of 32-row "
+             "wavefronts with one, two and three)", staged);
   MK_REQUIRE(staged < 8 || (num_splits == 1 && rows_per_tile == 32 &&
-                            staged / 8 <= mk_attention_mfma_wide(d)),
-             "attention: the kernel of 32-row wavefronts takes unsplit keys, head sizes 64 and "
-             "128 (two key groups with 128 only) and 32 rows per wavefront");
+                            ((mk_attention_mfma_wide(d) >> (staged / 8 - 1)) & 1)),
+             "attention: the kernel of 32-row wavefronts takes unsplit keys, 32 rows per "
+             "wavefront and head sizes 64 (one or three key groups) and 128 (one or two)");
   MK_REQUIRE(!staged || staged >= 8 ||
                  (num_splits == 1 && staged <= mk_attention_mfma_staged(d, rows_per_tile)),
              "attention: staging in LDS takes unsplit keys, head sizes 64 and 128 and 16 or 32 "

@@ -36,6 +36,10 @@ constexpr int kAttentionStagedWorkgroups = 64;
 constexpr int kAttentionWideWorkgroups64 = 512;
 constexpr int kAttentionWideWorkgroups128 = 256;
 constexpr int kAttentionWideSplitWorkgroups128 = 128;
+// 14 heads of 64 with the keys in three chains: 2,048 tokens, 224 workgroups, 30.6 us against
+// 30.2; 4,096, 448: 64 against 89; 2,048 over 6,144: 102 against 139; 512 over 1,536, 56: 28
+// against 22
+constexpr int kAttentionWideSplitWorkgroups64 = 192;
 constexpr int kAttentionStagedMaxWaves = 16384;
 constexpr int kAttentionWideTileWaves = 400;
 constexpr int kAttentionMinBlocksPerSplit = 2;
@@ -164,13 +168,15 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   // blocks (`staged` 8, or 16 with the keys in two chains): workgroups of 128 rows of one
   // sequence, chosen from the number of such workgroups at which it measured faster.
   if (staged < 0 && !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 128) {
-    const int chains = t.mk_attention_mfma_wide(head_dim);
+    const int chains = t.mk_attention_mfma_wide(head_dim);   // bit n - 1: n chains exist
     const long long workgroups = (total_rows / 128) * n_kv;
     const long long full = head_dim == 64 ? kAttentionWideWorkgroups64 : kAttentionWideWorkgroups128;
-    if (chains >= 1 && workgroups >= full) {
+    const long long few = head_dim == 64 ? kAttentionWideSplitWorkgroups64 : kAttentionWideSplitWorkgroups128;
+    const int most = (chains & 4) ? 3 : ((chains & 2) ? 2 : 1);
+    if ((chains & 1) && workgroups >= full) {
       staged = 8;
-    } else if (chains >= 2 && workgroups >= kAttentionWideSplitWorkgroups128 && blocks >= 16) {
-      staged = 16;
+    } else if (most > 1 && workgroups >= few && blocks >= 16 * most) {
+      staged = 8 * most;
     }
     if (staged >= 8) rows = 32;
   }

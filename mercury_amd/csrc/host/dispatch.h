@@ -54,7 +54,7 @@ struct AttentionPlan {
   bool mfma = false;
   int rows = 16;          // rows per wavefront tile
   int staged = 0;         // 0, or how many groups of four wavefronts share a workgroup's keys;
-                          // 8 and 16: the kernel of 32-row wavefronts with one and two groups
+                          // 8, 16, 24: the kernel of 32-row wavefronts with one, two, three groups
   int splits = 1;
   int split_blocks = 0;
   int tile_rows = 16;     // rows per entry of the tile list: rows, or 4 * rows when staged

@@ -750,7 +750,8 @@ def test_attention_wide_tiles_for_prompts(tile_rows, d, n_q, n_kv, window, split
     (16, 64, 3, 1, 64, 4),
     # the kernel of 32-row wavefronts and 64-key blocks (32 x 32 x 16 products)
     (32, 64, 14, 2, 16, 8), (32, 64, 3, 1, 64, 8), (32, 64, 8, 8, 32, 8), (32, 64, 16, 1, 128, 8),
-    (32, 128, 8, 2, 32, 8), (32, 128, 3, 1, 16, 8), (32, 128, 4, 4, 16, 16), (32, 128, 14, 2, 64, 16)])
+    (32, 128, 8, 2, 32, 8), (32, 128, 3, 1, 16, 8), (32, 128, 4, 4, 16, 16), (32, 128, 14, 2, 64, 16),
+    (32, 64, 14, 2, 16, 24), (32, 64, 5, 1, 32, 24)])
 @pytest.mark.parametrize("window", [None, 40])
 def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, groups, window):
     """Workgroups whose wavefronts share the keys and values of one sequence through LDS, in
@@ -779,7 +780,7 @@ def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, groups
 
 
 @pytest.mark.parametrize("d,n_q,n_kv,page,groups", [
-    (64, 14, 2, 16, 8), (128, 6, 2, 16, 8), (128, 6, 2, 64, 16)])
+    (64, 14, 2, 16, 8), (128, 6, 2, 16, 8), (128, 6, 2, 64, 16), (64, 6, 2, 32, 24)])
 @pytest.mark.parametrize("window", [None, 200, 700])
 def test_attention_of_32_row_wavefronts_over_long_prompts(d, n_q, n_kv, page, groups, window):
     """The prompt kernel of 32-row wavefronts walks its key blocks in three stretches: blocks
@@ -819,11 +820,12 @@ def test_attention_through_lds_is_refused_where_it_does_not_fit():
     with pytest.raises((KernelArgumentError, RuntimeError)):
         run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
                       kernel="mfma", staged=True)
-    # two chains of key blocks exist for 128-wide heads only
-    q = rounded(rnd(40, 2, 64, seed=1), torch.bfloat16)
-    with pytest.raises((KernelArgumentError, RuntimeError)):
-        run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
-                      kernel="mfma", tile_rows=32, staged=16)
+    # two chains of key blocks exist for 128-wide heads only, three for 64-wide only
+    for d, groups in ((64, 16), (128, 24)):
+        q = rounded(rnd(40, 2, d, seed=1), torch.bfloat16)
+        with pytest.raises((KernelArgumentError, RuntimeError)):
+            run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
+                          kernel="mfma", tile_rows=32, staged=groups)
 
 
 @pytest.mark.parametrize("batch,context", [(1, 4096), (3, 1500), (64, 300)])
