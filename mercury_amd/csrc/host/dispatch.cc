@@ -175,7 +175,9 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
     const int most = (chains & 4) ? 3 : ((chains & 2) ? 2 : 1);
     if ((chains & 1) && workgroups >= full) {
       staged = 8;
-    } else if (most > 1 && workgroups >= few && blocks >= 16 * most) {
+    } else if (most > 1 && workgroups >= few && blocks >= 32 * most) {
+      // chains of at least 16 blocks of 64 keys each: a single 2,048-token prompt of 14 heads
+      // of 64 is a tie (30.6 against 30.2 us) and stays with the 16-row kernel
       staged = 8 * most;
     }
     if (staged >= 8) rows = 32;
