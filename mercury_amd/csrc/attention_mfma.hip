@@ -693,10 +693,19 @@ __global__ __launch_bounds__(64 * ATTN_WAVES * KG, (RT == 1 ? (KG > 2 ? KG : 2) 
 // into KG chains side by side).
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16;
 
+// Where chunk `chunk` (16 bytes) of key `key` lies in a buffer, in 16-byte units: sixteen
+// consecutive keys' rows of one chunk, which sixteen lanes read together, fall on all 64
+// banks (rows of 128 bytes alternate between the banks' halves, so the key's bit 0 picks the
+// half and bits 1-3 permute the chunk; rows of 256 bytes cover the banks, so bits 0-3 do).
+template <int D>
+__device__ __forceinline__ int wide_chunk_swizzle(int key, int chunk) {
+  return D == 64 ? ((chunk ^ (key >> 1)) & 7) : ((chunk ^ key) & 15);
+}
+
 template <int D>
 __device__ __forceinline__ int wide_key_offset(int key, int chunk) {   // in 16-byte units
   constexpr int CH = D / 8;
-  return key * CH + (chunk & ~7) + ((chunk ^ key) & 7);
+  return key * CH + wide_chunk_swizzle<D>(key, chunk);
 }
 
 // The loads of one block by one wavefront (D / 16 instructions), into the ring buffer at
@@ -714,7 +723,7 @@ __device__ __forceinline__ WideLane wide_lane(int page_size, int lane, int wave)
   constexpr int KEYS_PER_LOAD = 512 / D, CH = D / 8;
   const int key = wave * KEYS_PER_LOAD + lane / CH;      // of load j = 0; load j is 4 j loads on
   const int slot = lane % CH;
-  const int chunk = (slot & ~7) | ((slot ^ key) & 7);    // the chunk that lies at the lane's slot
+  const int chunk = wide_chunk_swizzle<D>(key, slot);    // the chunk that lies at the lane's slot
   const int dim = ((wave % (D / 64)) * 64 + lane) % D;
   WideLane out;
   out.k_at = (uint32_t)(key & 15) * (uint32_t)(D * 2) + (uint32_t)chunk * 16u;
