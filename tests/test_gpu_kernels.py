@@ -262,11 +262,15 @@ def test_the_tile_configuration_follows_the_problem():
     assert lib.mk_gated_tiled_config(32, 18944, 3584) == 7 and lib.mk_gated_tiled_config(32, 27648, 5120) == 1
     assert lib.mk_gated_tiled_config(32, 4864, 896) == 4
     assert lib.mk_gated_tiled_config(512, 27648, 5120) == 0
-    # 256 x 192 where 256 columns leave the last round of tiles half empty: 18944 pairs of
-    # rows at 512 rows of x (158 us against 167 in 128 x 256), 4608 columns at 2,048
-    assert lib.mk_gated_tiled_config(512, 18944, 3584) == 6
+    # 256 x 192 where 256 columns leave the last round of tiles half empty: 4608 columns at
+    # 2,048 rows of x (72 us against 90 in 128 x 256)
     assert lib.mk_linear_tiled_config(2048, 4608, 3584, 2) == 6
-    assert lib.mk_gated_tiled_config(2048, 18944, 3584) == 0
+    # 256 x 320, the most products per byte a stage brings, where its tiles fill the chip:
+    # 18944 pairs of rows at 512 rows of x (126 us against 179 in 128 x 256, 183 in 256 x 192),
+    # at 2,048 (448 against 488 in 256 x 256); 4864 pairs at 2,048 (45 against 54 in 256 x 192)
+    assert lib.mk_gated_tiled_config(512, 18944, 3584) == 9
+    assert lib.mk_gated_tiled_config(2048, 18944, 3584) == 9
+    assert lib.mk_gated_tiled_config(2048, 4864, 896) == 9
 
 
 def test_which_skinny_projections_are_split():
