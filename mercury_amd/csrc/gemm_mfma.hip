@@ -725,7 +725,9 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
   };
   // The products of a stage, with the loads of stage `ahead` handed out between them: all up
   // front (SPREAD 0), half before each half of k (1), or a few before every row of MFMA
-  // tiles (2).  Requests that arrive in one burst per stage take longer to be served.
+  // tiles (2).  Requests that arrive in one burst per stage take longer to be served, but a
+  // stage asked for earlier is there earlier: the 256 x 256 tile, with one stage of
+  // lookahead, is 2-5 % faster with all of them up front (8,192 cubed: 853 against 900 us).
   auto products = [&](const bf16_t* buffer, int ahead, bf16_t* into) __attribute__((always_inline)) {
     const bf16_t* xs = buffer;
     const bf16_t* ws = buffer + BM * TK;
@@ -913,7 +915,7 @@ static void launch_tiled(int config, const void* x, const void* w, const void* b
                          int bias_dtype, void* out, int M, int N, int K, int ldo, int slices,
                          hipStream_t stream, const QkvTarget& target = QkvTarget()) {
   switch (config) {
-    case 0: launch_tiled_cfg<256, 256, 2, 4, 4, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
+    case 0: launch_tiled_cfg<256, 256, 2, 4, 4, 0, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
     case 1: launch_tiled_cfg<128, 256, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
     case 2: launch_tiled_cfg<128, 128, 3, 2, 4, 2, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
     case 3: launch_tiled_cfg<128, 128, 2, 2, 2, 1, EPI>(x, w, bias, bias_dtype, out, M, N, K, ldo, slices, target, stream); break;
