@@ -14,6 +14,10 @@ Beside the published peaks both fractions are also given against what this machi
 the same run: a streaming read of a 2 GiB matrix by the engine's one-row projection, and a
 8192 x 8192 x 8192 bfloat16 product by its tiled matrix-core kernel (`measured`).
 
+    python bench.py --attention
+
+times the prompt attention kernel alone at the three models' head shapes, and
+
     python bench.py --shape 32b --serve
 
 runs a whole workload through the scheduler instead (64 requests with prompts of 2,048 tokens,
@@ -79,6 +83,9 @@ def parse_args(argv=None):
                         "half the context through the scheduler, prompts in portions of "
                         "--serve-chunk tokens beside the others' decoding, each decoded to the "
                         "context; one line with the generated tokens a second")
+    p.add_argument("--attention", action="store_true",
+                   help="instead of the engine's steps: the prompt attention kernel alone at the "
+                        "head shapes of the three models, a table of times and PFLOP/s")
     p.add_argument("--serve-requests", type=int, default=64)
     p.add_argument("--serve-chunk", type=int, default=512)
     return p.parse_args(argv)
@@ -304,12 +311,75 @@ def serve_main(args, model_name: str, cfg: dict, full_layers: int) -> int:
     return 0
 
 
+def attention_main(args) -> int:
+    """The attention kernel by itself, as the model's layers call it: queries of prompt
+    portions over a filled paged cache, the kernel and its shape chosen by the planner."""
+    import numpy as np
+    import torch
+
+    from mercury_amd.engine.batch import StepContext
+    from mercury_amd.kernels import ops
+
+    dev = "cuda:0"
+
+    def context(spans):
+        step = StepContext()
+        counts, starts = [c for c, _ in spans], [s for _, s in spans]
+        cu = np.zeros(len(spans) + 1, dtype=np.int64)
+        np.cumsum(counts, out=cu[1:])
+        seq = np.repeat(np.arange(len(spans)), counts)
+        positions = np.arange(int(cu[-1])) - cu[seq] + np.asarray(starts)[seq]
+        put = lambda a: torch.tensor(np.asarray(a), dtype=torch.int32, device=dev)
+        step.num_tokens, step.num_seqs = int(cu[-1]), len(spans)
+        step.token_ids = put(np.zeros(int(cu[-1])))
+        step.positions, step.token_seq, step.cu_q = put(positions), put(seq), put(cu)
+        step.kv_len = put(np.asarray(starts) + np.asarray(counts))
+        step.state_slots = put(np.arange(len(spans)))
+        step.spans = [(int(cu[i]), counts[i], starts[i]) for i in range(len(spans))]
+        step.max_q_len, step.max_kv_len = max(counts), max(s + c for c, s in spans)
+        step.all_decode = step.max_q_len == 1
+        return step
+
+    def run(spans, n_q, n_kv, d, repeats=10):
+        step = context(spans)
+        per = -(-max(c + s for c, s in spans) // BLOCK_SIZE)
+        table = torch.arange(len(spans) * per, dtype=torch.int32, device=dev).view(len(spans), per)
+        k_cache = torch.randn(len(spans) * per, n_kv, BLOCK_SIZE, d, device=dev).bfloat16()
+        v_cache = torch.randn(len(spans) * per, n_kv, d, BLOCK_SIZE, device=dev).bfloat16()
+        q = torch.randn(step.num_tokens, n_q * d, device=dev).bfloat16()
+        call = lambda: ops.attention(q, n_q * d, k_cache, v_cache, step, table, n_q, n_kv, d,
+                                     d ** -0.5, kernel="mfma")
+        for _ in range(3):
+            call()
+        begin, end = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+        begin.record()
+        for _ in range(repeats):
+            call()
+        end.record()
+        end.synchronize()
+        us = begin.elapsed_time(end) / repeats * 1e3
+        flops = sum(4.0 * n_q * d * (c * s + c * (c + 1) / 2) for c, s in spans)
+        return us, flops / us / 1e9
+
+    print("| heads x size (kv heads) | tokens (over a prefix) | sequences | us | PFLOP/s | of 2.5 |")
+    print("|---|---|---|---|---|---|")
+    for n_q, n_kv, d in ((14, 2, 64), (28, 4, 64), (28, 4, 128), (40, 8, 128)):
+        for count, prefix, seqs in ((2048, 0, 1), (8192, 0, 1), (2048, 0, 4), (2048, 30720, 1),
+                                    (1024, 15360, 16)):
+            us, rate = run([(count, prefix)] * seqs, n_q, n_kv, d)
+            print(f"| {n_q} x {d} ({n_kv}) | {count} ({prefix}) | {seqs} | {us:.0f} | {rate:.3f} | "
+                  f"{100 * rate / 2.5:.0f} % |", flush=True)
+    return 0
+
+
 def main(argv=None) -> int:
     args = parse_args(argv)
     if args.gpus != 1:
         print(f"bench.py measures one GPU; --gpus {args.gpus} is not supported (this engine "
               "has no multi-GPU path)")
         return 2
+    if args.attention:
+        return attention_main(args)
     model_name, shape = SHAPES[args.shape]
     cfg = dict(shape)
     full_layers = cfg["num_hidden_layers"]
