@@ -16,7 +16,7 @@ the same run: a streaming read of a 2 GiB matrix by the engine's one-row project
 
     python bench.py --attention
 
-times the prompt attention kernel alone at the three models' head shapes, and
+times the prompt attention kernel alone at the models' head shapes, and
 
     python bench.py --shape 32b --serve
 
