@@ -224,10 +224,11 @@ def build_library(name: str, force: bool = False, verbose: bool = True) -> Path:
     threads, errors = [], []
     headers = b"".join(p.read_bytes() for p in sorted(CSRC.glob("*.h")) + sorted(HOST_DIR.glob("*.h")))
     for src, obj, cmd in zip(sources, objects, compiles):
-        # An object whose command, source and headers are what they were is kept.
+        # An object whose command, source and headers are what they were is kept, unless the
+        # caller asked for everything to be compiled again.
         wanted = hashlib.sha256(" ".join(cmd).encode() + src.read_bytes() + headers).hexdigest()
         mark = obj.with_suffix(".o.stamp")
-        if obj.is_file() and mark.is_file() and mark.read_text().strip() == wanted:
+        if not force and obj.is_file() and mark.is_file() and mark.read_text().strip() == wanted:
             continue
 
         def work(cmd=cmd, src=src, mark=mark, wanted=wanted):
