@@ -117,7 +117,8 @@ class Bench:
             model="random", random_weights=True, weight_seed=seed, weight_std=0.02,
             device="cuda:0", dtype=dtype, block_size=BLOCK_SIZE, num_blocks=pages,
             max_running=max_batch + 1, prefill_budget=prefill_budget,
-            max_model_len=max(context, LONG_PREFILL_TOKENS) + 128, seed=seed,
+            max_model_len=min(max(context, LONG_PREFILL_TOKENS) + 128,
+                              cfg.get("max_position_embeddings", 1 << 30)), seed=seed,
             lookahead=lookahead)
         self.engine = Engine(self.engine_cfg, model_config=cfg, eos_token_ids=())
         self.runner, self.manager = self.engine.executor.runner, self.engine.manager
@@ -388,6 +389,13 @@ def main(argv=None) -> int:
     if args.serve:
         return serve_main(args, model_name, cfg, full_layers)
     max_batch = args.batch if args.no_points else max(args.batch, 64)
+    # requests are given a little room beyond the context they are measured at
+    limit = cfg.get("max_position_embeddings", 1 << 30) - max_batch - 16
+    if args.context > limit:
+        print(f"[bench] context {args.context} leaves no room below the model's "
+              f"{cfg['max_position_embeddings']} positions: measuring at {limit}",
+              file=sys.stderr, flush=True)
+        args.context = limit
     bench = Bench(cfg, args.dtype, max_batch, args.context, args.seed, not args.no_lookahead)
 
     main_run = bench.decode(args.batch, args.context, args.steps, args.warmup)
