@@ -87,3 +87,43 @@ def test_mixed_steps_use_the_prompt_kernel_when_a_portion_is_long(core):
     """A portion of 512 tokens beside 63 decoded ones: the prompt kernel for all of them."""
     p = plan(core, 14, 2, 64, [512] + [1] * 63, 4096)
     assert p["staged"] in (1, 2, 4) and p["splits"] == 1
+
+
+def test_the_qkv_projection_is_one_kernel_where_that_is_faster(core):
+    """Projection, bias, rotation and cache write in one kernel: the skinny one for few rows of
+    a small matrix (1152 x 896 at 8 rows: 6.0 us against 10.6 as partial sums and a finishing
+    kernel), the tiled one for many rows.  A matrix of 24 MB or more at up to 256 rows goes as
+    K-split partial sums and a finishing kernel (4608 x 3584 at 8..64 rows: 14.0..16.5 us
+    against 15.2..30.7 in the one skinny kernel)."""
+    skinny, tiled, partials, unfused = 0, 1, 2, 3
+    for rows, want in ((1, skinny), (8, skinny), (16, skinny), (64, tiled), (2048, tiled)):
+        assert core.choose_qkv(BF16, BF16, rows, 1152, 896, 64, 64, 16, True) == want
+    for rows, want in ((1, partials), (8, partials), (64, partials), (256, partials), (2048, tiled)):
+        assert core.choose_qkv(BF16, BF16, rows, 4608, 3584, 128, 128, 16, True) == want
+        assert core.choose_qkv(BF16, BF16, rows, 7168, 5120, 128, 128, 16, True) == want
+    # what the fused kernels do not take: heads that are no multiple of 32 wide, a rotation
+    # over part of the head, interleaved pairs
+    assert core.choose_qkv(BF16, BF16, 8, 18 * 48, 168, 48, 48, 16, True) in (partials, unfused)
+    assert core.choose_qkv(BF16, BF16, 8, 1152, 896, 64, 32, 16, True) == unfused
+    assert core.choose_qkv(BF16, BF16, 8, 1152, 896, 64, 64, 16, False) == unfused
+
+
+def test_projections_into_the_residual_stream(core):
+    """Few rows: K in slices with partial sums where the matrix is large enough for bandwidth
+    to matter (the 0.5B down projection, 8.7 MB, at 8 rows: 5.2 us in 8 slices against 9.5
+    whole), all of K in one workgroup where latency is the cost (the 0.5B o projection, 1.6 MB);
+    the skinny kernel up to 16 rows of a matrix under 20 MB, tiles beyond."""
+    by_skinny, slices = core.plan_partials(8, 896, 4864)
+    assert by_skinny and slices == 8
+    by_skinny, slices = core.plan_partials(8, 3584, 18944)
+    assert not by_skinny and slices >= 2          # 136 MB: tiles stream it faster
+    by_skinny, slices = core.plan_partials(64, 3584, 18944)
+    assert not by_skinny and slices >= 2
+    generic, skinny, skinny_acc, tiled = 0, 1, 2, 3
+    F32 = 0
+    assert core.choose_linear(BF16, 8, 896, 896, False, True, F32, 0) == skinny_acc
+    assert core.choose_linear(BF16, 2048, 896, 896, False, True, F32, 0) == tiled
+    assert core.choose_linear(BF16, 1, 151936, 896, False, False, F32, 0) == skinny      # the head
+    assert core.choose_linear(BF16, 8, 151936, 896, False, False, F32, 0) == tiled
+    assert core.choose_linear(BF16, 8, 896, 900, False, True, F32, 0) == generic         # K % 8
+    assert core.choose_linear(F32, 8, 896, 896, False, True, F32, 0) == generic
