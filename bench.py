@@ -152,7 +152,7 @@ class Bench:
             self.engine.submit(rid, self.tokens(prompt_len), steps + warmup + stagger + batch + 8,
                                lambda e: None, params=SamplingParams(ignore_eos=True))
             rids.append(rid)
-        self.engine._drain_commands()
+        self.engine._take_commands()
         t0 = time.time()
         while any(r.remaining > 1 for r in self.engine.sched.running) or self.engine.sched.waiting:
             self.engine.step()          # prompts, in portions under the token budget
@@ -176,7 +176,7 @@ class Bench:
         kv_bytes = kv_tokens * self.runner.kv_bytes_per_token()
         for rid in rids:
             self.engine.abort(rid)
-        self.engine._drain_commands()
+        self.engine._take_commands()
         assert self.engine.leaked_blocks() == 0
         ms = 1e3 * elapsed / steps
         timed = self.engine.metrics.step_records()[-steps:]
@@ -256,7 +256,7 @@ class Bench:
             self.counter += 1
             self.engine.submit(rid, self.tokens(prompt_len), new_tokens, sink,
                                params=SamplingParams(ignore_eos=True))
-        self.engine._drain_commands()
+        self.engine._take_commands()
         self.sync()
         start = time.perf_counter()
         steps = mixed = 0

@@ -71,6 +71,11 @@ class EngineConfig:
     max_step_records: int = 500_000
     debug_invariants: bool = False
     use_graphs: bool = True
+    # Captured decode graphs: one per (number of sequences, length bound), sharing one index
+    # buffer and one workspace; at most max_graphs are kept (the least recently used goes),
+    # and steps of more than max_graph_batch sequences are launched without a graph.
+    max_graph_batch: int = 256
+    max_graphs: int = 96
     # Start a decode step before the previous one's tokens have been read, when the scheduler
     # expects the same requests to go on (needs use_graphs).
     lookahead: bool = True

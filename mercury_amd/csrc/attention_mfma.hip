@@ -1258,13 +1258,10 @@ extern "C" int mk_attention_mfma_supported(int head_dim, int page_size) {
   return d_ok && page_size >= 16 && mk_is_pow2(page_size);
 }
 
-extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
-                                 const void* k_cache, const void* v_cache, const int* tile_seq,
-                                 const int* tile_row0, int num_tiles, const int* cu_q,
-                                 const int* kv_len, const int* block_table, int table_stride,
-                                 int page_size, int n_q, int n_kv, int d, float scale, int window,
-                                 int rows_per_tile, int staged, int num_splits, int split_blocks,
-                                 float* part_o, float* part_ml, hipStream_t stream) {
+extern "C" int mk_attention_mfma_check(int q_stride, int out_stride, int num_tiles, int page_size,
+                                       int n_q, int n_kv, int d, float scale, int window,
+                                       int rows_per_tile, int staged, int num_splits,
+                                       int split_blocks, int has_workspace) {
   MK_REQUIRE(num_tiles >= 0 && n_q > 0 && n_kv > 0, "attention: bad sizes");
   MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
              n_q, n_kv);
@@ -1273,7 +1270,7 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
              "32, 64, 96, 128, 192, 256 and pages of 16 or more are",
              d, page_size);
   MK_REQUIRE(num_splits >= 1 && num_splits <= 1024 && n_kv <= 65535, "attention: bad grid");
-  MK_REQUIRE(num_splits == 1 || (part_o && part_ml), "attention: key splits need a workspace");
+  MK_REQUIRE(num_splits == 1 || has_workspace, "attention: key splits need a workspace");
   MK_REQUIRE(q_stride % 8 == 0 && out_stride % 4 == 0,
              "attention: row strides %d/%d break 16-byte alignment", q_stride, out_stride);
   MK_REQUIRE(window >= 0, "attention: negative window");
@@ -1295,6 +1292,21 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
                  (num_splits == 1 && staged <= mk_attention_mfma_staged(d, rows_per_tile)),
              "attention: staging in LDS takes unsplit keys, head sizes 64 and 128 and 16 or 32 "
              "rows per wavefront (one key group with 32)");
+  return 0;
+}
+
+extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
+                                 const void* k_cache, const void* v_cache, const int* tile_seq,
+                                 const int* tile_row0, int num_tiles, const int* cu_q,
+                                 const int* kv_len, const int* block_table, int table_stride,
+                                 int page_size, int n_q, int n_kv, int d, float scale, int window,
+                                 int rows_per_tile, int staged, int num_splits, int split_blocks,
+                                 float* part_o, float* part_ml, hipStream_t stream) {
+  if (int code = mk_attention_mfma_check(q_stride, out_stride, num_tiles, page_size, n_q, n_kv, d,
+                                         scale, window, rows_per_tile, staged, num_splits,
+                                         split_blocks, part_o && part_ml)) {
+    return code;
+  }
   if (num_tiles == 0) return 0;
   AttnParams p;
   p.q = (const bf16_t*)q;

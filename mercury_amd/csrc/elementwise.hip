@@ -8,19 +8,19 @@
 
 template <typename T>
 __global__ void embed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
-                             float* __restrict__ out, int hidden, int vocab) {
+                             float* __restrict__ out, int hidden, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   // Ids are validated on the host; the clamp only keeps a bad id from reading outside.
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
   const T* row = table + (size_t)id * hidden;
   float* dst = out + (size_t)t * hidden;
-  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = Elem<T>::load(row + i);
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = Elem<T>::load(row + i) * scale;
 }
 
 // bfloat16 rows of a multiple of 8 elements: 16 bytes in, 32 bytes out per thread and turn.
 __global__ void embed_bf16x8_kernel(const int* __restrict__ ids, const bf16_t* __restrict__ table,
-                                    float* __restrict__ out, int hidden, int vocab) {
+                                    float* __restrict__ out, int hidden, int vocab, float scale) {
   const int t = blockIdx.x;
   int id = ids[t];
   id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
@@ -28,35 +28,61 @@ __global__ void embed_bf16x8_kernel(const int* __restrict__ ids, const bf16_t* _
   float4* dst = (float4*)(out + (size_t)t * hidden);
   for (int i = threadIdx.x; i < hidden / 8; i += blockDim.x) {
     const uint4 u = row[i];
-    dst[2 * i] = make_float4(__uint_as_float(u.x << 16), __uint_as_float(u.x & 0xffff0000u),
-                             __uint_as_float(u.y << 16), __uint_as_float(u.y & 0xffff0000u));
-    dst[2 * i + 1] = make_float4(__uint_as_float(u.z << 16), __uint_as_float(u.z & 0xffff0000u),
-                                 __uint_as_float(u.w << 16), __uint_as_float(u.w & 0xffff0000u));
+    dst[2 * i] = make_float4(__uint_as_float(u.x << 16) * scale,
+                             __uint_as_float(u.x & 0xffff0000u) * scale,
+                             __uint_as_float(u.y << 16) * scale,
+                             __uint_as_float(u.y & 0xffff0000u) * scale);
+    dst[2 * i + 1] = make_float4(__uint_as_float(u.z << 16) * scale,
+                                 __uint_as_float(u.z & 0xffff0000u) * scale,
+                                 __uint_as_float(u.w << 16) * scale,
+                                 __uint_as_float(u.w & 0xffff0000u) * scale);
   }
 }
 
 extern "C" int mk_embed(const int* ids, const void* table, int dtype, float* out, int tokens,
-                        int hidden, int vocab, hipStream_t stream) {
+                        int hidden, int vocab, float scale, hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes T=%d H=%d V=%d", tokens,
              hidden, vocab);
   if (tokens == 0) return 0;
   if (dtype == MK_BF16 && hidden % 8 == 0) {
     const int chunks = hidden / 8;
     embed_bf16x8_kernel<<<tokens, chunks >= 256 ? 256 : (chunks + 63) / 64 * 64, 0, stream>>>(
-        ids, (const bf16_t*)table, out, hidden, vocab);
+        ids, (const bf16_t*)table, out, hidden, vocab, scale);
     MK_LAUNCH_CHECK("embed");
     return 0;
   }
   const int threads = hidden >= 256 ? 256 : 64;
   if (dtype == MK_F32)
     embed_kernel<float><<<tokens, threads, 0, stream>>>(ids, (const float*)table, out, hidden,
-                                                        vocab);
+                                                        vocab, scale);
   else if (dtype == MK_BF16)
     embed_kernel<bf16_t><<<tokens, threads, 0, stream>>>(ids, (const bf16_t*)table, out, hidden,
-                                                         vocab);
+                                                         vocab, scale);
   else
     MK_REQUIRE(false, "embed: unknown dtype %d", dtype);
   MK_LAUNCH_CHECK("embed");
+  return 0;
+}
+
+// ------------------------------------------------------------------------------- logit cap
+
+// x <- cap * tanh(x / cap), in place: a smooth bound on the logits' size.  tanh from one
+// exponential: tanh(z) = 1 - 2 / (exp(2 z) + 1), exact at both ends (exp overflows to inf,
+// the quotient goes to 0).
+__global__ void logit_cap_kernel(float* __restrict__ x, long long n, float cap) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  const float z = x[i] / cap;
+  x[i] = cap * (1.f - 2.f / (__expf(2.f * z) + 1.f));
+}
+
+extern "C" int mk_logit_cap(float* logits, long long count, float cap, hipStream_t stream) {
+  MK_REQUIRE(count >= 0 && cap > 0.f, "logit_cap: bad arguments n=%lld cap=%g", count, (double)cap);
+  if (count == 0) return 0;
+  const long long blocks = (count + 255) / 256;
+  MK_REQUIRE(blocks < (1ll << 31), "logit_cap: %lld elements are too many for one launch", count);
+  logit_cap_kernel<<<(unsigned)blocks, 256, 0, stream>>>(logits, count, cap);
+  MK_LAUNCH_CHECK("logit_cap");
   return 0;
 }
 

@@ -5,7 +5,7 @@
 #include <mutex>
 #include <string>
 
-#include "kernels.h"
+#include "errors.h"
 
 namespace mercury {
 

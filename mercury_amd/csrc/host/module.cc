@@ -14,7 +14,8 @@
 namespace py = pybind11;
 using namespace mercury;
 
-void bind_device(py::module_& m);     // kernels, programs and the step runner (device.cc)
+void bind_program(py::module_& m);    // operation kinds, programs, the step packer
+void bind_ops(py::module_& m);        // the built-in operations (csrc/ops)
 
 namespace {
 
@@ -295,6 +296,7 @@ PYBIND11_MODULE(mercury_host, m) {
         }
         return out;
       })
+      .def_property_readonly("num_groups", &CacheManager::num_groups)
       .def("group_of", &CacheManager::group_of_slot, "The group a cache slot belongs to.")
       .def_property_readonly("state_slots", [](CacheManager& m) { return &m.state_slots(); },
                              py::return_value_policy::reference_internal)
@@ -635,5 +637,6 @@ PYBIND11_MODULE(mercury_host, m) {
         return out;
       });
 
-  bind_device(m);
+  bind_program(m);
+  bind_ops(m);
 }

@@ -1,65 +1,51 @@
 // A model's step as data: the list of operations one step launches, built once from the
 // model's parts, and the code that walks it, one call per step.
 //
-// Registers (all in a workspace the caller provides):
-//   h        float32 [T, H]   the residual stream; persistent over the step
-//   x        dtype   [T, H]   the last norm's output
-//   pending  float32 [P, T, H] partial sums of the last projection that the next norm adds
-//                             into h in the same pass (none when the projection added its
-//                             output into h itself)
-//   logits   float32 [R, V]
-// An operation allocates its outputs and temporaries from one of two arenas, alternating, so
-// that what the previous operation left is still there to read; `measure` walks the same code
-// without launching and reports the sizes a step needs.
+// The walk knows nothing of what an operation computes.  An operation is a registered kind
+// (op_abi.h: a name, a run function, optionally a function that says which row-tile lists a
+// step must carry for it) and a block of parameter bytes; kinds are registered at run time,
+// the package's own parts and anybody else's alike.  An entry may also be a *caller-run* step:
+// the walk stops there, the caller does that work itself on the same registers, and the walk
+// resumes behind it.
+//
+// Registers (op_abi.h) live in a workspace the caller provides: h and logits for the whole
+// step; x and pending in the arena of the operation that produced them.  Operations allocate
+// from one of two arenas in turn, so what the previous operation left is there to read and
+// what the one before left is gone: x and pending are alive for exactly one operation, and
+// the walk refuses (in a dry walk too, so at build time) a program in which an operation
+// reads an x that is no longer there or would drop partial sums nobody added up.
 #pragma once
 
 #include <cstddef>
 #include <cstdint>
+#include <map>
 #include <string>
 #include <vector>
 
-#include "dispatch.h"
+#include "errors.h"
+#include "op_abi.h"
 
 namespace mercury {
 
-// How a position encoding transforms q and k: rotation by tabulated angles over the first
-// `rotary_dim` dims of a head, pairing dim j with j + rotary_dim/2 ("half") or 2j with 2j+1
-// ("interleaved"); rotary_dim 0 is no transformation.
-struct PositionDesc {
-  int rotary_dim = 0;
-  const float* cos = nullptr;
-  const float* sin = nullptr;
-  int table_positions = 0;
-  bool interleaved = false;
+struct OpKind {
+  std::string name;
+  mk_op_run_fn run = nullptr;
+  mk_op_tiles_fn tiles = nullptr;
+  int flags = 0;
 };
 
-enum class OpKind { EMBED, NORM, ATTENTION, GATED_MLP, HEAD, HOST };
+// name -> kind, for the process.  Registering a name again replaces the kind for programs
+// built afterwards (programs hold their kinds by value).
+class OpRegistry {
+ public:
+  static OpRegistry& instance();
+  void add(const OpKind& kind);
+  const OpKind& get(const std::string& name) const;
+  bool has(const std::string& name) const { return kinds_.count(name) != 0; }
+  std::vector<std::string> names() const;
 
-struct Op {
-  OpKind kind = OpKind::HOST;
-  // EMBED
-  const void* table = nullptr;
-  int table_dtype = 0, vocab = 0;
-  // NORM, and the norm inside HEAD
-  const void* norm_w = nullptr;
-  int norm_w_dtype = 0;
-  float eps = 0.f;
-  // ATTENTION
-  const void *w_qkv = nullptr, *b_qkv = nullptr, *w_o = nullptr, *b_o = nullptr;
-  int b_qkv_dtype = 0, b_o_dtype = 0;
-  int n_q = 0, n_kv = 0, head_dim = 0;
-  PositionDesc pos;
-  void *k_cache = nullptr, *v_cache = nullptr;
-  int group = 0, page_size = 0, window = 0;
-  float scale = 0.f;
-  bool writes = true;
-  // GATED_MLP
-  const void *w_gate_up = nullptr, *w_down = nullptr;
-  int inter = 0;
-  // HEAD
-  const void* head_w = nullptr;
-  // HOST: the execution-list entry the caller runs itself
-  int host_index = -1;
+ private:
+  std::map<std::string, OpKind> kinds_;
 };
 
 // The index arrays of a step on the device, and what the host knows of it.
@@ -71,13 +57,11 @@ struct StepView {
   std::vector<int> widths;
   std::vector<int> counts;            // tokens per sequence
   int max_q_len = 0, max_kv_len = 0;
-  // attention tile lists by rows per tile (device), as the packer laid them out
-  struct Tiles {
-    int group = 0, tile_rows = 0, count = 0;
-    const int *seq = nullptr, *row0 = nullptr;
-  };
-  std::vector<Tiles> tiles;
-  const Tiles& tiles_for(int group, int tile_rows) const;
+  std::vector<mk_tile_list> tiles;    // as the packer laid them out
+
+  // A step of this shape with no device arrays behind it, for dry walks.
+  static StepView shape_only(const std::vector<int>& counts, int num_rows, int max_kv_len,
+                             int num_groups);
 };
 
 class Arena {
@@ -100,14 +84,21 @@ class Arena {
 };
 
 struct RunState {
-  // in: where to start, and partial sums a caller-run layer left (pointer, slice count)
+  // in: where to start, and what a caller-run step left for the operation behind it
   int begin = 0;
+  const void* x = nullptr;
+  int x_rows = 0;
   const float* pending = nullptr;
   int pending_count = 0;
-  // out: the operation the walk stopped before (ops.size() when it ran to the end)
+  // in, optional: a residual stream and room for logits of the caller's own (a single
+  // operation run on tensors that exist already); the workspace is then all arena
+  float* own_h = nullptr;
+  float* own_logits = nullptr;
+  // out: the entry the walk stopped before (size() when it ran to the end), and the
+  // registers as they stand there
   int stopped_at = 0;
   float* h = nullptr;
-  float* logits = nullptr;
+  float* logits = nullptr;      // null until an operation filled them
 };
 
 struct WorkspaceNeed {
@@ -121,29 +112,47 @@ class Program {
   int dtype() const { return dtype_; }
   int hidden() const { return hidden_; }
   int vocab() const { return vocab_; }
-  std::vector<Op>& ops() { return ops_; }
-  const std::vector<Op>& ops() const { return ops_; }
 
-  // The (heads-per-group, window, head size, page size ...) signatures of the program's
-  // attention operations, each with the tile lists a step of these counts needs.
+  // Append an operation of a registered kind; the parameter bytes are copied.
+  void append(const std::string& kind, const void* params, size_t bytes);
+  // Append a step the caller runs itself; `index` is the caller's own name for it, and
+  // `gives_x` says whether it leaves an x for the operation behind it.
+  void append_caller_step(int index, bool gives_x);
+
+  size_t size() const { return entries_.size(); }
+  // The kind's name, or "host" for a caller-run step.
+  std::string kind_of(size_t i) const;
+  int caller_index(size_t i) const { return entries_.at(i).caller_index; }
+
   struct TileNeed {
     int group, tile_rows;
   };
+  // The row-tile lists a step of this shape must carry for the program's operations.
   std::vector<TileNeed> tile_needs(const std::vector<int>& counts, int max_q_len,
                                    int max_kv_len) const;
 
-  WorkspaceNeed measure(const StepView& step) const;
-  // Walk the operations from state.begin until the end or a HOST operation.  `workspace`
-  // must hold measure(step).total() bytes.
+  // Walk without launching: what a step of this shape needs of its workspace.  Throws when
+  // the operations do not fit together.  given_x_rows > 0: the caller brings an x of that
+  // many rows for the first operation (a program that is one operation of a model).
+  WorkspaceNeed measure(const StepView& step, int given_x_rows = 0) const;
+  // Walk from state.begin until the end or a caller-run step.  `workspace` must hold
+  // measure(step).total() bytes.
   void run(const StepView& step, char* workspace, size_t workspace_bytes, void* stream,
            RunState& state) const;
 
  private:
+  struct Entry {
+    OpKind kind;                 // run == nullptr: a caller-run step
+    std::vector<char> params;    // 16-byte aligned copy (see append)
+    size_t offset = 0;
+    int caller_index = -1;
+    bool gives_x = false;
+  };
   void walk(const StepView& step, char* workspace, size_t workspace_bytes, void* stream,
             RunState& state, bool dry, WorkspaceNeed* need) const;
 
   int dtype_, hidden_, vocab_;
-  std::vector<Op> ops_;
+  std::vector<Entry> entries_;
 };
 
 }  // namespace mercury

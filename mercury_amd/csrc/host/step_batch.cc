@@ -7,7 +7,7 @@
 #include <cstring>
 #include <set>
 
-#include "kernels.h"
+#include "errors.h"
 
 namespace mercury {
 
@@ -35,7 +35,7 @@ StepView PackedStep::view(const int32_t* device) const {
   v.max_q_len = max_q_len;
   v.max_kv_len = max_kv_len;
   for (const TileList& t : tiles) {
-    StepView::Tiles out;
+    mk_tile_list out;
     out.group = t.group;
     out.tile_rows = t.tile_rows;
     out.count = t.count;
@@ -44,6 +44,23 @@ StepView PackedStep::view(const int32_t* device) const {
     v.tiles.push_back(out);
   }
   return v;
+}
+
+int count_tiles(const std::vector<int>& counts, int group, int tile_rows) {
+  int total = 0;
+  for (int c : counts) total += (c * group + tile_rows - 1) / tile_rows;
+  return total;
+}
+
+void build_tiles(const std::vector<int>& counts, int group, int tile_rows, std::vector<int>& seq,
+                 std::vector<int>& row0) {
+  for (int s = 0; s < (int)counts.size(); ++s) {
+    const int n = (counts[s] * group + tile_rows - 1) / tile_rows;
+    for (int i = 0; i < n; ++i) {
+      seq.push_back(s);
+      row0.push_back(i * tile_rows);
+    }
+  }
 }
 
 std::vector<int> PackedStep::layout() const {

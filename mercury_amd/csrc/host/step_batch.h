@@ -6,7 +6,7 @@
 // Layout, all int32: token ids [T], absolute positions [T], token -> sequence [T], prefix
 // sums of the sequences' token counts [S+1], lengths once this step's tokens are written [S],
 // state slots [S], wanted rows [R], one block table per cache group [S, W] (-1: none / given
-// back), and the tile lists the step's attention kernels walk.
+// back), and the row-tile lists the program's operations asked for.
 #pragma once
 
 #include <cstdint>
@@ -15,6 +15,7 @@
 
 #include "cache_manager.h"
 #include "program.h"
+#include "row_tiles.h"
 #include "scheduler.h"
 
 namespace mercury {
@@ -65,7 +66,7 @@ class StepPacker {
 
   // table_width < 0: as many columns as the longest sequence needs.  `program` may be null
   // (then no tile lists are laid out).  `check_ids` off when the ids are not the host's to know.
-  // kv_bound > 0: the step is planned (attention key splits) as if its longest sequence had
+  // kv_bound > 0: the step is planned (how operations split long sequences) as if its longest sequence had
   // that many tokens, as a captured graph needs that later, longer steps will replay.
   PackedStep pack(const std::vector<SeqInput>& seqs, const Program* program, int table_width,
                   bool check_ids = true, int kv_bound = 0);

@@ -1,12 +1,16 @@
-// C interface of the gfx950 kernel library.  Pointers are device pointers unless a comment
-// says otherwise; `stream` is a hipStream_t.  Functions validate their arguments on the host
-// against what the kernel and its grid assume, return 0 on success and non-zero after
-// recording a message for mk_last_error().  Dtype codes: 0 = float32, 1 = bfloat16.
+// C interface of the gfx950 kernel libraries.  This file is the one declaration of every
+// entry point: the host core's table of function pointers and the ctypes signatures of the
+// Python side are both derived from it (a line "// @library NAME" says which library the
+// declarations after it belong to; mk_last_error and mk_abi_version are in both).
+// Pointers are device pointers unless a comment says otherwise; `stream` is a hipStream_t.
+// Functions validate their arguments on the host against what the kernel and its grid
+// assume, return 0 on success and non-zero after recording a message for mk_last_error().
+// Dtype codes: 0 = float32, 1 = bfloat16.
 #pragma once
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 12
+#define MK_ABI_VERSION 13
 
 #ifdef __cplusplus
 extern "C" {
@@ -15,9 +19,14 @@ extern "C" {
 const char* mk_last_error();
 int mk_abi_version();
 
-// out[t, :] = table[ids[t], :] as float32 (the residual stream starts here).
+// @library core: float32 arithmetic, float32 or bfloat16 storage
+
+// out[t, :] = table[ids[t], :] * scale as float32 (the residual stream starts here).
 int mk_embed(const int* ids, const void* table, int dtype, float* out, int tokens, int hidden,
-             int vocab, hipStream_t stream);
+             int vocab, float scale, hipStream_t stream);
+
+// logits[i] = cap * tanh(logits[i] / cap) for i < count, in place.
+int mk_logit_cap(float* logits, long long count, float cap, hipStream_t stream);
 
 // RMSNorm of rows of the float32 residual stream h, optionally after adding `num_partials`
 // partial sums [p, row, hidden] (stride between partials in elements) into h.  `rows`, when
@@ -69,7 +78,7 @@ int mk_qkv_finish(const float* partials, int num_partials, long long partial_str
 int mk_fill_normal(void* out, int dtype, long long n, unsigned long long key, float mean,
                    float std, hipStream_t stream);
 
-// ---- library "mfma": bfloat16 kernels on the matrix cores
+// @library mfma: bfloat16 kernels on the matrix cores
 
 // y = x W^T for 1 <= M <= 16 rows of x, K split into `slices` (ask mk_linear_skinny_slices
 // for a good count): out is float32 [slices, M, N], to be summed over the slices.
@@ -145,8 +154,13 @@ int mk_attention_mfma_max_rows(int head_dim);
 // four wavefronts taking the key blocks in turn; for many rows per sequence, keys unsplit.
 // staged = 8: the prompt kernel built on 32 x 32 x 16 products (wavefronts of 32 rows, blocks
 // of 64 keys; tiles of 128 rows, rows_per_tile = 32), where mk_attention_mfma_wide says so.
+// mk_attention_mfma_check: what mk_attention_mfma checks of its arguments before it launches,
+// without the launch (0: it would take them; else mk_last_error() says why not).
 int mk_attention_mfma_staged(int head_dim, int rows_per_tile);
 int mk_attention_mfma_wide(int head_dim);
+int mk_attention_mfma_check(int q_stride, int out_stride, int num_tiles, int page_size, int n_q,
+                            int n_kv, int d, float scale, int window, int rows_per_tile,
+                            int staged, int num_splits, int split_blocks, int has_workspace);
 int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       const void* k_cache, const void* v_cache, const int* tile_seq,
                       const int* tile_row0, int num_tiles, const int* cu_q, const int* kv_len,
@@ -155,7 +169,7 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       int num_splits, int split_blocks, float* part_o, float* part_ml,
                       hipStream_t stream);
 
-// ---- library "core" again
+// @library core
 
 // parts: optional scratch of rows * 64 * 8 bytes; with it, few rows of a large vocabulary
 // are searched by 64 workgroups per row.

@@ -1,12 +1,17 @@
-// Bindings of what talks to the GPU: the kernel libraries, the decisions which kernel runs
-// what, programs, and the step packer.
+// Bindings of the built-in operations: the kernel libraries, the decisions which kernel runs
+// what, the parameter blocks of the built-in operation kinds, and the launch sequences as
+// functions of device addresses (what the Python faces of the kernels call, so that a kernel
+// test and a step's program go through the same code).
 #include <pybind11/pybind11.h>
 #include <pybind11/stl.h>
 
+#include <cstring>
+
+#include "../host/program.h"
+#include "builtin.h"
 #include "dispatch.h"
 #include "kernels.h"
-#include "program.h"
-#include "step_batch.h"
+#include "launch.h"
 
 namespace py = pybind11;
 using namespace mercury;
@@ -18,35 +23,20 @@ T* as_ptr(uintptr_t p) {
   return reinterpret_cast<T*>(p);
 }
 
-// Chunks as Python gives them: (key, token ids, start, wanted indices).
-struct Chunks {
-  std::vector<std::vector<int32_t>> tokens;
-  std::vector<SeqInput> seqs;
-  explicit Chunks(const py::handle& list) {
-    const size_t n = (size_t)py::len(list);
-    tokens.resize(n);
-    seqs.resize(n);
-    size_t i = 0;
-    for (const py::handle& item : list) {
-      py::object key, toks, start, want;
-      if (py::isinstance<py::tuple>(item)) {
-        py::tuple t = py::reinterpret_borrow<py::tuple>(item);
-        key = t[0]; toks = t[1]; start = t[2]; want = t[3];
-      } else {
-        key = item.attr("key"); toks = item.attr("tokens");
-        start = item.attr("start"); want = item.attr("want");
-      }
-      for (const py::handle& tok : toks) tokens[i].push_back(py::cast<int32_t>(tok));
-      SeqInput& s = seqs[i];
-      s.key = py::cast<std::string>(py::str(key));
-      s.tokens = tokens[i].data();
-      s.count = (int)tokens[i].size();
-      s.start = py::cast<int>(start);
-      for (const py::handle& w : want) s.want.push_back(py::cast<int>(w));
-      ++i;
-    }
-  }
-};
+template <typename T>
+T get(const py::dict& d, const char* key, T fallback) {
+  return d.contains(key) && !d[key].is_none() ? py::cast<T>(d[key]) : fallback;
+}
+
+template <typename T>
+T* ptr_of(const py::dict& d, const char* key) {
+  return as_ptr<T>(get<uintptr_t>(d, key, 0));
+}
+
+template <typename P>
+py::bytes blob(const P& params) {
+  return py::bytes(reinterpret_cast<const char*>(&params), sizeof params);
+}
 
 py::dict plan_to_py(const AttentionPlan& p) {
   py::dict d;
@@ -60,11 +50,93 @@ py::dict plan_to_py(const AttentionPlan& p) {
   return d;
 }
 
+// The q/k/v side of an attention as Python describes it: addresses and sizes by name.
+QkvArgs qkv_from(const py::dict& d) {
+  QkvArgs a;
+  a.w = ptr_of<const void>(d, "w_qkv");
+  a.bias = ptr_of<const void>(d, "b_qkv");
+  a.bias_dtype = get<int>(d, "b_qkv_dtype", kF32);
+  a.n_q = get<int>(d, "n_q", 0);
+  a.n_kv = get<int>(d, "n_kv", 0);
+  a.head_dim = get<int>(d, "head_dim", 0);
+  a.pos.rotary_dim = get<int>(d, "rotary_dim", 0);
+  a.pos.cos = ptr_of<const float>(d, "cos");
+  a.pos.sin = ptr_of<const float>(d, "sin");
+  a.pos.table_positions = get<int>(d, "table_positions", 0);
+  a.pos.interleaved = get<bool>(d, "interleaved", false) ? 1 : 0;
+  a.k_cache = ptr_of<void>(d, "k_cache");
+  a.v_cache = ptr_of<void>(d, "v_cache");
+  a.page_size = get<int>(d, "page_size", 1);
+  a.writes = get<bool>(d, "writes", true);
+  if (a.n_q <= 0 || a.n_kv <= 0 || a.head_dim <= 0 || a.n_q % a.n_kv) {
+    throw KernelError("attention: bad head counts or head size");
+  }
+  return a;
+}
+
+AttendArgs attend_from(const py::dict& d) {
+  AttendArgs a;
+  a.n_q = get<int>(d, "n_q", 0);
+  a.n_kv = get<int>(d, "n_kv", 0);
+  a.head_dim = get<int>(d, "head_dim", 0);
+  a.page_size = get<int>(d, "page_size", 0);
+  a.window = get<int>(d, "window", 0);
+  a.scale = get<float>(d, "scale", 0.f);
+  a.k_cache = ptr_of<const void>(d, "k_cache");
+  a.v_cache = ptr_of<const void>(d, "v_cache");
+  return a;
+}
+
+StepArrays arrays_from(const py::dict& d) {
+  StepArrays s;
+  s.positions = ptr_of<const int>(d, "positions");
+  s.token_seq = ptr_of<const int>(d, "token_seq");
+  s.cu_q = ptr_of<const int>(d, "cu_q");
+  s.kv_len = ptr_of<const int>(d, "kv_len");
+  s.table = ptr_of<const int>(d, "table");
+  s.table_stride = get<int>(d, "table_stride", 0);
+  return s;
+}
+
+void* scratch_alloc(void* arena, size_t bytes) { return static_cast<Arena*>(arena)->alloc(bytes); }
+
+// An operation context over memory the Python caller provides.
+struct Face {
+  Arena arena;
+  mk_op_context ctx;
+  Face(int dtype, uintptr_t stream, char* base, size_t size, bool dry) {
+    arena.reset(base, size, dry);
+    std::memset(&ctx, 0, sizeof ctx);
+    ctx.stream = as_ptr<void>(stream);
+    ctx.dry = dry ? 1 : 0;
+    ctx.dtype = dtype;
+    ctx.arena = &arena;
+    ctx.alloc = &scratch_alloc;
+  }
+};
+
+// Run a launch sequence over scratch memory of the caller's: once dry, to learn how much it
+// allocates; `alloc(bytes) -> address` is then asked for that much; then for real.
+template <typename F>
+auto with_scratch(int dtype, uintptr_t stream, const py::object& alloc, F body) {
+  Face dry(dtype, stream, nullptr, 0, true);
+  Launch measure(&dry.ctx);
+  body(measure);
+  const size_t need = dry.arena.peak();
+  uintptr_t base = 0;
+  if (need) {
+    if (alloc.is_none()) throw KernelError("this launch needs scratch memory and was given none");
+    base = py::cast<uintptr_t>(alloc(need));
+  }
+  Face wet(dtype, stream, as_ptr<char>(base), need, false);
+  Launch launch(&wet.ctx);
+  return body(launch);
+}
+
 }  // namespace
 
-void bind_device(py::module_& m) {
-  py::register_exception<KernelError>(m, "KernelError", PyExc_RuntimeError);
-  py::register_exception<BatchError>(m, "BatchError", PyExc_ValueError);
+void bind_ops(py::module_& m) {
+  register_builtin_ops();
 
   m.def("load_kernels", &load_kernel_library, py::arg("name"), py::arg("path"));
   m.def("kernels_loaded", [](const std::string& name) {
@@ -100,183 +172,198 @@ void bind_device(py::module_& m) {
         py::arg("window"), py::arg("counts"), py::arg("max_q_len"), py::arg("max_kv_len"),
         py::arg("force") = 0, py::arg("tile_rows") = -1, py::arg("staged") = -1,
         py::arg("splits") = 0, py::arg("split_blocks") = 0);
-  m.def("build_tiles", [](const std::vector<int>& counts, int group, int tile_rows) {
-    std::vector<int> seq, row0;
-    build_tiles(counts, group, tile_rows, seq, row0);
-    return py::make_tuple(seq, row0);
+  m.def("validate_attention_plan", [](const py::dict& plan, int head_dim, int page_size, int n_q,
+                                      int n_kv) {
+    AttentionPlan p;
+    p.mfma = py::cast<bool>(plan["mfma"]);
+    p.rows = py::cast<int>(plan["rows"]);
+    p.staged = py::cast<int>(plan["staged"]);
+    p.splits = py::cast<int>(plan["splits"]);
+    p.split_blocks = py::cast<int>(plan["split_blocks"]);
+    p.tile_rows = py::cast<int>(plan["tile_rows"]);
+    p.num_tiles = py::cast<int>(plan["num_tiles"]);
+    return plan_defect(p, head_dim, page_size, n_q, n_kv);
+  }, "Why the matrix-core attention would refuse this plan, or an empty string.");
+
+  // ---- parameter blocks of the built-in operation kinds
+  m.def("embed_params", [](uintptr_t table, int table_dtype, int vocab, float scale) {
+    EmbedParams p;
+    p.table = as_ptr<const void>(table);
+    p.table_dtype = table_dtype;
+    p.vocab = vocab;
+    p.scale = scale;
+    return blob(p);
+  }, py::arg("table"), py::arg("table_dtype"), py::arg("vocab"), py::arg("scale") = 1.f);
+  m.def("norm_params", [](uintptr_t weight, int weight_dtype, float eps, bool select_rows) {
+    NormParams p;
+    p.weight = as_ptr<const void>(weight);
+    p.weight_dtype = weight_dtype;
+    p.eps = eps;
+    p.select_rows = select_rows ? 1 : 0;
+    return blob(p);
+  }, py::arg("weight"), py::arg("weight_dtype"), py::arg("eps"), py::arg("select_rows") = false);
+  m.def("attention_params", [](const py::kwargs& kw) {
+    const py::dict d = kw;
+    AttentionParams p;
+    p.qkv = qkv_from(d);
+    p.w_o = ptr_of<const void>(d, "w_o");
+    p.b_o = ptr_of<const void>(d, "b_o");
+    p.b_o_dtype = get<int>(d, "b_o_dtype", kF32);
+    p.group = get<int>(d, "group", 0);
+    p.window = get<int>(d, "window", 0);
+    p.scale = get<float>(d, "scale", 0.f);
+    return blob(p);
   });
+  m.def("gated_mlp_params", [](uintptr_t w_gate_up, uintptr_t w_down, int inter) {
+    GatedMlpParams p;
+    p.w_gate_up = as_ptr<const void>(w_gate_up);
+    p.w_down = as_ptr<const void>(w_down);
+    p.inter = inter;
+    return blob(p);
+  });
+  m.def("head_params", [](uintptr_t weight, uintptr_t bias, int bias_dtype, float cap) {
+    HeadParams p;
+    p.weight = as_ptr<const void>(weight);
+    p.bias = as_ptr<const void>(bias);
+    p.bias_dtype = bias_dtype;
+    p.cap = cap;
+    return blob(p);
+  }, py::arg("weight"), py::arg("bias") = 0, py::arg("bias_dtype") = 0, py::arg("cap") = 0.f);
 
-  // ---- programs
-  py::class_<Program, std::shared_ptr<Program>>(m, "Program")
-      .def(py::init<int, int, int>(), py::arg("dtype"), py::arg("hidden"), py::arg("vocab"))
-      .def_property_readonly("num_ops", [](const Program& p) { return p.ops().size(); })
-      .def_property_readonly("kinds", [](const Program& p) {
-        static const char* names[] = {"embed", "norm", "attention", "gated_mlp", "head", "host"};
-        std::vector<std::string> out;
-        for (const Op& op : p.ops()) out.push_back(names[(int)op.kind]);
-        return out;
-      })
-      .def("embed", [](Program& p, uintptr_t table, int dtype, int vocab) {
-        Op op;
-        op.kind = OpKind::EMBED;
-        op.table = as_ptr<void>(table);
-        op.table_dtype = dtype;
-        op.vocab = vocab;
-        p.ops().push_back(op);
-      })
-      .def("norm", [](Program& p, uintptr_t weight, int dtype, float eps) {
-        Op op;
-        op.kind = OpKind::NORM;
-        op.norm_w = as_ptr<void>(weight);
-        op.norm_w_dtype = dtype;
-        op.eps = eps;
-        p.ops().push_back(op);
-      })
-      .def("attention", [](Program& p, uintptr_t w_qkv, uintptr_t b_qkv, int b_qkv_dtype,
-                           uintptr_t w_o, uintptr_t b_o, int b_o_dtype, int n_q, int n_kv,
-                           int head_dim, int rotary_dim, uintptr_t cos, uintptr_t sin,
-                           int table_positions, bool interleaved, uintptr_t k_cache,
-                           uintptr_t v_cache, int group, int page_size, float scale, int window,
-                           bool writes) {
-        Op op;
-        op.kind = OpKind::ATTENTION;
-        op.w_qkv = as_ptr<void>(w_qkv);
-        op.b_qkv = as_ptr<void>(b_qkv);
-        op.b_qkv_dtype = b_qkv_dtype;
-        op.w_o = as_ptr<void>(w_o);
-        op.b_o = as_ptr<void>(b_o);
-        op.b_o_dtype = b_o_dtype;
-        op.n_q = n_q;
-        op.n_kv = n_kv;
-        op.head_dim = head_dim;
-        op.pos.rotary_dim = rotary_dim;
-        op.pos.cos = as_ptr<float>(cos);
-        op.pos.sin = as_ptr<float>(sin);
-        op.pos.table_positions = table_positions;
-        op.pos.interleaved = interleaved;
-        op.k_cache = as_ptr<void>(k_cache);
-        op.v_cache = as_ptr<void>(v_cache);
-        op.group = group;
-        op.page_size = page_size;
-        op.scale = scale;
-        op.window = window;
-        op.writes = writes;
-        p.ops().push_back(op);
-      }, py::arg("w_qkv"), py::arg("b_qkv"), py::arg("b_qkv_dtype"), py::arg("w_o"), py::arg("b_o"),
-           py::arg("b_o_dtype"), py::arg("n_q"), py::arg("n_kv"), py::arg("head_dim"),
-           py::arg("rotary_dim"), py::arg("cos"), py::arg("sin"), py::arg("table_positions"),
-           py::arg("interleaved"), py::arg("k_cache"), py::arg("v_cache"), py::arg("group"),
-           py::arg("page_size"), py::arg("scale"), py::arg("window"), py::arg("writes"))
-      .def("gated_mlp", [](Program& p, uintptr_t w_gate_up, uintptr_t w_down, int inter) {
-        Op op;
-        op.kind = OpKind::GATED_MLP;
-        op.w_gate_up = as_ptr<void>(w_gate_up);
-        op.w_down = as_ptr<void>(w_down);
-        op.inter = inter;
-        p.ops().push_back(op);
-      })
-      .def("head", [](Program& p, uintptr_t norm_w, int norm_dtype, float eps, uintptr_t head_w) {
-        Op op;
-        op.kind = OpKind::HEAD;
-        op.norm_w = as_ptr<void>(norm_w);
-        op.norm_w_dtype = norm_dtype;
-        op.eps = eps;
-        op.head_w = as_ptr<void>(head_w);
-        p.ops().push_back(op);
-      })
-      .def("host", [](Program& p, int index) {
-        Op op;
-        op.kind = OpKind::HOST;
-        op.host_index = index;
-        p.ops().push_back(op);
-      })
-      .def("host_index", [](const Program& p, int op) { return p.ops().at((size_t)op).host_index; })
-      .def("workspace_bytes", [](const Program& p, const PackedStep& step) {
-        return p.measure(step.view(nullptr)).total();
-      })
-      .def("run", [](const Program& p, const PackedStep& step, uintptr_t ints, uintptr_t workspace,
-                     size_t workspace_bytes, uintptr_t stream, int begin, uintptr_t pending,
-                     int pending_count) {
-        RunState state;
-        state.begin = begin;
-        state.pending = as_ptr<const float>(pending);
-        state.pending_count = pending_count;
-        p.run(step.view(as_ptr<const int32_t>(ints)), as_ptr<char>(workspace), workspace_bytes,
-              as_ptr<void>(stream), state);
-        return py::make_tuple(state.stopped_at, (uintptr_t)state.h, (uintptr_t)state.logits,
-                              (uintptr_t)state.pending, state.pending_count);
-      }, py::arg("step"), py::arg("ints"), py::arg("workspace"), py::arg("workspace_bytes"),
-           py::arg("stream"), py::arg("begin") = 0, py::arg("pending") = 0,
-           py::arg("pending_count") = 0,
-           "Launch the operations from `begin` to the end or to the next caller-run layer; "
-           "returns (stopped_at, h, logits, pending, pending_count) as device addresses.");
-
-  py::class_<PackedStep>(m, "PackedStep")
-      .def_readonly("num_tokens", &PackedStep::num_tokens)
-      .def_readonly("num_seqs", &PackedStep::num_seqs)
-      .def_readonly("num_rows", &PackedStep::num_rows)
-      .def_readonly("max_q_len", &PackedStep::max_q_len)
-      .def_readonly("max_kv_len", &PackedStep::max_kv_len)
-      .def_readonly("counts", &PackedStep::counts)
-      .def_readonly("starts", &PackedStep::starts)
-      .def_readonly("widths", &PackedStep::widths)
-      .def_readonly("fresh_slots", &PackedStep::fresh_slots)
-      .def_readonly("total", &PackedStep::total)
-      .def_property_readonly("host_address", [](const PackedStep& p) { return (uintptr_t)p.host; })
-      .def_property_readonly("spans", [](const PackedStep& p) {
-        py::list out;
-        for (size_t s = 0; s < p.counts.size(); ++s) {
-          out.append(py::make_tuple(p.firsts[s], p.counts[s], p.starts[s]));
-        }
-        return out;
-      })
-      .def_property_readonly("offsets", [](const PackedStep& p) {
-        py::dict d;
-        d["token_ids"] = py::make_tuple(p.off_ids, p.num_tokens);
-        d["positions"] = py::make_tuple(p.off_positions, p.num_tokens);
-        d["token_seq"] = py::make_tuple(p.off_token_seq, p.num_tokens);
-        d["cu_q"] = py::make_tuple(p.off_cu_q, p.num_seqs + 1);
-        d["kv_len"] = py::make_tuple(p.off_kv_len, p.num_seqs);
-        d["state_slots"] = py::make_tuple(p.off_slots, p.num_seqs);
-        d["logit_rows"] = py::make_tuple(p.off_rows, p.num_rows);
-        py::list tables;
-        for (size_t g = 0; g < p.off_tables.size(); ++g) {
-          tables.append(py::make_tuple(p.off_tables[g], p.num_seqs, p.widths[g]));
-        }
-        d["tables"] = tables;
-        py::list tiles;
-        for (const PackedStep::TileList& t : p.tiles) {
-          tiles.append(py::make_tuple(t.group, t.tile_rows, t.count, t.off_seq, t.off_row0));
-        }
-        d["tiles"] = tiles;
-        return d;
-      })
-      .def("layout", [](const PackedStep& p) { return py::tuple(py::cast(p.layout())); })
-      .def("host_list", [](const PackedStep& p) {
-        return std::vector<int32_t>(p.host, p.host + p.total);
-      });
-
-  py::class_<StepPacker>(m, "StepPacker")
-      .def(py::init([](std::shared_ptr<CacheManager> manager, int vocab, int max_positions,
-                       bool pinned) {
-        auto* packer = new StepPacker(manager, vocab, max_positions);
-        packer->set_pinned(pinned);
-        return packer;
-      }), py::arg("manager"), py::arg("vocab_size"), py::arg("max_positions"),
-           py::arg("pinned") = true)
-      .def("pack", [](StepPacker& packer, py::handle chunks, std::shared_ptr<Program> program,
-                      int table_width, bool check_ids, int kv_bound) {
-        Chunks c(chunks);
-        return packer.pack(c.seqs, program.get(), table_width, check_ids, kv_bound);
-      }, py::keep_alive<0, 1>(), py::arg("chunks"), py::arg("program") = nullptr,
-           py::arg("table_width") = -1, py::arg("check_ids") = true, py::arg("kv_bound") = 0)
-      .def("pack_plan", [](StepPacker& packer, const Plan& plan, std::shared_ptr<Program> program,
-                           int table_width, int kv_bound) {
-        return packer.pack_plan(plan, program.get(), table_width, kv_bound);
-      }, py::keep_alive<0, 1>(), py::arg("plan"), py::arg("program") = nullptr,
-           py::arg("table_width") = -1, py::arg("kv_bound") = 0)
-      .def("upload", [](StepPacker& packer, const PackedStep& step, uintptr_t device,
-                        uintptr_t stream) {
-        packer.upload(step, as_ptr<void>(device), as_ptr<void>(stream));
-      });
+  // ---- the launch sequences, by device address
+  m.def("launch_embed", [](uintptr_t ids, uintptr_t table, int table_dtype, uintptr_t out,
+                           int tokens, int hidden, int vocab, float scale, uintptr_t stream) {
+    Face f(kF32, stream, nullptr, 0, false);
+    Launch l(&f.ctx);
+    embed(l, as_ptr<const int>(ids), as_ptr<const void>(table), table_dtype, as_ptr<float>(out),
+          tokens, hidden, vocab, scale);
+  });
+  m.def("launch_rmsnorm", [](uintptr_t h, int tokens, int hidden, uintptr_t pending,
+                             int pending_count, uintptr_t weight, int weight_dtype, float eps,
+                             uintptr_t rows, int out_rows, uintptr_t out, int out_dtype,
+                             uintptr_t stream) {
+    Face f(out_dtype, stream, nullptr, 0, false);
+    Launch l(&f.ctx);
+    rmsnorm(l, as_ptr<float>(h), tokens, hidden, as_ptr<const float>(pending), pending_count,
+            as_ptr<const void>(weight), weight_dtype, eps, as_ptr<const int>(rows), out_rows,
+            as_ptr<void>(out));
+  });
+  m.def("launch_silu_mul", [](uintptr_t gate_up, uintptr_t out, int dtype, int tokens, int inter,
+                              uintptr_t stream) {
+    Face f(dtype, stream, nullptr, 0, false);
+    Launch l(&f.ctx);
+    silu_mul(l, as_ptr<const void>(gate_up), tokens, inter, as_ptr<void>(out));
+  });
+  m.def("launch_logit_cap", [](uintptr_t logits, long long count, float cap, uintptr_t stream) {
+    Face f(kF32, stream, nullptr, 0, false);
+    Launch l(&f.ctx);
+    logit_cap(l, as_ptr<float>(logits), count, cap);
+  });
+  m.def("launch_linear", [](uintptr_t x, int m_, uintptr_t w, int n, int k, int dtype,
+                            uintptr_t bias, int bias_dtype, uintptr_t out, int out_dtype,
+                            bool accumulate, int kernel, int tile_config, uintptr_t stream) {
+    Face f(dtype, stream, nullptr, 0, false);
+    Launch l(&f.ctx);
+    LinearForce force;
+    force.kernel = kernel;
+    force.tile_config = tile_config;
+    linear(l, as_ptr<const void>(x), m_, as_ptr<const void>(w), n, k, as_ptr<const void>(bias),
+           bias_dtype, as_ptr<void>(out), out_dtype, accumulate, force);
+  });
+  m.def("launch_linear_partials", [](uintptr_t x, int m_, uintptr_t w, int n, int k, int dtype,
+                                     const py::object& alloc, uintptr_t stream) {
+    int slices = 0;
+    float* out = with_scratch(dtype, stream, alloc, [&](Launch& l) {
+      return linear_partials(l, as_ptr<const void>(x), m_, as_ptr<const void>(w), n, k, slices);
+    });
+    return py::make_tuple((uintptr_t)out, slices);
+  });
+  m.def("launch_project", [](uintptr_t x, int m_, uintptr_t w, int n, int k, int dtype,
+                             uintptr_t bias, int bias_dtype, uintptr_t h, const py::object& alloc,
+                             uintptr_t stream) {
+    const float* pending = nullptr;
+    int count = 0;
+    with_scratch(dtype, stream, alloc, [&](Launch& l) {
+      project_into_stream(l, as_ptr<const void>(x), m_, as_ptr<const void>(w), n, k,
+                          as_ptr<const void>(bias), bias_dtype, as_ptr<float>(h), pending, count);
+      return 0;
+    });
+    return py::make_tuple((uintptr_t)pending, count);
+  }, "h += x W^T (+ bias), or partial sums left for the next norm: (address, how many).");
+  m.def("launch_gated", [](uintptr_t x, int m_, int k, uintptr_t w, int inter, int dtype,
+                           int tile_config, const py::object& alloc, uintptr_t stream) {
+    void* act = with_scratch(dtype, stream, alloc, [&](Launch& l) {
+      return gated(l, as_ptr<const void>(x), m_, k, as_ptr<const void>(w), inter, tile_config);
+    });
+    return (uintptr_t)act;
+  });
+  m.def("launch_qkv_project", [](uintptr_t x, int m_, int k, int dtype, const py::dict& args,
+                                 const py::dict& arrays, int kind, int tile_config,
+                                 const py::object& alloc, uintptr_t stream) {
+    const QkvArgs a = qkv_from(args);
+    const StepArrays s = arrays_from(arrays);
+    QkvForce force;
+    force.kind = kind;
+    force.tile_config = tile_config;
+    const Queries q = with_scratch(dtype, stream, alloc, [&](Launch& l) {
+      return qkv_project(l, as_ptr<const void>(x), m_, k, a, s, force);
+    });
+    return py::make_tuple((uintptr_t)q.q, q.stride);
+  }, "Returns (address of the rotated queries, their row stride in elements).");
+  m.def("launch_rope_kv_write", [](uintptr_t qkv, int row_stride, int m_, int dtype,
+                                   const py::dict& args, const py::dict& arrays, uintptr_t stream) {
+    Face f(dtype, stream, nullptr, 0, false);
+    Launch l(&f.ctx);
+    rope_kv_write(l, as_ptr<void>(qkv), row_stride, m_, qkv_from(args), arrays_from(arrays));
+  });
+  m.def("launch_qkv_finish", [](uintptr_t parts, int slices, int m_, int out_dtype,
+                                const py::dict& args, const py::dict& arrays,
+                                const py::object& alloc, uintptr_t stream) {
+    const QkvArgs a = qkv_from(args);
+    const StepArrays s = arrays_from(arrays);
+    void* q = with_scratch(out_dtype, stream, alloc, [&](Launch& l) {
+      return qkv_finish(l, as_ptr<const float>(parts), slices, m_, a, s, out_dtype);
+    });
+    return (uintptr_t)q;
+  });
+  m.def("launch_attention", [](uintptr_t q, int q_stride, int dtype, const py::dict& args,
+                               const py::dict& arrays, const std::vector<int>& counts,
+                               int max_q_len, int max_kv_len, const py::dict& force_in,
+                               const py::object& tiles, uintptr_t out, const py::object& alloc,
+                               uintptr_t stream) {
+    const AttendArgs a = attend_from(args);
+    const StepArrays s = arrays_from(arrays);
+    AttendForce force;
+    force.kernel = get<int>(force_in, "kernel", 0);
+    force.tile_rows = get<int>(force_in, "tile_rows", -1);
+    force.staged = get<int>(force_in, "staged", -1);
+    force.splits = get<int>(force_in, "splits", 0);
+    force.split_blocks = get<int>(force_in, "split_blocks", 0);
+    mk_step_view view;
+    std::memset(&view, 0, sizeof view);
+    view.num_seqs = (int)counts.size();
+    view.counts = counts.data();
+    for (int c : counts) view.num_tokens += c;
+    view.max_q_len = max_q_len;
+    view.max_kv_len = max_kv_len;
+    // the tile list the plan will walk, from the caller
+    const AttentionPlan plan = plan_for(dtype, a, view, force);
+    mk_tile_list list;
+    std::memset(&list, 0, sizeof list);
+    if (plan.mfma) {
+      const py::tuple t = tiles(a.n_q / a.n_kv, plan.tile_rows);
+      list.group = a.n_q / a.n_kv;
+      list.tile_rows = plan.tile_rows;
+      list.seq = as_ptr<const int>(py::cast<uintptr_t>(t[0]));
+      list.row0 = as_ptr<const int>(py::cast<uintptr_t>(t[1]));
+      list.count = py::cast<int>(t[2]);
+      view.num_tile_lists = 1;
+      view.tile_lists = &list;
+    }
+    void* result = with_scratch(dtype, stream, alloc, [&](Launch& l) {
+      return attend(l, Queries{as_ptr<const void>(q), q_stride}, a, s, view, force,
+                    as_ptr<void>(out));
+    });
+    return (uintptr_t)result;
+  });
 }

@@ -118,23 +118,6 @@ QkvKind choose_qkv(int x_dtype, int w_dtype, int m, int width, int k, int head_d
   return QkvKind::PARTIALS_FINISH;
 }
 
-int count_tiles(const std::vector<int>& counts, int group, int tile_rows) {
-  int total = 0;
-  for (int c : counts) total += (c * group + tile_rows - 1) / tile_rows;
-  return total;
-}
-
-void build_tiles(const std::vector<int>& counts, int group, int tile_rows, std::vector<int>& seq,
-                 std::vector<int>& row0) {
-  for (int s = 0; s < (int)counts.size(); ++s) {
-    const int n = (counts[s] * group + tile_rows - 1) / tile_rows;
-    for (int i = 0; i < n; ++i) {
-      seq.push_back(s);
-      row0.push_back(i * tile_rows);
-    }
-  }
-}
-
 AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, int n_kv, int window,
                              const std::vector<int>& counts, int max_q_len, int max_kv_len,
                              int force, int tile_rows, int staged_in, int splits_in,
@@ -228,6 +211,17 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
     plan.split_blocks = split_blocks_in;
   }
   return plan;
+}
+
+std::string plan_defect(const AttentionPlan& plan, int head_dim, int page_size, int n_q, int n_kv) {
+  if (!plan.mfma) return "";
+  const KernelTable& t = need_mfma();
+  const int width = n_q * head_dim;
+  if (t.mk_attention_mfma_check(width, width, plan.num_tiles, page_size, n_q, n_kv, head_dim, 1.f, 0,
+                                plan.rows, plan.staged, plan.splits, plan.split_blocks, 1) == 0) {
+    return "";
+  }
+  return t.mfma_error();
 }
 
 }  // namespace mercury

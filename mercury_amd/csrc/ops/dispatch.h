@@ -1,11 +1,12 @@
 // Which kernel runs an operation of a given shape.  These decisions are pure functions of
-// sizes and element types; the Python faces of the kernels (kernels/ops.py) and the step
-// programs (program.cc) both ask here, so that what the tests exercise kernel by kernel is
-// what a step launches.
+// sizes and element types; the launch sequences (launch.cc) ask here, whoever calls them.
 #pragma once
 
 #include <cstdint>
+#include <string>
 #include <vector>
+
+#include "../host/row_tiles.h"
 
 namespace mercury {
 
@@ -67,9 +68,9 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
                              const std::vector<int>& counts, int max_q_len, int max_kv_len,
                              int force = 0, int tile_rows = -1, int staged = -1,
                              int splits = 0, int split_blocks = 0);
-int count_tiles(const std::vector<int>& counts, int group, int tile_rows);
-// tile_seq and tile_row0, `num_tiles` entries each, appended to `out`.
-void build_tiles(const std::vector<int>& counts, int group, int tile_rows, std::vector<int>& seq,
-                 std::vector<int>& row0);
+
+// Why the matrix-core attention would refuse to run `plan` for these sizes ("" when it takes
+// it): the kernel entry point's own argument checks, without the launch.
+std::string plan_defect(const AttentionPlan& plan, int head_dim, int page_size, int n_q, int n_kv);
 
 }  // namespace mercury

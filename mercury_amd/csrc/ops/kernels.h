@@ -4,30 +4,15 @@
 // the host core runs with "core" alone when "mfma" was never loaded.
 #pragma once
 
-#include <stdexcept>
 #include <string>
 
+#include "../host/errors.h"
 #include "../mercury_kernels.h"
+// MK_CORE_FUNCTIONS(X) and MK_MFMA_FUNCTIONS(X): the entry points of the two libraries by
+// name, written by the build from the declarations in mercury_kernels.h.
+#include "kernel_names.inc"
 
 namespace mercury {
-
-class KernelError : public std::runtime_error {
- public:
-  using std::runtime_error::runtime_error;
-};
-
-#define MK_CORE_FUNCTIONS(X)                                                                 \
-  X(mk_embed) X(mk_rmsnorm) X(mk_silu_mul) X(mk_rope_kv_write) X(mk_linear_generic)          \
-  X(mk_attention_generic) X(mk_qkv_finish) X(mk_argmax) X(mk_sample_scratch_bytes)           \
-  X(mk_sample) X(mk_fill_normal)
-
-#define MK_MFMA_FUNCTIONS(X)                                                                 \
-  X(mk_linear_skinny_slices) X(mk_linear_skinny) X(mk_linear_skinny_unsplit)                 \
-  X(mk_linear_skinny_acc) X(mk_gated_skinny) X(mk_qkv_skinny) X(mk_qkv_tiled)                \
-  X(mk_gated_tiled) X(mk_linear_tiled_slices) X(mk_linear_tiled_partials) X(mk_linear_tiled) \
-  X(mk_attention_mfma_supported) X(mk_attention_mfma_max_rows) X(mk_attention_mfma_staged)   \
-  X(mk_attention_mfma_wide)                                                                  \
-  X(mk_attention_mfma)
 
 struct KernelTable {
 #define MK_DECLARE(name) decltype(&::name) name = nullptr;

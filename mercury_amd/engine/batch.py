@@ -75,6 +75,27 @@ class StepContext:
         return cached
 
 
+    def as_view(self, program=None) -> dict:
+        """The step by device address, as ``Program.run_on`` takes it; with the row-tile lists
+        `program` needs for a step of this shape."""
+        ptr = lambda t: 0 if t is None else t.data_ptr()
+        counts = [count for _first, count, _start in self.spans]
+        tiles = []
+        if program is not None:
+            for group, rows in program.tile_needs(counts, self.max_q_len, self.max_kv_len):
+                seq, row0, count = self.tiles(group, rows)
+                tiles.append((group, rows, ptr(seq), ptr(row0), count))
+        return {
+            "counts": counts, "num_rows": self.num_logit_rows,
+            "max_q_len": self.max_q_len, "max_kv_len": self.max_kv_len,
+            "token_ids": ptr(self.token_ids), "positions": ptr(self.positions),
+            "token_seq": ptr(self.token_seq), "cu_q": ptr(self.cu_q), "kv_len": ptr(self.kv_len),
+            "state_slots": ptr(self.state_slots), "logit_rows": ptr(self.logit_rows),
+            "tables": [(ptr(t), t.shape[1]) for t in self.block_tables],
+            "tiles": tiles,
+        }
+
+
 def context_from_packed(packed, ints: torch.Tensor) -> StepContext:
     """A step context over `ints`, the int32 tensor (on the device, or on the host for tests)
     that holds the packed step."""

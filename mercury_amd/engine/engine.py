@@ -14,9 +14,9 @@ runs a plan on the GPU (reference for the API and its meanings: mercury/engine.p
 
 from __future__ import annotations
 
-import queue
 import threading
 import time
+from collections import deque
 from typing import Callable
 
 from ..cache import CacheManager, PageHasher
@@ -28,18 +28,53 @@ SamplingParams = _core.SamplingParams
 Sink = Callable[[StreamEvent], None]
 
 
-def autosize_blocks(cfg: EngineConfig, kv_bytes_per_token: int, device) -> int:
-    """Pages that fit in the memory that is free once the weights are resident
-    (reference: mercury/config.py:164-185)."""
+# What the captured decode graphs may cost beside the buffers they share: the launch records
+# of a few hundred kernels each (measured well under a megabyte a graph).
+GRAPH_RECORD_BYTES = 2 << 20
+
+
+def autosize_blocks(cfg: EngineConfig, kv_bytes_per_token: int, device, reserve_bytes: int = 0) -> int:
+    """Pages that fit in the memory that is free once the weights are resident, after
+    `reserve_bytes` are set aside for what is allocated later: the workspace and index buffer
+    of the largest step, the buffers the captured graphs share, and the graphs themselves
+    (reference: mercury/config.py:164-185, which reserves for weights not yet loaded; here
+    the weights are loaded when this is called, and the reservation is for the rest)."""
     import torch
 
     free, _total = torch.cuda.mem_get_info(torch.device(device))
-    budget = int(free * cfg.gpu_memory_fraction)
+    budget = int(max(0, free - reserve_bytes) * cfg.gpu_memory_fraction)
     per_page = max(1, kv_bytes_per_token * cfg.block_size)
     pages = budget // per_page
     if pages < 1:
-        raise RuntimeError(f"only {free / 2**30:.1f} GiB are free; there is no room for a cache")
+        raise RuntimeError(
+            f"only {free / 2**30:.1f} GiB are free and {reserve_bytes / 2**30:.1f} GiB are set "
+            f"aside for the steps' buffers; there is no room for a cache")
     return pages
+
+
+class _Inbox:
+    """What other threads ask of the loop, in the order they asked: the loop takes everything
+    at once at the top of a pass, and sleeps on the inbox when it has nothing to run."""
+
+    def __init__(self):
+        self._items: deque = deque()
+        self._ready = threading.Condition()
+
+    def post(self, kind: str, payload) -> None:
+        with self._ready:
+            self._items.append((kind, payload))
+            self._ready.notify()
+
+    def take_all(self) -> list:
+        with self._ready:
+            items = list(self._items)
+            self._items.clear()
+        return items
+
+    def wait(self, timeout: float) -> None:
+        with self._ready:
+            if not self._items:
+                self._ready.wait(timeout)
 
 
 class Engine:
@@ -47,7 +82,12 @@ class Engine:
     `cfg.random_weights`, builds the model that `model_config` (a ``config.json`` as a dict) or
     the ``config.json`` at `cfg.model` describes and draws its weights from `cfg.weight_seed`.
     Tests pass `executor` (anything with `execute(plan)`) and, with it, the cache manager it
-    checks against."""
+    checks against.
+
+    One pass of the loop is `step()`.  Whoever calls it owns the loop: the caller's own
+    thread (`step`, `run_until_idle`, `generate`), or, after `start()`, a thread of the
+    engine's that runs passes until `shutdown()`.  `submit` and `abort` may come from any
+    thread either way; they only post to the inbox."""
 
     def __init__(self, cfg: EngineConfig, executor=None, manager: CacheManager | None = None,
                  clock: Callable[[], float] = time.perf_counter, eos_token_ids=None,
@@ -70,12 +110,13 @@ class Engine:
             max_step_records=cfg.max_step_records)
         self.sched = self.core.scheduler
         self.metrics = self.core      # counters, summary(), step_records()
-        self._commands: queue.Queue = queue.Queue()
-        self._sinks: dict = {}
-        self._wake, self._stop = threading.Event(), threading.Event()
-        self._thread = None
-        self._lock = threading.Lock()
-        self._submitted = 0
+        self._inbox = _Inbox()
+        self._listeners: dict = {}                  # request id -> sink
+        self._listeners_guard = threading.Lock()
+        self._accepted = 0                          # requests submit() has queued so far
+        self._worker: threading.Thread | None = None
+        self._serving = threading.Event()
+        self._worker_error: BaseException | None = None
 
     @property
     def eos_ids(self) -> set:
@@ -115,73 +156,134 @@ class Engine:
         if model.max_positions:
             cfg.validate_against(model.max_positions)
         has_state = any(layer.mixer.state_spec() is not None for layer in model.layers)
+        graph_batch = min(cfg.max_graph_batch, cfg.max_running)
         if cfg.num_blocks < 0:
-            cfg.num_blocks = autosize_blocks(cfg, model.kv_bytes_per_token(cfg.torch_dtype), device)
+            reserve = Engine.reserve_bytes(model, cfg, device, graph_batch)
+            cfg.num_blocks = autosize_blocks(cfg, model.kv_bytes_per_token(cfg.torch_dtype), device,
+                                             reserve)
             cfg.validate_against(model.max_positions or cfg.max_model_len)
         manager = CacheManager(model.cache_slots, cfg.num_blocks, cfg.block_size, cfg.max_running,
                                has_state)
         runner = ModelRunner(model, manager, cfg.torch_dtype, device, cfg.max_model_len,
-                             use_graphs=cfg.use_graphs)
+                             use_graphs=cfg.use_graphs, max_graph_batch=graph_batch,
+                             max_graphs=cfg.max_graphs)
         return (GpuExecutor(runner, Sampler(cfg.seed), lookahead=cfg.lookahead), manager,
                 model.eos_token_ids)
+
+    @staticmethod
+    def reserve_bytes(model, cfg: EngineConfig, device, graph_batch: int) -> int:
+        """Device memory the engine will allocate after the cache: measured on the model's
+        program, built over caches without pages, for the largest step the scheduler can plan
+        under `prefill_budget` and `max_running` and for the largest captured decode step."""
+        import torch
+
+        from ..kernels import lib as kernel_lib
+        from .runner import ModelRunner, sizing_caches
+
+        kernel_lib.load("core")
+        if cfg.torch_dtype == torch.bfloat16:
+            kernel_lib.load("mfma")
+        # the groups as the cache manager will form them, from a manager of one page
+        has_state = any(layer.mixer.state_spec() is not None for layer in model.layers)
+        sizing = CacheManager(model.cache_slots, 1, cfg.block_size, cfg.max_running, has_state)
+        groups = {slot: sizing.group_of(slot) for slot in model.cache_slots}
+        model.prepare(cfg.max_model_len, device)
+        caches = sizing_caches(model, groups, cfg.block_size, cfg.torch_dtype, device)
+        states = {i: torch.empty((0, *layer.mixer.state_spec().shape),
+                                 dtype=layer.mixer.state_spec().dtype, device=device)
+                  for i, layer in enumerate(model.layers) if layer.mixer.state_spec() is not None}
+        program = model.compile(caches, states)
+        needs = ModelRunner.step_needs(program, max(1, sizing.num_groups), cfg.block_size,
+                                       cfg.max_model_len, min(cfg.prefill_budget, cfg.max_model_len),
+                                       cfg.max_running, graph_batch if cfg.use_graphs else 0)
+        graphs = cfg.max_graphs * GRAPH_RECORD_BYTES if cfg.use_graphs else 0
+        # buffers grow by a quarter beyond what a step asks for
+        return int(1.25 * (needs["eager_workspace"] + needs["eager_ints"])
+                   + needs["graph_workspace"] + needs["graph_ints"] + graphs)
 
     # ---------------------------------------------------------------- lifecycle
 
     def start(self) -> None:
-        """Run the loop on a thread of its own until `shutdown`."""
-        if self._thread is not None:
+        """Hand the loop to a thread of the engine's own, until `shutdown`."""
+        if self._worker is not None:
             return
-        self._thread = threading.Thread(target=self._run, name="mercury-amd-engine", daemon=True)
-        self._thread.start()
+        self._serving.set()
+        self._worker_error = None
+        self._worker = threading.Thread(target=self._serve, name="mercury-amd-loop", daemon=True)
+        self._worker.start()
 
     def shutdown(self, timeout: float = 5.0) -> None:
-        self._stop.set()
-        self._wake.set()
-        if self._thread is not None:
-            self._thread.join(timeout)
-            self._thread = None
+        """Stop the engine's thread after the pass it is in.  Raises what the thread died of,
+        if it died, and TimeoutError when it does not come back in `timeout` seconds."""
+        worker, self._worker = self._worker, None
+        self._serving.clear()
+        if worker is None:
+            return
+        self._inbox.post("wake", None)
+        worker.join(timeout)
+        if worker.is_alive():
+            self._worker = worker
+            raise TimeoutError(f"the engine's thread did not stop within {timeout} s")
+        if self._worker_error is not None:
+            raise self._worker_error
 
-    def _run(self) -> None:
-        while not self._stop.is_set():
-            if self.step() is None:
-                self._wake.wait(self.cfg.idle_sleep_s)
-                self._wake.clear()
+    def _serve(self) -> None:
+        try:
+            while self._serving.is_set():
+                if self.step() is None:
+                    self._inbox.wait(self.cfg.idle_sleep_s)
+        except BaseException as error:      # kept for shutdown() to raise on the caller's thread
+            self._worker_error = error
+            self._serving.clear()
 
     # ---------------------------------------------------------------- client side
 
     def submit(self, rid: str, prompt_ids: list, max_tokens: int, sink: Sink,
                params: SamplingParams | None = None, session_id: str | None = None,
                arrival: float | None = None) -> None:
-        """Queue a request.  A request that can never run (an empty prompt, more tokens than
-        one request may hold) is answered at once with an "error" event and not queued."""
-        arrival = self.clock() if arrival is None else arrival
-        why = self.core.refusal(len(prompt_ids), max_tokens)
-        if why is not None:
+        """Queue a request; its events go to `sink`, called on the loop's thread.  A request
+        that can never run (an empty prompt, more tokens than one request may hold) gets an
+        "error" event here and now, and is not queued."""
+        now = self.clock()
+        refusal = self.core.refusal(len(prompt_ids), max_tokens)
+        if refusal is not None:
             self.core.count_rejected()
-            sink(StreamEvent(rid=rid, kind="error", message=why, t=self.clock()))
+            sink(StreamEvent(rid=rid, kind="error", message=refusal, t=now))
             return
-        request = self.core.make_request(rid, prompt_ids, max_tokens, arrival, params, session_id)
-        with self._lock:
-            self._sinks[rid] = sink
-            self._submitted += 1
-        self._commands.put(("add", request))
-        self._wake.set()
+        request = self.core.make_request(rid, prompt_ids, max_tokens,
+                                         now if arrival is None else arrival, params, session_id)
+        with self._listeners_guard:
+            self._listeners[rid] = sink
+            self._accepted += 1
+        self._inbox.post("add", request)
 
     def abort(self, rid: str) -> None:
-        self._commands.put(("abort", rid))
-        self._wake.set()
+        """Ask the loop to end request `rid`; its sink receives the closing event."""
+        self._inbox.post("abort", rid)
+
+    def run_until_idle(self) -> int:
+        """On the caller's thread: passes until nothing is queued or running.  Returns how many
+        passes ran a step."""
+        if self._worker is not None:
+            raise RuntimeError("the engine's own thread runs the loop; shutdown() first")
+        ran = 0
+        self._take_commands()
+        while self.sched.has_work():
+            if self.step() is not None:
+                ran += 1
+        return ran
 
     def generate(self, prompts: list, params=None, max_tokens: int = 16) -> list:
         """Blocking: run every prompt (a list of token ids each) to completion and return the
         generated token ids, one list per prompt.  `params` is one SamplingParams for all or a
         list with one per prompt; `max_tokens` likewise an int or a list."""
-        if self._thread is not None:
+        if self._worker is not None:
             raise RuntimeError("generate() drives the loop itself; do not call it after start()")
         n = len(prompts)
         params = params if isinstance(params, list) else [params] * n
         budgets = max_tokens if isinstance(max_tokens, list) else [max_tokens] * n
         outputs, errors = [[] for _ in range(n)], {}
-        base = self._submitted
+        first = self._accepted
 
         def sink_for(i):
             def sink(event):
@@ -192,13 +294,10 @@ class Engine:
             return sink
 
         for i, prompt in enumerate(prompts):
-            self.submit(f"gen-{base + i}", prompt, budgets[i], sink_for(i),
-                        params=params[i])
+            self.submit(f"gen-{first + i}", prompt, budgets[i], sink_for(i), params=params[i])
         if errors:
             raise ValueError("; ".join(f"prompt {i}: {m}" for i, m in sorted(errors.items())))
-        self._drain_commands()
-        while self.sched.has_work():
-            self.step()
+        self.run_until_idle()
         return outputs
 
     # ---------------------------------------------------------------- the loop
@@ -207,7 +306,7 @@ class Engine:
         """One pass: take commands, plan, run the plan, apply its results.  Returns the step's
         record, or None when there was nothing to run."""
         started = time.perf_counter()
-        self._drain_commands()
+        self._take_commands()
         plan, events = self.core.schedule(self.clock())
         self._deliver(events)
         if not plan:
@@ -222,32 +321,32 @@ class Engine:
                                   getattr(result, "device_seconds", 0.0),
                                   time.perf_counter() - started)
 
-    def _drain_commands(self) -> None:
-        while True:
-            try:
-                kind, payload = self._commands.get_nowait()
-            except queue.Empty:
-                return
+    def _take_commands(self) -> None:
+        for kind, payload in self._inbox.take_all():
             if kind == "add":
                 self.core.add(payload)
-                continue
-            events = self.core.abort(payload, self.clock())
-            if not events:
-                with self._lock:
-                    self._sinks.pop(payload, None)    # already finished, or never queued
-            self._deliver(events)
+            elif kind == "abort":
+                events = self.core.abort(payload, self.clock())
+                if not events:
+                    # finished already, or never queued: nobody to tell
+                    with self._listeners_guard:
+                        self._listeners.pop(payload, None)
+                self._deliver(events)
 
     def _deliver(self, events: list) -> None:
         for event in events:
-            closing = event.kind == "done"
-            with self._lock:
-                sink = self._sinks.pop(event.rid, None) if closing else self._sinks.get(event.rid)
+            with self._listeners_guard:
+                if event.kind == "done":
+                    sink = self._listeners.pop(event.rid, None)
+                else:
+                    sink = self._listeners.get(event.rid)
             if sink is None:
                 continue
             try:
                 sink(event)
             except Exception:
-                self.abort(event.rid)   # a sink that raises means nobody is listening any more
+                # a sink that raises has stopped listening: end its request
+                self.abort(event.rid)
 
     # ---------------------------------------------------------------- reporting
 
@@ -264,11 +363,14 @@ class Engine:
             "allocator": self.manager.snapshot(),
             "scheduler": self.sched.snapshot(),
             "engine": self.core.summary(),
-            "submitted": self._submitted,
+            "submitted": self._accepted,
+            "executor": self.executor.snapshot() if hasattr(self.executor, "snapshot") else {},
         }
 
     def leaked_blocks(self) -> int:
+        """Pages held although no request is live (0 when the bookkeeping is whole)."""
         return self.manager.leaked_pages()
 
     def drain_request_records(self) -> list:
+        """The records of requests finished since the last call."""
         return self.core.drain_finished()

@@ -100,7 +100,7 @@ class GpuExecutor:
         self.model_config = runner.model.config
         self.kv_bytes = runner.kv_bytes
         manager = runner.manager
-        self.lookahead = (bool(lookahead) and runner.use_graphs and runner.program is not None
+        self.lookahead = (bool(lookahead) and runner.use_graphs
                           and not runner.states and all(g.window is None for g in manager.groups))
         self._ahead: _Ahead | None = None
         self._ring = _PinnedRing(max(256, runner.max_graph_batch))
@@ -175,4 +175,5 @@ class GpuExecutor:
         r = self.runner
         return {"device": str(r.device), "dtype": str(r.dtype).replace("torch.", ""),
                 "kv_bytes": r.kv_bytes, "cache_slots": len(r.kv),
-                "kv_bytes_per_token": r.kv_bytes_per_token()}
+                "kv_bytes_per_token": r.kv_bytes_per_token(), "memory": r.memory_report(),
+                "lookahead": dict(self.stats)}

@@ -56,11 +56,13 @@ HIPCC_FLAGS = [
 ]
 
 
-# The host core: C++ (pybind11) for the cache manager, the scheduler, step packing and the
-# launch sequence of a step.  Compiled with the host compiler; it reaches the kernel libraries
+# The host core: C++ (pybind11) for the cache manager, the scheduler, step packing, the walk
+# over a step's program and the built-in operations' launch sequences.  Compiled with the host compiler; it reaches the kernel libraries
 # and the HIP runtime through dlopen/dlsym, so it links against neither.
 HOST_NAME = "host"
-HOST_DIR = CSRC / "host"
+HOST_DIR = CSRC / "host"     # what knows no operation: cache, scheduler, packer, program walk
+OPS_DIR = CSRC / "ops"       # the built-in operations, their launch sequences and choices
+KERNEL_HEADER = CSRC / "mercury_kernels.h"
 HOST_FLAGS = ["-O2", "-std=c++17", "-fPIC", "-fvisibility=hidden", "-ffp-contract=off", "-pthread",
               "-D__HIP_PLATFORM_AMD__", "-Wall", "-Wno-unused-function"]
 
@@ -103,8 +105,66 @@ def library_name(name: str) -> str:
 
 def _sources(name: str) -> list:
     if name == HOST_NAME:
-        return sorted(HOST_DIR.glob("*.cc"))
+        return sorted(HOST_DIR.glob("*.cc")) + sorted(OPS_DIR.glob("*.cc"))
     return [CSRC / s for s in LIBRARIES[name]]
+
+
+def _host_headers() -> list:
+    return sorted(HOST_DIR.glob("*.h")) + sorted(OPS_DIR.glob("*.h"))
+
+
+def kernel_prototypes() -> dict:
+    """library name -> [(function name, return type, [parameter types])], read from the one
+    declaration of the kernel libraries' C interface (``csrc/mercury_kernels.h``).  A line
+    ``// @library NAME`` says which library the declarations after it belong to; what stands
+    before the first such line is in every library."""
+    import re
+
+    out = {name: [] for name in LIBRARIES}
+    current = None
+    text = KERNEL_HEADER.read_text()
+    # keep the markers, drop every other comment
+    text = re.sub(r"//\s*@library\s+(\w+).*", r"@library \1;", text)
+    text = re.sub(r"//.*", "", text)
+    text = re.sub(r"^\s*#.*$", "", text, flags=re.M)
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    for statement in text.split(";"):
+        statement = " ".join(statement.split())
+        marker = re.search(r"@library (\w+)$", statement)
+        if marker:
+            current = marker.group(1)
+            if current not in out:
+                raise BuildError(f"{KERNEL_HEADER.name} names an unknown library {current!r}")
+            continue
+        match = re.search(r"([\w ]+?[\w\*]) ?\b(mk_\w+) ?\((.*)\)$", statement)
+        if not match:
+            continue
+        returns, name, params = match.group(1).strip(), match.group(2), match.group(3).strip()
+        returns = returns.split("{")[-1].strip()          # the extern "C" brace
+        types = []
+        if params and params != "void":
+            for param in params.split(","):
+                param = param.strip()
+                types.append("pointer" if "*" in param else " ".join(param.split()[:-1]))
+        for lib in ([current] if current else list(out)):
+            out[lib].append((name, returns, types))
+    return out
+
+
+def _write_kernel_names(folder: Path) -> Path:
+    """The lists of entry points by library as X-macros, for the host core's table of function
+    pointers (their types come from the declarations themselves, by decltype)."""
+    common = {"mk_last_error", "mk_abi_version"}
+    lines = ["// Written by the build from mercury_kernels.h; not a source file."]
+    for lib, protos in kernel_prototypes().items():
+        names = " ".join(f"X({name})" for name, _, _ in protos if name not in common)
+        lines.append(f"#define MK_{lib.upper()}_FUNCTIONS(X) {names}")
+    folder.mkdir(parents=True, exist_ok=True)
+    path = folder / "kernel_names.inc"
+    text = "\n".join(lines) + "\n"
+    if not path.is_file() or path.read_text() != text:
+        path.write_text(text)
+    return path
 
 
 def source_hash(name: str) -> str:
@@ -113,7 +173,7 @@ def source_hash(name: str) -> str:
     if name == HOST_NAME:
         digest.update(" ".join(HOST_FLAGS).encode())
         digest.update(sys.version.encode())
-        headers += sorted(HOST_DIR.glob("*.h"))
+        headers += _host_headers()
     else:
         digest.update(" ".join(HIPCC_FLAGS).encode())
     for path in _sources(name) + headers:
@@ -177,14 +237,14 @@ def _rocm_root() -> Path:
     raise BuildError("the ROCm headers were not found (looked at $ROCM_PATH and /opt/rocm)")
 
 
-def _host_commands(sources: list, objects: list, target: Path) -> tuple:
+def _host_commands(sources: list, objects: list, target: Path, generated: Path) -> tuple:
     import sysconfig
 
     import pybind11
 
     cxx, rocm = _host_compiler(), _rocm_root()
     includes = ["-I", pybind11.get_include(), "-I", sysconfig.get_paths()["include"],
-                "-I", str(rocm / "include"), "-I", str(CSRC), "-I", str(HOST_DIR)]
+                "-I", str(rocm / "include"), "-I", str(CSRC), "-I", str(generated)]
     compiles = [[cxx, *HOST_FLAGS, *includes, "-c", str(src), "-o", str(obj)]
                 for src, obj in zip(sources, objects)]
     # No HIP runtime is linked: the core finds, at run time, the one the process already uses.
@@ -212,7 +272,9 @@ def build_library(name: str, force: bool = False, verbose: bool = True) -> Path:
     if name == HOST_NAME:
         if verbose:
             _say(f"compiling the host core: {len(sources)} sources -> {out_dir}")
-        compiles, link = _host_commands(sources, objects, partial)
+        generated = obj_dir / "include"
+        _write_kernel_names(generated)
+        compiles, link = _host_commands(sources, objects, partial, generated)
     else:
         hipcc = _hipcc()
         if verbose:
@@ -222,7 +284,7 @@ def build_library(name: str, force: bool = False, verbose: bool = True) -> Path:
         link = [hipcc, f"--offload-arch={ARCH}", "-shared", "-fPIC", "-fno-gpu-rdc", "-o",
                 str(partial), *map(str, objects)]
     threads, errors = [], []
-    headers = b"".join(p.read_bytes() for p in sorted(CSRC.glob("*.h")) + sorted(HOST_DIR.glob("*.h")))
+    headers = b"".join(p.read_bytes() for p in sorted(CSRC.glob("*.h")) + _host_headers())
     for src, obj, cmd in zip(sources, objects, compiles):
         # An object whose command, source and headers are what they were is kept, unless the
         # caller asked for everything to be compiled again.

@@ -11,51 +11,25 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 from . import build
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
-P, I, F, L = c_void_p, c_int, c_float, c_longlong
+_CTYPES = {"pointer": c_void_p, "int": c_int, "float": c_float, "long long": c_longlong,
+           "unsigned long long": c_ulonglong, "hipStream_t": c_void_p, "const char*": c_char_p}
 
-# name -> argument types (every function returns int)
-_SIGNATURES = {
-    "core": {
-        "mk_embed": [P, P, I, P, I, I, I, P],
-        "mk_rmsnorm": [P, P, I, L, P, I, F, P, P, I, I, I, P],
-        "mk_silu_mul": [P, P, I, I, I, P],
-        "mk_rope_kv_write": [P, I, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, P],
-        "mk_linear_generic": [P, P, I, P, I, P, I, I, I, I, I, I, I, P],
-        "mk_attention_generic": [P, I, P, I, P, P, I, P, P, P, I, I, I, I, I, F, I, I, P],
-        "mk_qkv_finish": [P, I, L, P, I, P, I, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
-        "mk_argmax": [P, I, I, L, P, P, P],
-        "mk_argmax_static_max_rows": [],
-        "mk_argmax_static": [P, I, I, L, P, P],
-        "mk_sample_scratch_bytes": [I, I],
-        "mk_sample": [P, I, I, L, P, P, P, P, P, P],
-        "mk_fill_normal": [P, I, L, c_ulonglong, F, F, P],
-    },
-    "mfma": {
-        "mk_linear_skinny_slices": [I, I, I],
-        "mk_linear_skinny": [P, P, P, I, I, I, I, P],
-        "mk_linear_skinny_unsplit": [I, I, I],
-        "mk_linear_skinny_acc": [P, P, P, I, P, I, I, I, P],
-        "mk_gated_skinny": [P, P, P, I, I, I, P],
-        "mk_qkv_skinny": [P, P, P, I, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, P],
-        "mk_qkv_tiled": [P, P, P, I, P, P, P, I, P, P, P, I, P, P, I, I, I, I, I, I, I, I, P],
-        "mk_gated_tiled_config": [I, I, I],
-        "mk_gated_tiled": [P, P, P, I, I, I, I, P],
-        "mk_linear_tiled_slices": [I, I, I],
-        "mk_linear_tiled_partials": [P, P, P, I, I, I, I, P],
-        "mk_linear_tiled_configs": [],
-        "mk_linear_tiled_config": [I, I, I, I],
-        "mk_linear_tiled": [P, P, P, I, P, I, I, I, I, I, I, I, P],
-        "mk_attention_mfma_supported": [I, I],
-        "mk_attention_mfma_max_rows": [I],
-        "mk_attention_mfma_staged": [I, I],
-        "mk_attention_mfma_wide": [I],
-        "mk_attention_mfma": [P, I, P, I, P, P, P, P, I, P, P, P, I, I, I, I, I, F, I, I, I, I, I, P, P, P],
-    },
-}
 
-_RETURNS_SIZE = {"mk_sample_scratch_bytes"}    # byte counts; everything else returns int
+def _signatures(name: str) -> dict:
+    """function name -> (return ctype, [argument ctypes]) for the library `name`, from the
+    declarations in ``csrc/mercury_kernels.h``: the header is the one place a signature is
+    written down."""
+    out = {}
+    for fn_name, returns, params in build.kernel_prototypes()[name]:
+        try:
+            out[fn_name] = (_CTYPES[returns], [_CTYPES[p] for p in params])
+        except KeyError as e:
+            raise KernelLibraryError(
+                f"{fn_name}: mercury_kernels.h uses a type this loader does not know: {e}") from None
+    return out
+
 
 _loaded: dict = {}
 
@@ -79,17 +53,20 @@ def load(name: str = "core") -> ctypes.CDLL:
         lib = ctypes.CDLL(str(path))
     except OSError as e:
         raise KernelLibraryError(f"cannot load {path}: {e}") from e
-    lib.mk_last_error.restype = c_char_p
-    lib.mk_last_error.argtypes = []
     lib.mk_abi_version.restype = c_int
+    lib.mk_abi_version.argtypes = []
     if lib.mk_abi_version() != ABI_VERSION:
         raise KernelLibraryError(
             f"{path} has ABI {lib.mk_abi_version()}, this package expects {ABI_VERSION}; rebuild"
         )
-    for fn_name, argtypes in _SIGNATURES[name].items():
-        fn = getattr(lib, fn_name)
+    for fn_name, (restype, argtypes) in _signatures(name).items():
+        try:
+            fn = getattr(lib, fn_name)
+        except AttributeError:
+            raise KernelLibraryError(
+                f"{path} has no entry point {fn_name}; rebuild the kernel libraries") from None
         fn.argtypes = argtypes
-        fn.restype = c_longlong if fn_name in _RETURNS_SIZE else c_int
+        fn.restype = restype
     # The host core launches a step's kernels itself and decides which kernel runs what: it
     # opens the same library.
     from ..hostcore import core

@@ -73,76 +73,13 @@ def _i32(t: torch.Tensor, name: str) -> None:
         raise KernelArgumentError(f"{name} must be int32, got {t.dtype}")
 
 
-# ------------------------------------------------------------------------------ row-wise ops
-
-
-def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t] = table[ids[t]] as float32 [T, H]."""
-    _dev(ids, table, out)
-    _i32(ids, "ids")
-    tokens, (vocab, hidden) = ids.shape[0], table.shape
-    if out is None:
-        out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
-    if out.shape != (tokens, hidden) or out.dtype != torch.float32:
-        raise KernelArgumentError("embed: out must be float32 [T, H]")
-    lib = _lib.load("core")
-    _lib.check(lib, lib.mk_embed(_ptr(ids), _ptr(table), dtype_code(table.dtype), _ptr(out),
-                                 tokens, hidden, vocab, _stream()), "embed")
-    return out
-
-
-def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
-            rows: torch.Tensor | None = None, partials: torch.Tensor | None = None,
-            out: torch.Tensor | None = None) -> torch.Tensor:
-    """RMSNorm of the float32 residual stream h [T, H] into `out_dtype`.
-
-    `partials` [P, T, H] float32 are first summed into h (and h is updated); `rows` selects
-    and orders the rows to normalise.
-    """
-    _dev(h, weight, rows, partials, out)
-    if h.dtype != torch.float32 or h.dim() != 2:
-        raise KernelArgumentError("rmsnorm: h must be float32 [T, H]")
-    tokens, hidden = h.shape
-    if weight.shape != (hidden,):
-        raise KernelArgumentError(f"rmsnorm: weight {tuple(weight.shape)} does not match H={hidden}")
-    n_partials, stride = 0, 0
-    if partials is not None:
-        if partials.dtype != torch.float32 or partials.shape[1:] != h.shape:
-            raise KernelArgumentError("rmsnorm: partials must be float32 [P, T, H]")
-        n_partials, stride = partials.shape[0], tokens * hidden
-    out_rows = tokens
-    if rows is not None:
-        _i32(rows, "rows")
-        out_rows = rows.shape[0]
-    if out is None:
-        out = torch.empty((out_rows, hidden), dtype=out_dtype, device=h.device)
-    if out.shape != (out_rows, hidden) or out.dtype != out_dtype:
-        raise KernelArgumentError("rmsnorm: out has the wrong shape or dtype")
-    lib = _lib.load("core")
-    _lib.check(lib, lib.mk_rmsnorm(_ptr(h), _ptr(partials), n_partials, stride, _ptr(weight),
-                                   dtype_code(weight.dtype), float(eps), _ptr(rows), _ptr(out),
-                                   dtype_code(out_dtype), out_rows, hidden, _stream()), "rmsnorm")
-    return out
-
-
-def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
-    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up [T, 2I]."""
-    _dev(gate_up, out)
-    tokens, two_i = gate_up.shape
-    if two_i % 2:
-        raise KernelArgumentError("silu_mul: the last dimension must be even")
-    inter = two_i // 2
-    if out is None:
-        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
-    if out.shape != (tokens, inter) or out.dtype != gate_up.dtype:
-        raise KernelArgumentError("silu_mul: out has the wrong shape or dtype")
-    lib = _lib.load("core")
-    _lib.check(lib, lib.mk_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), tokens,
-                                    inter, _stream()), "silu_mul")
-    return out
-
-
-# --------------------------------------------------------------------------------- projection
+# --------------------------------------------------------------------------------- plumbing
+#
+# Which kernel runs a projection, a q/k/v projection or an attention of given sizes, and with
+# which arguments, is written down once, in the host core (csrc/ops/launch.cc, with the
+# decisions and the measurements behind them in csrc/ops/dispatch.cc).  The functions below
+# check shapes, allocate results and call those launch sequences by device address; a step's
+# program calls the same ones.
 
 
 def _core():
@@ -160,11 +97,110 @@ def _ensure(x: torch.Tensor):
     return _core()
 
 
-SKINNY_MAX_ROWS = 64           # most rows the fused skinny q/k/v kernel takes
+class Scratch:
+    """Memory for what a launch sequence allocates by itself (results and temporaries): one
+    byte tensor, asked for once the sequence knows how much it needs; results are views of
+    it, which keep it alive."""
 
-# Which kernel runs a projection, a q/k/v projection or an attention of given sizes is decided
-# in the host core (csrc/host/dispatch.cc), where the measurements behind every threshold are
-# written down; the step programs ask the same functions.
+    def __init__(self, device):
+        self.device, self.tensor = device, None
+
+    def __call__(self, nbytes: int) -> int:
+        self.tensor = torch.empty(int(nbytes), dtype=torch.uint8, device=self.device)
+        return self.tensor.data_ptr()
+
+    def view(self, address: int, shape: tuple, dtype: torch.dtype) -> torch.Tensor:
+        count = 1
+        for n in shape:
+            count *= n
+        if count == 0 or self.tensor is None:
+            return torch.empty(shape, dtype=dtype, device=self.device)
+        offset = address - self.tensor.data_ptr()
+        size = count * torch.empty((), dtype=dtype).element_size()
+        if offset < 0 or offset + size > self.tensor.numel():
+            raise RuntimeError("a launch sequence's result lies outside its scratch memory")
+        return self.tensor[offset:offset + size].view(dtype).view(*shape)
+
+
+# ------------------------------------------------------------------------------ row-wise ops
+
+
+def embed(ids: torch.Tensor, table: torch.Tensor, out: torch.Tensor | None = None,
+          scale: float = 1.0) -> torch.Tensor:
+    """out[t] = table[ids[t]] * scale as float32 [T, H]."""
+    _dev(ids, table, out)
+    _i32(ids, "ids")
+    tokens, (vocab, hidden) = ids.shape[0], table.shape
+    if out is None:
+        out = torch.empty((tokens, hidden), dtype=torch.float32, device=table.device)
+    if out.shape != (tokens, hidden) or out.dtype != torch.float32:
+        raise KernelArgumentError("embed: out must be float32 [T, H]")
+    _ensure(table).launch_embed(_ptr(ids), _ptr(table), dtype_code(table.dtype), _ptr(out), tokens,
+                                hidden, vocab, float(scale), _stream())
+    return out
+
+
+def rmsnorm(h: torch.Tensor, weight: torch.Tensor, eps: float, out_dtype: torch.dtype,
+            rows: torch.Tensor | None = None, partials: torch.Tensor | None = None,
+            out: torch.Tensor | None = None) -> torch.Tensor:
+    """RMSNorm of the float32 residual stream h [T, H] into `out_dtype`.
+
+    `partials` [P, T, H] float32 are first summed into h (and h is updated); `rows` selects
+    and orders the rows to normalise.
+    """
+    _dev(h, weight, rows, partials, out)
+    if h.dtype != torch.float32 or h.dim() != 2:
+        raise KernelArgumentError("rmsnorm: h must be float32 [T, H]")
+    tokens, hidden = h.shape
+    if weight.shape != (hidden,):
+        raise KernelArgumentError(f"rmsnorm: weight {tuple(weight.shape)} does not match H={hidden}")
+    n_partials = 0
+    if partials is not None:
+        if partials.dtype != torch.float32 or partials.shape[1:] != h.shape:
+            raise KernelArgumentError("rmsnorm: partials must be float32 [P, T, H]")
+        n_partials = partials.shape[0]
+    out_rows = tokens
+    if rows is not None:
+        _i32(rows, "rows")
+        out_rows = rows.shape[0]
+    if out is None:
+        out = torch.empty((out_rows, hidden), dtype=out_dtype, device=h.device)
+    if out.shape != (out_rows, hidden) or out.dtype != out_dtype:
+        raise KernelArgumentError("rmsnorm: out has the wrong shape or dtype")
+    _ensure(h).launch_rmsnorm(_ptr(h), tokens, hidden, _ptr(partials), n_partials, _ptr(weight),
+                              dtype_code(weight.dtype), float(eps), _ptr(rows), out_rows,
+                              _ptr(out), dtype_code(out_dtype), _stream())
+    return out
+
+
+def silu_mul(gate_up: torch.Tensor, out: torch.Tensor | None = None) -> torch.Tensor:
+    """out[t, i] = silu(gate_up[t, i]) * gate_up[t, I + i] for gate_up [T, 2I]."""
+    _dev(gate_up, out)
+    tokens, two_i = gate_up.shape
+    if two_i % 2:
+        raise KernelArgumentError("silu_mul: the last dimension must be even")
+    inter = two_i // 2
+    if out is None:
+        out = torch.empty((tokens, inter), dtype=gate_up.dtype, device=gate_up.device)
+    if out.shape != (tokens, inter) or out.dtype != gate_up.dtype:
+        raise KernelArgumentError("silu_mul: out has the wrong shape or dtype")
+    _ensure(gate_up).launch_silu_mul(_ptr(gate_up), _ptr(out), dtype_code(gate_up.dtype), tokens,
+                                     inter, _stream())
+    return out
+
+
+def logit_cap(logits: torch.Tensor, cap: float) -> torch.Tensor:
+    """logits <- cap * tanh(logits / cap), in place (float32)."""
+    _dev(logits)
+    if logits.dtype != torch.float32 or cap <= 0:
+        raise KernelArgumentError("logit_cap: float32 logits and a positive cap are required")
+    _ensure(logits).launch_logit_cap(_ptr(logits), logits.numel(), float(cap), _stream())
+    return logits
+
+
+# --------------------------------------------------------------------------------- projection
+
+SKINNY_MAX_ROWS = 64           # most rows the fused skinny q/k/v kernel takes
 
 
 def wants_partials(x: torch.Tensor, w: torch.Tensor) -> bool:
@@ -190,15 +226,10 @@ def linear_partials(x: torch.Tensor, w: torch.Tensor) -> torch.Tensor:
         raise KernelArgumentError(f"linear_partials: x {tuple(x.shape)} / W {tuple(w.shape)} not eligible")
     m, k = x.shape
     n = w.shape[0]
-    lib = _lib.load("mfma")
-    skinny, slices = _core().plan_partials(m, n, k)
-    out = torch.empty((slices, m, n), dtype=torch.float32, device=x.device)
-    if skinny:
-        code = lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream())
-    else:
-        code = lib.mk_linear_tiled_partials(_ptr(x), _ptr(w), _ptr(out), m, n, k, slices, _stream())
-    _lib.check(lib, code, "linear_partials")
-    return out
+    scratch = Scratch(x.device)
+    address, slices = _ensure(x).launch_linear_partials(_ptr(x), m, _ptr(w), n, k,
+                                                        dtype_code(x.dtype), scratch, _stream())
+    return scratch.view(address, (slices, m, n), torch.float32)
 
 
 def fuses_gating(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
@@ -211,27 +242,22 @@ def fuses_gating(x: torch.Tensor, w_gate_up: torch.Tensor) -> bool:
 
 def gated_projection(x: torch.Tensor, w_gate_up: torch.Tensor,
                      tile_config: int | None = None) -> torch.Tensor:
-    """act = silu(x Wg^T) * (x Wu^T) for bfloat16 x and W = [Wg | Wu] stacked [2 I, K]: one
+    """act = silu(x Wg^T) * (x Wu^T) for W = [Wg | Wu] stacked [2 I, K]: for bfloat16 one
     kernel on the matrix cores, the gating in the projection's epilogue (the skinny kernel for
     few rows, the tiled one for many; `tile_config` forces the tiled one with that tile
-    configuration, -1 for its own choice)."""
+    configuration, -1 for its own choice); otherwise the projection and the gating kernel."""
     _dev(x, w_gate_up)
-    if not fuses_gating(x, w_gate_up) or x.shape[1] != w_gate_up.shape[1]:
+    if x.shape[1] != w_gate_up.shape[1] or w_gate_up.shape[0] % 2:
+        raise KernelArgumentError("gated_projection: operands do not match")
+    if tile_config is not None and not fuses_gating(x, w_gate_up):
         raise KernelArgumentError("gated_projection: operands not eligible")
     m, k = x.shape
     inter = w_gate_up.shape[0] // 2
-    act = torch.empty((m, inter), dtype=torch.bfloat16, device=x.device)
-    lib = _lib.load("mfma")
-    # From 8 rows on the tiled kernel streams the weights faster than the skinny one
-    # (18944 x 3584 at 1, 8, 16, 32 rows: skinny 50, 57, 63, 80 us; tiles 55, 55, 55, 58).
-    skinny = _core().gated_is_skinny(m)
-    if skinny and tile_config is None:
-        code = lib.mk_gated_skinny(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k, _stream())
-    else:
-        code = lib.mk_gated_tiled(_ptr(x), _ptr(w_gate_up), _ptr(act), m, inter, k,
-                                  -1 if tile_config is None else tile_config, _stream())
-    _lib.check(lib, code, "gated_projection")
-    return act
+    scratch = Scratch(x.device)
+    address = _ensure(x).launch_gated(_ptr(x), m, k, _ptr(w_gate_up), inter, dtype_code(x.dtype),
+                                      -2 if tile_config is None else int(tile_config), scratch,
+                                      _stream())
+    return scratch.view(address, (m, inter), x.dtype)
 
 
 def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
@@ -269,32 +295,30 @@ def linear(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None = None,
         return out
     if kernel == "mfma" and (x.dtype != torch.bfloat16 or k % 8):
         raise KernelArgumentError("linear: the matrix-core kernels take bfloat16 with K % 8 == 0")
-    # 0: the float32-arithmetic kernel; 1: a few rows straight from HBM into the matrix cores;
-    # 2: the same, added into `out`; 3: tiles through LDS
-    kind = _ensure(x).choose_linear(dtype_code(x.dtype), m, n, k, bias is not None, accumulate,
-                                    dtype_code(out_dtype), {"auto": 0, "generic": 1, "mfma": 2}[kernel])
-    if kind != 0:
-        lib = _lib.load("mfma")
-        if kind == 1:
-            _lib.check(lib, lib.mk_linear_skinny(_ptr(x), _ptr(w), _ptr(out), m, n, k, 1, _stream()),
-                       "linear")
-            return out
-        if kind == 2:
-            _lib.check(lib, lib.mk_linear_skinny_acc(
-                _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
-                _ptr(out), m, n, k, _stream()), "linear")
-            return out
-        _lib.check(lib, lib.mk_linear_tiled(
-            _ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
-            _ptr(out), dtype_code(out_dtype), int(accumulate), m, n, k, n, tile_config,
-            _stream()), "linear")
-        return out
-    lib = _lib.load("core")
-    _lib.check(lib, lib.mk_linear_generic(
-        _ptr(x), _ptr(w), dtype_code(x.dtype), _ptr(bias),
-        dtype_code(bias.dtype) if bias is not None else F32, _ptr(out), dtype_code(out_dtype),
-        int(accumulate), m, n, k, k, n, _stream()), "linear")
+    _ensure(x).launch_linear(_ptr(x), m, _ptr(w), n, k, dtype_code(x.dtype), _ptr(bias),
+                             dtype_code(bias.dtype) if bias is not None else F32, _ptr(out),
+                             dtype_code(out_dtype), bool(accumulate),
+                             {"auto": 0, "generic": 1, "mfma": 2}[kernel], int(tile_config),
+                             _stream())
     return out
+
+
+def project_into_stream(x: torch.Tensor, w: torch.Tensor, bias: torch.Tensor | None,
+                        h: torch.Tensor) -> torch.Tensor | None:
+    """h += x W^T (+ bias), the way a step's program does it: where partial sums over slices of
+    K stream the weights faster they are returned ([P, T, H] float32) for the next norm to add,
+    and h is left as it is; otherwise None."""
+    _dev(x, w, bias, h)
+    if h.dtype != torch.float32 or h.shape != (x.shape[0], w.shape[0]) or x.shape[1] != w.shape[1]:
+        raise KernelArgumentError("project_into_stream: shapes do not match the float32 stream")
+    m, k = x.shape
+    n = w.shape[0]
+    scratch = Scratch(x.device)
+    address, count = _ensure(x).launch_project(_ptr(x), m, _ptr(w), n, k, dtype_code(x.dtype),
+                                               _ptr(bias),
+                                               dtype_code(bias.dtype) if bias is not None else F32,
+                                               _ptr(h), scratch, _stream())
+    return scratch.view(address, (count, m, n), torch.float32) if count else None
 
 
 # ---------------------------------------------------------------------- positions and the cache
@@ -314,6 +338,40 @@ def _check_caches(what, k_cache, v_cache, n_kv, head_dim, dtype) -> int:
     return page_size
 
 
+def _check_tables(what, cos, sin, rotary_dim) -> int:
+    if not rotary_dim:
+        return 0
+    if cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32 \
+            or cos.shape != sin.shape or cos.shape[1] != rotary_dim // 2:
+        raise KernelArgumentError(f"{what}: float32 cos and sin tables of the rotary width are required")
+    return cos.shape[0]
+
+
+def _qkv_args(what, w, bias, cos, sin, k_cache, v_cache, n_q, n_kv, head_dim, rotary_dim,
+              write_kv, interleaved, dtype) -> dict:
+    """The q/k/v side of an attention by name, as the launch sequences take it; checks the
+    tables and the caches against the sizes."""
+    page_size = _check_caches(what, k_cache, v_cache, n_kv, head_dim, dtype) if write_kv else 1
+    return dict(
+        w_qkv=_ptr(w), b_qkv=_ptr(bias), b_qkv_dtype=dtype_code(bias.dtype) if bias is not None else F32,
+        n_q=n_q, n_kv=n_kv, head_dim=head_dim, rotary_dim=rotary_dim, cos=_ptr(cos), sin=_ptr(sin),
+        table_positions=_check_tables(what, cos, sin, rotary_dim), interleaved=bool(interleaved),
+        k_cache=_ptr(k_cache) if write_kv else 0, v_cache=_ptr(v_cache) if write_kv else 0,
+        page_size=page_size, writes=bool(write_kv))
+
+
+def _arrays(what, tokens, positions, token_seq, block_table, cu_q=None, kv_len=None) -> dict:
+    _i32(positions, "positions")
+    _i32(token_seq, "token_seq")
+    _i32(block_table, "block_table")
+    if positions.shape[0] != tokens or token_seq.shape[0] != tokens:
+        raise KernelArgumentError(f"{what}: positions/token_seq must have one entry per token")
+    if block_table.dim() != 2:
+        raise KernelArgumentError(f"{what}: the block table is [sequences, pages]")
+    return dict(positions=_ptr(positions), token_seq=_ptr(token_seq), cu_q=_ptr(cu_q),
+                kv_len=_ptr(kv_len), table=_ptr(block_table), table_stride=block_table.shape[1])
+
+
 def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor | None,
                   positions: torch.Tensor, token_seq: torch.Tensor, block_table: torch.Tensor,
                   k_cache: torch.Tensor | None, v_cache: torch.Tensor | None, n_q: int,
@@ -330,76 +388,32 @@ def rope_kv_write(qkv: torch.Tensor, cos: torch.Tensor | None, sin: torch.Tensor
     qkv as float32 partial sums [P, T, width] is summed (plus `bias`) first, and the rotated q
     comes back as a new [T, n_q d] tensor of `out_dtype`."""
     _dev(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache, bias)
+    heads_kv = n_kv if write_kv else 0
+    width = (n_q + 2 * heads_kv) * head_dim
     if qkv.dim() == 3:
-        if interleaved and rotary_dim:
-            raise KernelArgumentError("rope: partial sums are finished in the half-split layout only")
-        return _qkv_finish(qkv, cos, sin, positions, token_seq, block_table, k_cache, v_cache,
-                           n_q, n_kv, head_dim, rotary_dim, write_kv, bias, out_dtype)
+        slices, tokens, got = qkv.shape
+        if qkv.dtype != torch.float32 or out_dtype is None:
+            raise KernelArgumentError("rope: partial sums are float32 and need an out_dtype")
+        if got != width:
+            raise KernelArgumentError(f"rope: partial sums of width {got} do not match the heads")
+        if bias is not None and bias.shape != (width,):
+            raise KernelArgumentError("rope: bias does not match the projection width")
+        args = _qkv_args("rope", None, bias, cos, sin, k_cache, v_cache, n_q, max(n_kv, 1),
+                         head_dim, rotary_dim, write_kv, interleaved, out_dtype)
+        scratch = Scratch(qkv.device)
+        address = _ensure(qkv).launch_qkv_finish(
+            _ptr(qkv), slices, tokens, dtype_code(out_dtype), args,
+            _arrays("rope", tokens, positions, token_seq, block_table), scratch, _stream())
+        return scratch.view(address, (tokens, n_q * head_dim), out_dtype)
     if bias is not None:
         raise KernelArgumentError("rope: a bias is only added to partial sums")
-    _i32(positions, "positions")
-    _i32(token_seq, "token_seq")
-    _i32(block_table, "block_table")
     tokens, row = qkv.shape
-    if positions.shape[0] != tokens or token_seq.shape[0] != tokens:
-        raise KernelArgumentError("rope: positions/token_seq must have one entry per token")
-    table_positions = 0
-    if rotary_dim:
-        if cos is None or sin is None or cos.dtype != torch.float32 or sin.dtype != torch.float32:
-            raise KernelArgumentError("rope: float32 cos and sin tables are required")
-        if cos.shape != sin.shape or cos.shape[1] != rotary_dim // 2:
-            raise KernelArgumentError(
-                f"rope: tables {tuple(cos.shape)} do not match rotary width {rotary_dim}")
-        table_positions = cos.shape[0]
-    page_size = 1
-    if write_kv:
-        page_size = _check_caches("rope", k_cache, v_cache, n_kv, head_dim, qkv.dtype)
-    lib = _lib.load("core")
-    _lib.check(lib, lib.mk_rope_kv_write(
-        _ptr(qkv), dtype_code(qkv.dtype), row, _ptr(cos), _ptr(sin), table_positions,
-        _ptr(positions), _ptr(token_seq), _ptr(block_table), block_table.shape[1],
-        _ptr(k_cache), _ptr(v_cache), page_size, n_q, n_kv, head_dim, rotary_dim,
-        int(bool(interleaved)), int(write_kv), tokens, _stream()), "rope_kv_write")
+    args = _qkv_args("rope", None, None, cos, sin, k_cache, v_cache, n_q, max(n_kv, 1), head_dim,
+                     rotary_dim, write_kv, interleaved, qkv.dtype)
+    _ensure(qkv).launch_rope_kv_write(_ptr(qkv), row, tokens, dtype_code(qkv.dtype), args,
+                                      _arrays("rope", tokens, positions, token_seq, block_table),
+                                      _stream())
     return qkv
-
-
-def _qkv_finish(parts, cos, sin, positions, token_seq, block_table, k_cache, v_cache, n_q, n_kv,
-                head_dim, rotary_dim, write_kv, bias, out_dtype):
-    _i32(positions, "positions")
-    _i32(token_seq, "token_seq")
-    _i32(block_table, "block_table")
-    slices, tokens, width = parts.shape
-    if parts.dtype != torch.float32 or out_dtype is None:
-        raise KernelArgumentError("rope: partial sums are float32 and need an out_dtype")
-    if width != (n_q + (2 * n_kv if write_kv else 0)) * head_dim:
-        raise KernelArgumentError(f"rope: partial sums of width {width} do not match the heads")
-    if bias is not None and bias.shape != (width,):
-        raise KernelArgumentError("rope: bias does not match the projection width")
-    table_positions = 0
-    if rotary_dim:
-        if cos is None or sin is None or cos.dtype != torch.float32 or cos.shape != sin.shape \
-                or cos.shape[1] != rotary_dim // 2:
-            raise KernelArgumentError("rope: float32 cos and sin tables of the rotary width are required")
-        table_positions = cos.shape[0]
-    page_size = _check_caches("rope", k_cache, v_cache, n_kv, head_dim, out_dtype) if write_kv else 1
-    q = torch.empty((tokens, n_q * head_dim), dtype=out_dtype, device=parts.device)
-    lib = _lib.load("core")
-    _lib.check(lib, lib.mk_qkv_finish(
-        _ptr(parts), slices, tokens * width, _ptr(bias),
-        dtype_code(bias.dtype) if bias is not None else F32, _ptr(q), dtype_code(out_dtype),
-        _ptr(cos), _ptr(sin), table_positions, _ptr(positions), _ptr(token_seq),
-        _ptr(block_table), block_table.shape[1], _ptr(k_cache), _ptr(v_cache), page_size, n_q,
-        n_kv if write_kv else 0, head_dim, rotary_dim, int(write_kv), tokens, _stream()),
-        "qkv_finish")
-    return q
-
-
-def _qkv_fusable(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int,
-                 half_layout: bool = True) -> bool:
-    if x.dtype not in _DTYPE_CODE or w.dtype not in _DTYPE_CODE:
-        return False
-    return _core().qkv_fusable(dtype_code(x.dtype), dtype_code(w.dtype), x.shape[0], x.shape[1],
-                               head_dim, rotary_dim, page_size, half_layout)
 
 
 def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int) -> bool:
@@ -411,6 +425,9 @@ def fuses_qkv(x, w: torch.Tensor, head_dim: int, rotary_dim: int, page_size: int
     return _qkv_kernel(x, w, head_dim, rotary_dim, page_size) in ("skinny", "tiled")
 
 
+_QKV_KINDS = ("skinny", "tiled", "partials", "plain")
+
+
 def _qkv_kernel(x, w, head_dim, rotary_dim, page_size, half_layout: bool = True):
     """ "skinny" (up to 64 rows: weights straight into the matrix cores, one workgroup per 32
     rows of W with all of K), "tiled" (any number of rows, through LDS, where whole-K tiles
@@ -418,7 +435,7 @@ def _qkv_kernel(x, w, head_dim, rotary_dim, page_size, half_layout: bool = True)
     kernel) or "plain" (the projection, then the rotation and cache-write kernel)."""
     kind = _ensure(x).choose_qkv(dtype_code(x.dtype), dtype_code(w.dtype), x.shape[0], w.shape[0],
                                  x.shape[1], head_dim, rotary_dim, page_size, half_layout)
-    return ("skinny", "tiled", "partials", "plain")[kind]
+    return _QKV_KINDS[kind]
 
 
 def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor | None,
@@ -429,64 +446,42 @@ def qkv_project(x, w: torch.Tensor, bias: torch.Tensor | None, cos: torch.Tensor
                 tile_config: int = -1, interleaved: bool = False) -> torch.Tensor:
     """q, k, v = x W^T + bias for W = [q heads | k heads | v heads]; q and k rotated by their
     positions; k and v written to the paged cache (`write_kv`; otherwise W holds the query
-    heads only).  Returns the rotated q [T, n_q d].
+    heads only).  Returns the rotated q, one row per token (the rows may be wider than
+    n_q d: when the projection and the rotation are two kernels, q stays in the projected
+    buffer).
 
     Where `fuses_qkv` says so, one kernel does all of it (projection, bias, rotation and cache
     write in its epilogue: the skinny kernel for few rows, the tiled one for many); otherwise
-    the projection (whole or as partial sums) is followed by `rope_kv_write`.  `fused` forces
-    one or the other, `tile_config` a tile configuration of the tiled kernel."""
+    the projection (whole or as partial sums) is followed by the rotation and cache write.
+    `fused` forces one or the other, `tile_config` a tile configuration of the tiled kernel."""
+    _dev(x, w, bias, cos, sin, positions, token_seq, block_table, k_cache, v_cache)
     heads_kv = n_kv if write_kv else 0
     width = (n_q + 2 * heads_kv) * head_dim
     if w.shape[0] != width or w.shape[1] != x.shape[1]:
         raise KernelArgumentError(f"qkv_project: W {tuple(w.shape)} is not [{width}, {x.shape[1]}]")
-    page_size = k_cache.shape[2] if write_kv and k_cache is not None else 1
-    half = not (interleaved and rotary_dim)
-    if fused is None:
-        kernel = _qkv_kernel(x, w, head_dim, rotary_dim, page_size, half)
-    elif not fused:
-        kernel = "partials" if half and wants_partials(x, w) else "plain"
-    elif not _qkv_fusable(x, w, head_dim, rotary_dim, page_size, half):
-        raise KernelArgumentError("qkv_project: these operands cannot take the fused kernel")
-    else:
-        kernel = "skinny" if x.shape[0] <= SKINNY_MAX_ROWS and tile_config < 0 else "tiled"
-    if kernel == "partials":
-        return rope_kv_write(linear_partials(x, w), cos, sin, positions, token_seq,
-                             block_table, k_cache, v_cache, n_q, heads_kv, head_dim,
-                             rotary_dim, write_kv, bias=bias, out_dtype=x.dtype)
-    if kernel == "plain":
-        return rope_kv_write(linear(x, w, bias), cos, sin, positions, token_seq, block_table,
-                             k_cache, v_cache, n_q, heads_kv, head_dim, rotary_dim, write_kv,
-                             interleaved=not half)
-    tokens, k = x.shape
-    _dev(x, w, bias, cos, sin, positions, token_seq, block_table, k_cache, v_cache)
-    _i32(positions, "positions")
-    _i32(token_seq, "token_seq")
-    _i32(block_table, "block_table")
-    if positions.shape[0] != tokens or token_seq.shape[0] != tokens:
-        raise KernelArgumentError("qkv_project: positions/token_seq must have one entry per token")
     if bias is not None and bias.shape != (width,):
         raise KernelArgumentError("qkv_project: bias does not match the projection width")
-    table_positions = 0
-    if rotary_dim:
-        if cos is None or sin is None or cos.dtype != torch.float32 or cos.shape != sin.shape \
-                or cos.shape[1] != rotary_dim // 2:
-            raise KernelArgumentError("qkv_project: float32 cos and sin tables of the rotary width are required")
-        table_positions = cos.shape[0]
-    if write_kv:
-        _check_caches("qkv_project", k_cache, v_cache, n_kv, head_dim, torch.bfloat16)
-    q = torch.empty((tokens, n_q * head_dim), dtype=torch.bfloat16, device=w.device)
-    lib = _lib.load("mfma")
-    args = (_ptr(x), _ptr(w), _ptr(bias), dtype_code(bias.dtype) if bias is not None else F32,
-            _ptr(q), _ptr(cos), _ptr(sin), table_positions, _ptr(positions), _ptr(token_seq),
-            _ptr(block_table), block_table.shape[1], _ptr(k_cache) if write_kv else 0,
-            _ptr(v_cache) if write_kv else 0, page_size, n_q, heads_kv, head_dim,
-            int(rotary_dim > 0), tokens, k)
-    if kernel == "skinny":
-        code = lib.mk_qkv_skinny(*args, _stream())
+    page_size = k_cache.shape[2] if write_kv and k_cache is not None else 1
+    half = not (interleaved and rotary_dim)
+    core = _ensure(x)
+    if fused is None:
+        kind = -1
+    elif not fused:
+        kind = 2 if half and wants_partials(x, w) else 3
+    elif not core.qkv_fusable(dtype_code(x.dtype), dtype_code(w.dtype), x.shape[0], x.shape[1],
+                              head_dim, rotary_dim, page_size, half):
+        raise KernelArgumentError("qkv_project: these operands cannot take the fused kernel")
     else:
-        code = lib.mk_qkv_tiled(*args, tile_config, _stream())
-    _lib.check(lib, code, "qkv_project")
-    return q
+        kind = 0 if x.shape[0] <= SKINNY_MAX_ROWS and tile_config < 0 else 1
+    tokens, k = x.shape
+    args = _qkv_args("qkv_project", w, bias, cos, sin, k_cache, v_cache, n_q, n_kv, head_dim,
+                     rotary_dim, write_kv, interleaved, x.dtype)
+    scratch = Scratch(x.device)
+    address, stride = core.launch_qkv_project(
+        _ptr(x), tokens, k, dtype_code(x.dtype), args,
+        _arrays("qkv_project", tokens, positions, token_seq, block_table), kind, int(tile_config),
+        scratch, _stream())
+    return scratch.view(address, (tokens, stride), x.dtype)
 
 
 def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
@@ -508,46 +503,37 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     through LDS; by default the step's size decides all three.
     """
     _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out)
-    _i32(block_table, "block_table")
     tokens = step.num_tokens
     if q.numel() < (tokens - 1) * q_stride + n_q * head_dim and tokens:
         raise KernelArgumentError("attention: q buffer too small")
     if block_table.dim() != 2 or block_table.shape[0] != step.num_seqs:
         raise KernelArgumentError("attention: the block table needs one row per sequence")
     page_size = _check_caches("attention", k_cache, v_cache, n_kv, head_dim, q.dtype)
-    if out is None:
-        out = torch.empty((tokens, n_q * head_dim), dtype=q.dtype, device=q.device)
+    if out is not None and (out.shape != (tokens, n_q * head_dim) or out.dtype != q.dtype):
+        raise KernelArgumentError("attention: out has the wrong shape or dtype")
     counts = [count for _first, count, _start in step.spans]
-    plan = _ensure(q).plan_attention(
-        dtype_code(q.dtype), head_dim, page_size, n_q, n_kv, int(window or 0), counts,
-        step.max_q_len, step.max_kv_len, force={"auto": 0, "generic": 1, "mfma": 2}[kernel],
-        tile_rows=-1 if tile_rows is None else int(tile_rows),
-        staged=-1 if staged is None else int(staged),
-        splits=split_override[0] if split_override is not None else 0,
-        split_blocks=split_override[1] if split_override is not None else 0)
-    if not plan["mfma"]:
-        lib = _lib.load("core")
-        _lib.check(lib, lib.mk_attention_generic(
-            _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
-            dtype_code(q.dtype), _ptr(step.positions), _ptr(step.token_seq), _ptr(block_table),
-            block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
-            int(window or 0), tokens, _stream()), "attention")
+    force = dict(kernel={"auto": 0, "generic": 1, "mfma": 2}[kernel],
+                 tile_rows=-1 if tile_rows is None else int(tile_rows),
+                 staged=-1 if staged is None else int(staged),
+                 splits=split_override[0] if split_override is not None else 0,
+                 split_blocks=split_override[1] if split_override is not None else 0)
+    args = dict(n_q=n_q, n_kv=n_kv, head_dim=head_dim, page_size=page_size,
+                window=int(window or 0), scale=float(scale), k_cache=_ptr(k_cache),
+                v_cache=_ptr(v_cache))
+
+    def tiles(group, rows):
+        seq, row0, count = step.tiles(group, rows)
+        return _ptr(seq), _ptr(row0), count
+
+    scratch = Scratch(q.device)
+    address = _ensure(q).launch_attention(
+        _ptr(q), int(q_stride), dtype_code(q.dtype), args,
+        _arrays("attention", tokens, step.positions, step.token_seq, block_table, step.cu_q,
+                step.kv_len),
+        counts, step.max_q_len, step.max_kv_len, force, tiles, _ptr(out), scratch, _stream())
+    if out is not None:
         return out
-    lib = _lib.load("mfma")
-    group = n_q // n_kv
-    rows, staged, splits, split_blocks = plan["rows"], plan["staged"], plan["splits"], plan["split_blocks"]
-    tile_seq, tile_row0, num_tiles = step.tiles(group, plan["tile_rows"])
-    part_o = part_ml = None
-    if splits > 1:
-        part_o = torch.empty((num_tiles, n_kv, splits, rows, head_dim), dtype=torch.float32, device=q.device)
-        part_ml = torch.empty((num_tiles, n_kv, splits, rows, 2), dtype=torch.float32, device=q.device)
-    _lib.check(lib, lib.mk_attention_mfma(
-        _ptr(q), q_stride, _ptr(out), n_q * head_dim, _ptr(k_cache), _ptr(v_cache),
-        _ptr(tile_seq), _ptr(tile_row0), num_tiles, _ptr(step.cu_q), _ptr(step.kv_len),
-        _ptr(block_table), block_table.shape[1], page_size, n_q, n_kv, head_dim, float(scale),
-        int(window or 0), rows, int(staged), splits, split_blocks, _ptr(part_o), _ptr(part_ml),
-        _stream()), "attention")
-    return out
+    return scratch.view(address, (tokens, n_q * head_dim), q.dtype)
 
 
 # ----------------------------------------------------------------------------------- sampling

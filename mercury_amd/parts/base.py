@@ -34,8 +34,11 @@ Interfaces
     returns None, by the part's own `apply` on the projected q and k.
 ``Part.lower(program, ...)``
     optional: append the part's operations to a step program of the host core, which then
-    launches them without coming back to Python (``csrc/host/program.*``).  A part without
-    `lower` is run through its `forward`; a model may mix both kinds, layer by layer.
+    launches them without coming back to Python (``csrc/host/program.*``).  An operation is
+    a registered kind (``hostcore.core.register_op``) and a block of parameter bytes; the
+    package's own kinds live in ``csrc/ops``.  A part without `lower` is run through its
+    `forward`; a model may mix both kinds, layer by layer.  A subclass that overrides
+    `forward` without defining `lower` again is run through its `forward` (`can_lower`).
 """
 
 from __future__ import annotations
@@ -147,10 +150,27 @@ class Part:
 
     # A part that can hand its work to the host core defines
     #     lower(self, program, ...) -> None
-    # appending its operations to `program`; `lowerable` says whether it does (a part may
-    # decide by its parameters, e.g. an attention whose position encoding applies itself
-    # cannot).
+    # appending its operations to `program`; `lowerable` says whether this instance does (a
+    # part may decide by its parameters, e.g. an attention whose position encoding applies
+    # itself cannot).
     lowerable = False
+
+    def can_lower(self) -> bool:
+        """Whether the host core may run this part in place of its `forward`: the instance
+        says so, its class (or a base) defines `lower`, and no class below that one overrides
+        `forward`: an override the lowered operations know nothing of would silently never
+        run."""
+        if not self.lowerable:
+            return False
+        lower_in = forward_in = None
+        for cls in type(self).__mro__:
+            if lower_in is None and "lower" in cls.__dict__:
+                lower_in = cls
+            if forward_in is None and "forward" in cls.__dict__:
+                forward_in = cls
+        if lower_in is None:
+            return False
+        return forward_in is None or issubclass(lower_in, forward_in)
 
 
 class Norm(Part):

@@ -32,13 +32,19 @@ class PreNormBlock(Part):
         return all(part.graph_safe for _, part in self._children())
 
     def lowerable_with(self, state) -> bool:
-        """Whether the host core can run the whole layer: every part hands over its work and
-        the mixer keeps no state of its own."""
-        return state is None and all(part.lowerable for _, part in self._children())
+        """Whether the host core can run the whole layer: every part hands over its work, and
+        a mixer with state of its own says that its operations take the state tensor
+        (`lowers_state`)."""
+        if state is not None and not getattr(self.mixer, "lowers_state", False):
+            return False
+        return all(part.can_lower() for _, part in self._children())
 
-    def lower(self, program, cache) -> None:
+    def lower(self, program, cache, state=None) -> None:
         self.norm_mixer.lower(program)
-        self.mixer.lower(program, cache)
+        if state is None:
+            self.mixer.lower(program, cache)
+        else:
+            self.mixer.lower(program, cache, state)
         if self.ffn is not None:
             self.norm_ffn.lower(program)
             self.ffn.lower(program)

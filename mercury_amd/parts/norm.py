@@ -2,6 +2,7 @@
 
 from __future__ import annotations
 
+from ..hostcore import core
 from ..kernels import ops
 from .base import Norm, TensorSpec
 
@@ -31,10 +32,13 @@ class RMSNorm(Norm):
         self.weight = params["weight"]
 
     def forward(self, h, out_dtype, rows=None, partials=None):
+        # one kernel; its launch is the one the lowered operation makes
         return ops.rmsnorm(h, self.weight, self.eps, out_dtype, rows=rows, partials=partials)
 
-    def lower(self, program) -> None:
-        program.norm(self.weight.data_ptr(), ops.dtype_code(self.weight.dtype), self.eps)
+    def lower(self, program, select_rows: bool = False) -> None:
+        """`select_rows`: normalise the step's wanted rows only (before an output head)."""
+        program.append("norm", core.norm_params(
+            self.weight.data_ptr(), ops.dtype_code(self.weight.dtype), self.eps, select_rows))
 
     def weight_bytes(self) -> int:
         return self.weight.numel() * self.weight.element_size()

@@ -9,8 +9,15 @@ import zlib
 from .engine.executor import ExecResult
 
 
+def stand_in_token(rid: str, index: int, vocab_size: int) -> int:
+    """The token the model-free executor emits as output `index` of request `rid`: a fixed
+    function of the two, so a test can say what a request must have produced however its
+    work was scheduled."""
+    return (zlib.crc32(rid.encode()) + 7919 * index) % vocab_size
+
+
 class DeterministicExecutor:
-    """Produces token (crc32(rid) + 7919 * index) % vocab without a model, after checking what
+    """Produces `stand_in_token(rid, index, vocab)` without a model, after checking what
     the real step function relies on: every work item starts where the request's computed
     tokens end and the request holds pages for all positions it touches, no page twice."""
 
@@ -23,7 +30,7 @@ class DeterministicExecutor:
         self.steps = self.prefill_tokens_seen = self.decode_tokens_seen = 0
 
     def token_for(self, rid: str, index: int) -> int:
-        return (zlib.crc32(rid.encode()) + index * 7919) % self.vocab_size
+        return stand_in_token(rid, index, self.vocab_size)
 
     def _check(self, work) -> None:
         r = work.request
@@ -63,18 +70,20 @@ class DeterministicExecutor:
         return ExecResult(tokens=tokens, forward_seconds=time.perf_counter() - started)
 
     def snapshot(self) -> dict:
-        return {"runner": "deterministic", "steps": self.steps, "device": "none"}
+        return {"device": "none", "executor": "model-free", "steps": self.steps,
+                "prefill_tokens": self.prefill_tokens_seen, "decode_tokens": self.decode_tokens_seen}
 
 
-class FakeClock:
-    """A clock the caller advances, so scheduling tests never depend on wall time."""
+class ManualClock:
+    """Time that stands still until the test moves it with `tick`; calling it reads it.  The
+    scheduler's waiting times and deadlines then depend on the test alone."""
 
-    def __init__(self, start: float = 1000.0):
-        self.now = start
+    def __init__(self, at: float = 0.0):
+        self.at = float(at)
 
     def __call__(self) -> float:
-        return self.now
+        return self.at
 
-    def advance(self, seconds: float) -> float:
-        self.now += seconds
-        return self.now
+    def tick(self, seconds: float) -> float:
+        self.at += seconds
+        return self.at

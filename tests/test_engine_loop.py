@@ -79,7 +79,7 @@ def test_a_tenth_of_requests_cancelled_leaks_nothing():
         h.submit(f"r{i}", [rng.randrange(40)] * 16 + [rng.randrange(9000) for _ in range(rng.randrange(1, 60))],
                  max_tokens=rng.randrange(4, 24))
         h.engine.step()
-        h.clock.advance(0.01)
+        h.clock.tick(0.01)
         if rng.random() < 0.1:
             live = [r.rid for r in h.engine.sched.running + h.engine.sched.waiting]
             if live:
@@ -174,7 +174,7 @@ def test_generate_blocks_until_every_prompt_is_done():
 def test_snapshot_and_step_log():
     h = build(policy="lpm_aging", num_blocks=32, max_running=1)
     h.submit("a", list(range(32)), max_tokens=3)
-    h.clock.advance(0.5)
+    h.clock.tick(0.5)
     h.submit("b", list(range(100, 132)), max_tokens=3)
     h.drain()
     snap = h.engine.snapshot()

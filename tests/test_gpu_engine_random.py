@@ -66,7 +66,7 @@ def test_random_requests_under_random_options(seed, tmp_path):
         for i, (p, m) in enumerate(zip(prompts, max_tokens)):
             engine.submit(f"{turn}-{i}", p, m, events[i].append,
                           params=SamplingParams(ignore_eos=True))
-        engine._drain_commands()
+        engine._take_commands()
         steps = 0
         while engine.sched.has_work():
             engine.step()

@@ -126,7 +126,7 @@ def test_temperature_sampling_is_per_request_reproducible():
         for i in which:
             eng.submit(f"req{i}", prompts[i], 6, lambda e, i=i: outs.setdefault(i, []).append(e),
                        params=SamplingParams(temperature=0.8, ignore_eos=True))
-        eng._drain_commands()
+        eng._take_commands()
         while eng.sched.has_work():
             eng.step()
         return {i: [e.token for e in ev if e.kind == "token"] for i, ev in outs.items()}
@@ -198,7 +198,7 @@ def test_a_graph_row_changes_its_owner(dtype):
         outs = {i: [] for i in range(len(prompts))}
         for i, (p, n) in enumerate(zip(prompts, lengths)):
             eng.submit(f"r{i}", list(p), n, outs[i].append, params=SamplingParams(ignore_eos=True))
-        eng._drain_commands()
+        eng._take_commands()
         while eng.sched.has_work():
             eng.step()
         assert eng.leaked_blocks() == 0
@@ -230,7 +230,7 @@ def run_requests(eng, submissions, max_tokens, aborts=(), **params):
             count += 1
         for rid in dict(aborts).get(step, []):
             eng.abort(rid)
-        eng._drain_commands()
+        eng._take_commands()
         if not eng.sched.has_work() and step > max(submissions):
             break
         eng.step()

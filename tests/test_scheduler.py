@@ -228,7 +228,7 @@ def grouped_stream(policy, groups=6, steps=600, seed=5, **cfg):
             suffix = [rng.randrange(9_000)] * rng.randrange(8, 32)
             h.submit(f"r{step}", prefixes[rng.randrange(groups)] + suffix, max_tokens=6)
         h.engine.step()
-        h.clock.advance(STEP_DT)
+        h.clock.tick(STEP_DT)
     return h
 
 
