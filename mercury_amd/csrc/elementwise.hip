@@ -86,6 +86,62 @@ extern "C" int mk_logit_cap(float* logits, long long count, float cap, hipStream
   return 0;
 }
 
+// ----------------------------------------------------------- per-request state of fixed size
+
+// State rows live in slots [num_slots, width] (float32); a sequence's slot is
+// slots[token_seq[t]].  Store: every token at absolute position `at_position` writes its row of
+// x into its sequence's slot.  Load: every token reads its sequence's row.
+template <typename T>
+__global__ void state_store_kernel(const T* __restrict__ x, float* __restrict__ state,
+                                   const int* __restrict__ slots, const int* __restrict__ token_seq,
+                                   const int* __restrict__ positions, int at_position, int width) {
+  const int t = blockIdx.x;
+  if (positions[t] != at_position) return;
+  float* dst = state + (size_t)slots[token_seq[t]] * width;
+  const T* src = x + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) dst[i] = Elem<T>::load(src + i);
+}
+
+template <typename T>
+__global__ void state_load_kernel(const float* __restrict__ state, const int* __restrict__ slots,
+                                  const int* __restrict__ token_seq, T* __restrict__ out, int width) {
+  const int t = blockIdx.x;
+  const float* src = state + (size_t)slots[token_seq[t]] * width;
+  T* dst = out + (size_t)t * width;
+  for (int i = threadIdx.x; i < width; i += blockDim.x) Elem<T>::store(dst + i, src[i]);
+}
+
+extern "C" int mk_state_store(const void* x, int dtype, float* state, const int* slots,
+                              const int* token_seq, const int* positions, int at_position,
+                              int tokens, int width, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && width > 0 && at_position >= 0, "state_store: bad sizes");
+  MK_REQUIRE(dtype == MK_F32 || dtype == MK_BF16, "state_store: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  const int threads = width >= 256 ? 256 : 64;
+  if (dtype == MK_F32)
+    state_store_kernel<float><<<tokens, threads, 0, stream>>>((const float*)x, state, slots,
+                                                              token_seq, positions, at_position, width);
+  else
+    state_store_kernel<bf16_t><<<tokens, threads, 0, stream>>>((const bf16_t*)x, state, slots,
+                                                               token_seq, positions, at_position, width);
+  MK_LAUNCH_CHECK("state_store");
+  return 0;
+}
+
+extern "C" int mk_state_load(const float* state, const int* slots, const int* token_seq, void* out,
+                             int dtype, int tokens, int width, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && width > 0, "state_load: bad sizes");
+  MK_REQUIRE(dtype == MK_F32 || dtype == MK_BF16, "state_load: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  const int threads = width >= 256 ? 256 : 64;
+  if (dtype == MK_F32)
+    state_load_kernel<float><<<tokens, threads, 0, stream>>>(state, slots, token_seq, (float*)out, width);
+  else
+    state_load_kernel<bf16_t><<<tokens, threads, 0, stream>>>(state, slots, token_seq, (bf16_t*)out, width);
+  MK_LAUNCH_CHECK("state_load");
+  return 0;
+}
+
 // --------------------------------------------------------------------------------- RMSNorm
 
 // Sum of p[0], p[stride], ..., p[(n-1) stride], four loads in flight at a time; the order of

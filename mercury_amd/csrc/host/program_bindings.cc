@@ -3,6 +3,8 @@
 #include <pybind11/pybind11.h>
 #include <pybind11/stl.h>
 
+#include <cstddef>
+
 #include "program.h"
 #include "step_batch.h"
 
@@ -64,6 +66,17 @@ void bind_program(py::module_& m) {
         "Register an operation kind: `run` and `tiles` are addresses of C functions with the "
         "signatures of op_abi.h (mk_op_run_fn, mk_op_tiles_fn); whoever registers keeps them alive.");
   m.def("op_kinds", []() { return OpRegistry::instance().names(); });
+  m.def("op_abi_layout", []() {
+    py::dict d;
+    d["context_size"] = sizeof(mk_op_context);
+    d["step_size"] = sizeof(mk_step_view);
+    d["tile_list_size"] = sizeof(mk_tile_list);
+    d["context_error_offset"] = offsetof(mk_op_context, error);
+    d["context_alloc_offset"] = offsetof(mk_op_context, alloc);
+    d["context_out_x_offset"] = offsetof(mk_op_context, out_x);
+    d["step_tables_offset"] = offsetof(mk_step_view, tables);
+    return d;
+  }, "Sizes and a few offsets of the structures of op_abi.h, for mirrors of them to check.");
   m.attr("OP_READS_X") = (int)MK_OP_READS_X;
   m.attr("OP_FOLDS_PENDING") = (int)MK_OP_FOLDS_PENDING;
 

@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 13
+#define MK_ABI_VERSION 14
 
 #ifdef __cplusplus
 extern "C" {
@@ -27,6 +27,16 @@ int mk_embed(const int* ids, const void* table, int dtype, float* out, int token
 
 // logits[i] = cap * tanh(logits[i] / cap) for i < count, in place.
 int mk_logit_cap(float* logits, long long count, float cap, hipStream_t stream);
+
+// Per-request state of fixed size: rows of `state` [slots, width] (float32), a sequence's row
+// being slots[token_seq[t]].  mk_state_store: every token at absolute position `at_position`
+// writes its row of x [tokens, width] into its sequence's slot.  mk_state_load: every token's
+// row of out is its sequence's row of the state.
+int mk_state_store(const void* x, int dtype, float* state, const int* slots, const int* token_seq,
+                   const int* positions, int at_position, int tokens, int width,
+                   hipStream_t stream);
+int mk_state_load(const float* state, const int* slots, const int* token_seq, void* out, int dtype,
+                  int tokens, int width, hipStream_t stream);
 
 // RMSNorm of rows of the float32 residual stream h, optionally after adding `num_partials`
 // partial sums [p, row, hidden] (stride between partials in elements) into h.  `rows`, when

@@ -151,6 +151,16 @@ def kernel_prototypes() -> dict:
     return out
 
 
+def kernel_abi_version() -> int:
+    """MK_ABI_VERSION as the header defines it."""
+    import re
+
+    match = re.search(r"#define\s+MK_ABI_VERSION\s+(\d+)", KERNEL_HEADER.read_text())
+    if not match:
+        raise BuildError(f"{KERNEL_HEADER.name} defines no MK_ABI_VERSION")
+    return int(match.group(1))
+
+
 def _write_kernel_names(folder: Path) -> Path:
     """The lists of entry points by library as X-macros, for the host core's table of function
     pointers (their types come from the declarations themselves, by decltype)."""

@@ -11,7 +11,7 @@ from ctypes import c_char_p, c_float, c_int, c_longlong, c_ulonglong, c_void_p
 
 from . import build
 
-ABI_VERSION = 13
+ABI_VERSION = build.kernel_abi_version()
 
 _CTYPES = {"pointer": c_void_p, "int": c_int, "float": c_float, "long long": c_longlong,
            "unsigned long long": c_ulonglong, "hipStream_t": c_void_p, "const char*": c_char_p}
