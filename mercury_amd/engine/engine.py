@@ -159,6 +159,7 @@ class Engine:
         graph_batch = min(cfg.max_graph_batch, cfg.max_running)
         if cfg.num_blocks < 0:
             reserve = Engine.reserve_bytes(model, cfg, device, graph_batch)
+            cfg.extra["reserved_bytes"] = reserve
             cfg.num_blocks = autosize_blocks(cfg, model.kv_bytes_per_token(cfg.torch_dtype), device,
                                              reserve)
             cfg.validate_against(model.max_positions or cfg.max_model_len)
