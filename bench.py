@@ -165,10 +165,15 @@ class Bench:
         for _ in range(untimed):
             self.engine.step()
         self.sync()
+        # The device's own clock over the same steps: one pair of events around all of them
+        # (a pair per step costs tens of microseconds a step, which a short step feels).
+        began, ended = (self.torch.cuda.Event(enable_timing=True) for _ in range(2))
         start = time.perf_counter()
+        began.record()
         for _ in range(steps):
             record = self.engine.step()
             assert record.num_decode == batch and record.num_prefill == 0
+        ended.record()
         self.sync()
         elapsed = time.perf_counter() - start
         assert max(r.num_computed for r in self.engine.sched.running) == context
@@ -179,8 +184,7 @@ class Bench:
         self.engine._take_commands()
         assert self.engine.leaked_blocks() == 0
         ms = 1e3 * elapsed / steps
-        timed = self.engine.metrics.step_records()[-steps:]
-        device_ms = 1e3 * sum(r.device_s for r in timed) / steps
+        device_ms = began.elapsed_time(ended) / steps
         return {"tok_s": batch * steps / elapsed, "ms": ms, "fill_s": fill_s, "device_ms": device_ms,
                 "prompt_len": prompt_len, "bytes": self.model.decode_weight_bytes() + kv_bytes}
 

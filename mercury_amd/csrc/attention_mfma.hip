@@ -770,9 +770,9 @@ __device__ __forceinline__ void wide_fetch(const AttnParams& p, TableWindow& tw,
     const unsigned int k_to = dst + (unsigned int)load * 1024u;
     const unsigned int v_to = dst + (unsigned int)(64 * D * 2) + (unsigned int)load * 1024u;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 : : "s"(k_to), "v"(mine.k_at), "s"(k_from) : "memory");
+                 : : "s"(k_to), "v"(mine.k_at), "s"(k_from) : "memory", "m0");
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 : : "s"(v_to), "v"(mine.v_at), "s"(v_from) : "memory");
+                 : : "s"(v_to), "v"(mine.v_at), "s"(v_from) : "memory", "m0");
   }
 }
 

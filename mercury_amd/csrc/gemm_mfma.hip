@@ -720,7 +720,8 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
       if (partial) from = past_k ? (const bf16_t*)tiled_zero_chunk : from;
       asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, off"
                    :
-                   : "s"(dst), "v"(from));
+                   : "s"(dst), "v"(from)
+                   : "m0");
     }
   };
   // The products of a stage, with the loads of stage `ahead` handed out between them: all up

@@ -191,8 +191,12 @@ int mk_argmax(const float* logits, int rows, int vocab, long long row_stride, in
 // mk_argmax_static_max_rows() rows; more rows are refused.  This entry point has no
 // counterpart in the reference: it is for callers that cannot allocate (code under HIP graph
 // capture, serving loops and harnesses that forbid hipMalloc).  Calls that overlap on one GPU
-// share the array and race; calls on one stream, one after the other, are safe.
+// share the array and race; calls on one stream, one after the other, are safe.  The first
+// call on a device asks the runtime where the array lies; mk_argmax_static_init() does only
+// that, for the current device, so that a caller can have it done before a stream capture
+// begins.  Both may be called from several threads.
 int mk_argmax_static_max_rows(void);
+int mk_argmax_static_init(void);
 int mk_argmax_static(const float* logits, int rows, int vocab, long long row_stride, int* out,
                      hipStream_t stream);
 

@@ -11,6 +11,8 @@
 // inclusive cumulative kept mass exceeds u * total.  Equal probabilities at the nucleus
 // edge are kept together.  Every pass over a row's vocabulary is shared out over 64
 // workgroups.
+#include <atomic>
+
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -110,15 +112,44 @@ extern "C" int mk_argmax(const float* logits, int rows, int vocab, long long row
 // address is asked for once per device (with that device current) and kept; only that address
 // is ever handed to a kernel.  Nothing in the array has to start at zero: each call's first
 // kernel writes every part that its second kernel reads.  Every call on a GPU uses that GPU's
-// one array, so two calls that overlap on one GPU (different streams) race.
+// one array, so two calls that overlap on one GPU (different streams) race.  The first call
+// on a device asks the runtime for the address, which is a query a stream capture should not
+// contain: a caller that captures calls mk_argmax_static_init() (or mk_argmax_static itself)
+// once on that device beforehand.
 #define ARGMAX_STATIC_MAX_ROWS 256
 static __device__ __align__(256) unsigned char
     argmax_static_scratch[ARGMAX_STATIC_MAX_ROWS * ARGMAX_PARTS * sizeof(MaxIdx)];
 
 #define ARGMAX_STATIC_MAX_DEVICES 64
-static void* g_argmax_scratch_of_device[ARGMAX_STATIC_MAX_DEVICES];
+// One address per device, each written once.  Threads that ask at the same time for a device
+// nobody has asked for yet all get the same answer from the runtime and store the same
+// value; the slots are atomic so that this is no data race.
+static std::atomic<void*> g_argmax_scratch_of_device[ARGMAX_STATIC_MAX_DEVICES];
+
+// The array's address on the current device, asked of the runtime at the first call per
+// device.  0 on success.
+static int argmax_static_scratch_address(void** out) {
+  int device = -1;
+  hipError_t e = hipGetDevice(&device);
+  MK_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(e));
+  MK_REQUIRE(device >= 0 && device < ARGMAX_STATIC_MAX_DEVICES, "argmax_static: device %d", device);
+  void* scratch = g_argmax_scratch_of_device[device].load(std::memory_order_acquire);
+  if (scratch == nullptr) {
+    e = hipGetSymbolAddress(&scratch, HIP_SYMBOL(argmax_static_scratch));
+    MK_REQUIRE(e == hipSuccess && scratch != nullptr, "argmax_static: hipGetSymbolAddress: %s",
+               hipGetErrorString(e));
+    g_argmax_scratch_of_device[device].store(scratch, std::memory_order_release);
+  }
+  *out = scratch;
+  return 0;
+}
 
 extern "C" int mk_argmax_static_max_rows(void) { return ARGMAX_STATIC_MAX_ROWS; }
+
+extern "C" int mk_argmax_static_init(void) {
+  void* scratch = nullptr;
+  return argmax_static_scratch_address(&scratch);
+}
 
 extern "C" int mk_argmax_static(const float* logits, int rows, int vocab, long long row_stride,
                                 int* out, hipStream_t stream) {
@@ -127,17 +158,8 @@ extern "C" int mk_argmax_static(const float* logits, int rows, int vocab, long l
              "argmax_static: %d rows; the library's own scratch holds at most %d (use mk_argmax "
              "with a buffer of the caller's)", rows, ARGMAX_STATIC_MAX_ROWS);
   if (rows == 0) return 0;
-  int device = -1;
-  hipError_t e = hipGetDevice(&device);
-  MK_REQUIRE(e == hipSuccess, "argmax_static: hipGetDevice: %s", hipGetErrorString(e));
-  MK_REQUIRE(device >= 0 && device < ARGMAX_STATIC_MAX_DEVICES, "argmax_static: device %d", device);
-  void* scratch = g_argmax_scratch_of_device[device];
-  if (scratch == nullptr) {
-    e = hipGetSymbolAddress(&scratch, HIP_SYMBOL(argmax_static_scratch));
-    MK_REQUIRE(e == hipSuccess && scratch != nullptr, "argmax_static: hipGetSymbolAddress: %s",
-               hipGetErrorString(e));
-    g_argmax_scratch_of_device[device] = scratch;
-  }
+  void* scratch = nullptr;
+  if (int code = argmax_static_scratch_address(&scratch)) return code;
   if (vocab >= 16384) {
     argmax_part_kernel<<<dim3(ARGMAX_PARTS, rows), 256, 0, stream>>>(logits, vocab, row_stride,
                                                                       (MaxIdx*)scratch);

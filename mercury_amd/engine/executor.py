@@ -26,10 +26,12 @@ class ExecResult:
 
 class _Pending:
     """Tokens on their way from the device into pinned host memory: `wait()` gives them as a
-    list.  `began` is the event recorded before the step's first kernel."""
+    list.  `began` is the event recorded before the step's first kernel, `previous` the event
+    that closed the step before this one on the same stream."""
 
-    def __init__(self, tokens_dev, host, done, began=None):
+    def __init__(self, tokens_dev, host, done, began=None, previous=None):
         self.host, self.done, self.began = host[:tokens_dev.shape[0]], done, began
+        self.previous = previous
         self.host.copy_(tokens_dev, non_blocking=True)
         self.done.record()
 
@@ -38,8 +40,17 @@ class _Pending:
         return self.host.tolist()
 
     def device_seconds(self) -> float:
-        """Time on the device from the step's first kernel to its tokens' copy (after wait)."""
-        return 1e-3 * self.began.elapsed_time(self.done) if self.began is not None else 0.0
+        """Time on the device from the step's start to its tokens' copy (after wait).  A step
+        launched ahead has its start event recorded while the step before it still runs; the
+        stream reaches that event only when the earlier step is done, but the step's own time
+        cannot begin before the earlier step's end either way: the later of the two counts, so
+        that the steps' times never overlap and add up to no more than the wall clock."""
+        if self.began is None:
+            return 0.0
+        own = self.began.elapsed_time(self.done)
+        if self.previous is not None:
+            own = min(own, self.previous.elapsed_time(self.done))
+        return 1e-3 * max(own, 0.0)
 
 
 class _PinnedRing:
@@ -55,6 +66,7 @@ class _PinnedRing:
         self.events = [torch.cuda.Event(enable_timing=True) for _ in range(depth)]
         self.starts = [torch.cuda.Event(enable_timing=True) for _ in range(depth)]
         self.next = 0
+        self.last_done = None      # the event that closed the most recent step
 
     def begin(self):
         """Record, now, the start event of the step whose tokens the next `pending` carries."""
@@ -66,10 +78,14 @@ class _PinnedRing:
         n = tokens_dev.shape[0]
         i = self.next
         self.next = (i + 1) % len(self.buffers)
+        previous = self.last_done
         if n > self.size:
-            return _Pending(tokens_dev, torch.empty(n, dtype=torch.int32, pin_memory=True),
-                            torch.cuda.Event(enable_timing=True), self.starts[i])
-        return _Pending(tokens_dev, self.buffers[i], self.events[i], self.starts[i])
+            made = _Pending(tokens_dev, torch.empty(n, dtype=torch.int32, pin_memory=True),
+                            torch.cuda.Event(enable_timing=True), self.starts[i], previous)
+        else:
+            made = _Pending(tokens_dev, self.buffers[i], self.events[i], self.starts[i], previous)
+        self.last_done = made.done
+        return made
 
 
 @dataclass

@@ -49,9 +49,11 @@ def test_the_line_of_one_gpu_keeps_the_contract():
     assert 0 < line["prefill"]["frac"] < 1
     assert set(line["points"]) == {"decode_b1", "decode_b64", "decode_b8_ctx256", "prefill_8192"}
     assert line["points"]["decode_b64"] > line["points"]["decode_b1"] > 0
-    # against what the machine itself reaches: a streaming read between 2 and 8 TB/s, a large
-    # product between 0.3 and 2.5 PFLOP/s; the step's device time (between two events, so with
+    # against what the machine itself reaches, as measured on this pool's cards: a streaming
+    # read of 5.6-6.4 TB/s, a large product of 1.0-1.35 PFLOP/s (the bounds leave a tenth on
+    # either side, and room for a faster product kernel); the step's device time (between two events, so with
     # the events' own cost, which a step of two layers feels) near its wall clock
-    assert 2000 < roof["measured_peak"] < 8000 and roof["frac_of_measured"] > roof["frac"]
-    assert 3e14 < line["prefill"]["measured_peak"] < 2.5e15
-    assert 0 < line["device_ms_per_step"] <= line["ms_per_step"] * 1.5
+    assert 5000 < roof["measured_peak"] < 7000 and roof["frac_of_measured"] > roof["frac"]
+    assert 0.9e15 < line["prefill"]["measured_peak"] < 1.8e15
+    # the steps' times on the device do not overlap, so they add up to no more than the wall clock
+    assert 0 < line["device_ms_per_step"] <= line["ms_per_step"] * 1.02

@@ -1,10 +1,19 @@
-"""Which attention kernel the host core picks for a step's shape (csrc/host/dispatch.cc): the
-choices behind the benchmark's numbers, each with the measurement that set its threshold.
+"""Which kernel the host core picks for a step's shape (csrc/ops/dispatch.cc).
+
+Most of this file does not pin the planner's present choices (those move whenever a
+threshold is measured again) but what must hold of every choice: the matrix-core attention
+accepts every plan the planner can emit (checked with the kernel entry point's own argument
+checks, without a launch), the tile lists have the length the plan says, key splits never
+leave a part without blocks, and a fused q/k/v kernel is only ever chosen for operands it
+takes.  A handful of choices behind the benchmark's numbers stay pinned at the end.
 The planner runs on the host; it only asks the kernel library what it has."""
+
+import random
 
 import pytest
 
-BF16 = 1
+F32, BF16 = 0, 1
+HEAD_SIZES = (16, 32, 48, 64, 80, 96, 112, 128, 160, 192, 256)
 
 
 @pytest.fixture(scope="module")
@@ -24,106 +33,149 @@ def plan(core, heads, kv_heads, size, counts, context, window=0, page=16):
     return core.plan_attention(BF16, size, page, heads, kv_heads, window, counts, max(counts), context)
 
 
-def test_decoding_splits_the_keys_in_fours(core):
-    """Few tiles: every tile's keys in as many parts as fill the chip with wavefronts, in
-    fours, which one workgroup's wavefronts add up before writing (8 sequences at 4,096, 14
-    heads of 64: 9.0 us with 64 parts against 11.5 with 63)."""
+def random_step(rng):
+    """(head size, page, heads, kv heads, window, tokens per sequence, longest length)."""
+    size = rng.choice(HEAD_SIZES)
+    page = rng.choice((8, 16, 32, 64, 128))
+    kv_heads = rng.choice((1, 2, 3, 4, 8))
+    heads = kv_heads * rng.choice((1, 2, 3, 4, 7, 8, 16))
+    window = rng.choice((0, 0, 0, 24, 1000, 5000))
+    kind = rng.random()
+    if kind < 0.35:          # decoding
+        counts = [1] * rng.choice((1, 2, 7, 8, 33, 64, 200, 256))
+    elif kind < 0.6:         # one prompt, short to very long
+        counts = [rng.choice((2, 17, 64, 100, 512, 2048, 4700, 8192, 30000))]
+    else:                    # portions beside decoded tokens
+        counts = [rng.choice((1, 1, 1, 2, 16, 100, 512, 2048)) for _ in range(rng.randint(1, 40))]
+    longest = max(counts) + rng.choice((0, 0, 5, 300, 4000, 30000))
+    return size, page, heads, kv_heads, window, counts, longest
+
+
+def test_every_plan_is_one_the_kernel_accepts(core):
+    rng = random.Random(11)
+    seen = {"generic": 0, "split": 0, "staged": 0, "wide": 0, "plain": 0}
+    for _ in range(3000):
+        size, page, heads, kv_heads, window, counts, longest = random_step(rng)
+        p = core.plan_attention(BF16, size, page, heads, kv_heads, window, counts, max(counts), longest)
+        case = (size, page, heads, kv_heads, window, counts[:4], len(counts), longest, p)
+        if not p["mfma"]:
+            seen["generic"] += 1
+            continue
+        # the entry point's own checks, without the launch
+        assert core.validate_attention_plan(p, size, page, heads, kv_heads) == "", case
+        group = heads // kv_heads
+        # the tile list the packer lays out is the one the plan counted
+        assert core.count_tiles(counts, group, p["tile_rows"]) == p["num_tiles"], case
+        seq, row0 = core.build_tiles(counts, group, p["tile_rows"])
+        assert len(seq) == len(row0) == p["num_tiles"], case
+        assert all(0 <= s < len(counts) for s in seq), case
+        assert all(r % p["tile_rows"] == 0 and r < counts[s] * group for s, r in zip(seq, row0)), case
+        assert p["tile_rows"] == (p["rows"] * 4 if p["staged"] else p["rows"]), case
+        # key splits: only without staging, never more parts than pairs of 32-key blocks of
+        # the longest span, in fours from four on
+        span = min(longest, window + max(counts)) if window else longest
+        blocks = max(1, -(-span // 32))
+        assert 1 <= p["splits"] <= max(1, blocks // 2) or p["splits"] == 1, case
+        if p["splits"] > 1:
+            assert p["staged"] == 0 and (p["splits"] < 4 or p["splits"] % 4 == 0), case
+        # the kernel of 32-row wavefronts: only where a sequence has at least 128 rows
+        if p["staged"] >= 8:
+            assert max(counts) * group >= 128 and p["rows"] == 32, case
+        seen["wide" if p["staged"] >= 8 else "staged" if p["staged"] else
+             "split" if p["splits"] > 1 else "plain"] += 1
+    # the generator reaches every kind of plan
+    assert all(n >= 30 for n in seen.values()), seen
+
+
+def test_float32_and_unsupported_sizes_take_the_float32_kernel(core):
+    for size in HEAD_SIZES:
+        assert not core.plan_attention(F32, size, 16, 8, 2, 0, [64], 64, 64)["mfma"]
+    assert not plan(core, 8, 2, 48, [64], 64)["mfma"]
+    assert not plan(core, 8, 2, 64, [64], 64, page=8)["mfma"]
+    with pytest.raises(RuntimeError, match="bfloat16 only"):
+        core.plan_attention(F32, 64, 16, 8, 2, 0, [64], 64, 64, force=2)
+
+
+def test_qkv_choices_are_ones_the_kernels_take(core):
+    rng = random.Random(5)
+    skinny, tiled, partials, unfused = 0, 1, 2, 3
+    counts = {skinny: 0, tiled: 0, partials: 0, unfused: 0}
+    for _ in range(3000):
+        size = rng.choice(HEAD_SIZES)
+        kv = rng.choice((1, 2, 4, 8))
+        heads = kv * rng.choice((1, 2, 4, 7))
+        width = (heads + 2 * kv) * size
+        k = rng.choice((64, 168, 896, 900, 1024, 3584, 5120))
+        rows = rng.choice((1, 2, 8, 16, 17, 64, 65, 256, 257, 2048))
+        rotary = rng.choice((0, size, size // 2))
+        half = rng.random() < 0.8
+        page = rng.choice((8, 16, 64))
+        dtype = BF16 if rng.random() < 0.85 else F32
+        kind = core.choose_qkv(dtype, dtype, rows, width, k, size, rotary, page, half)
+        counts[kind] += 1
+        fusable = core.qkv_fusable(dtype, dtype, rows, k, size, rotary, page, half)
+        case = (dtype, rows, width, k, size, rotary, page, half, kind)
+        if kind in (skinny, tiled):
+            assert fusable and dtype == BF16 and k % 8 == 0 and size % 32 == 0, case
+            assert rotary in (0, size) and (half or rotary == 0), case
+        if kind == skinny:
+            assert rows <= 64, case
+        if kind == partials:
+            # the finishing kernel rotates in the half-split layout only, and partial sums
+            # come from the matrix-core kernels
+            assert (half or rotary == 0) and core.wants_partials(dtype, dtype, rows, width, k), case
+        if dtype == F32 or k % 8:
+            assert kind == unfused, case
+    assert all(n >= 30 for n in counts.values()), counts
+
+
+def test_projection_choices_are_ones_the_kernels_take(core):
+    rng = random.Random(7)
+    generic, skinny, skinny_acc, tiled = 0, 1, 2, 3
+    for _ in range(2000):
+        m = rng.choice((1, 7, 8, 16, 17, 64, 65, 512))
+        n = rng.choice((896, 1000, 4864, 151936))
+        k = rng.choice((64, 896, 900, 4864))
+        bias, accumulate = rng.random() < 0.3, rng.random() < 0.5
+        dtype = BF16 if rng.random() < 0.8 else F32
+        out = F32 if accumulate or rng.random() < 0.5 else dtype
+        kind = core.choose_linear(dtype, m, n, k, bias, accumulate, out, 0)
+        case = (dtype, m, n, k, bias, accumulate, out, kind)
+        if dtype == F32 or k % 8:
+            assert kind == generic, case
+            assert not core.wants_partials(dtype, dtype, m, n, k), case
+            continue
+        assert kind != generic, case
+        if kind == skinny:          # float32 out, no bias, not accumulating: what it computes
+            assert out == F32 and not bias and not accumulate and m < 8, case
+        if kind == skinny_acc:
+            assert accumulate and m <= 64, case
+        if core.wants_partials(dtype, dtype, m, n, k):
+            by_skinny, slices = core.plan_partials(m, n, k)
+            assert slices >= 1 and (not by_skinny or m <= 16), case   # one slice: a whole product left as float32 for the next norm
+
+
+# ---- pinned: the choices behind the benchmark's numbers, each with its measurement
+
+
+def test_pinned_choices_of_the_benchmark_shapes(core):
+    # 0.5B decoding, 8 sequences at 4,096: the keys in 64 parts, in fours that one workgroup's
+    # wavefronts add up before writing (9.0 us against 11.5 with 63)
     p = plan(core, 14, 2, 64, [1] * 8, 4096)
     assert (p["staged"], p["rows"], p["splits"]) == (0, 16, 64)
-    p = plan(core, 14, 2, 64, [1], 4096)
-    assert p["splits"] == 64 and p["num_tiles"] == 1      # no more parts than pairs of key blocks
-    p = plan(core, 28, 4, 128, [1] * 8, 4096)
-    assert p["splits"] == 32
-    p = plan(core, 14, 2, 64, [1] * 64, 4096)
-    assert p["splits"] == 8
     # many sequences fill the chip by themselves
     assert plan(core, 40, 8, 128, [1] * 128, 4096)["splits"] == 1
-    # a short context has few blocks to hand out
-    assert plan(core, 14, 2, 64, [1] * 8, 100)["splits"] <= 2
-
-
-def test_prompts_go_through_lds(core):
-    """A 2,048-token prompt of 14 heads of 64 is 224 workgroups of 128 rows, fewer than compute
-    units: the 16-row kernel with the keys in four chains (30 us against 40 in the 32-row
-    kernel, a tie with its three chains)."""
-    p = plan(core, 14, 2, 64, [2048], 2048)
-    assert (p["staged"], p["rows"], p["tile_rows"], p["num_tiles"]) == (4, 16, 64, 224)   # x 2 kv heads
-    # 28 heads of 64: 448 workgroups, chains too short to cut: the 32-row kernel (44 us against 47)
-    assert plan(core, 28, 4, 64, [2048], 2048)["staged"] == 8
-    # 128-wide heads from 256 workgroups (28 heads, 2,048 tokens: 79 us against 96)
-    p = plan(core, 28, 4, 128, [2048], 2048)
-    assert (p["staged"], p["rows"], p["tile_rows"]) == (8, 32, 128)
-
-
-def test_long_prompts_take_32_row_wavefronts(core):
-    """8,192 tokens: 0.55-0.80 PFLOP/s in the 32-row kernel against 0.42-0.54 in the 16-row
-    one, at every head shape."""
-    for heads, kv_heads, size in ((14, 2, 64), (28, 4, 64), (28, 4, 128), (40, 8, 128)):
+    # 8,192-token prompts: the kernel of 32-row wavefronts at every head shape (0.55-0.80
+    # PFLOP/s against 0.42-0.54)
+    for heads, kv_heads, size in ((14, 2, 64), (28, 4, 128), (40, 8, 128)):
         p = plan(core, heads, kv_heads, size, [8192], 8192)
         assert (p["staged"], p["rows"]) == (8, 32)
-    assert plan(core, 14, 2, 64, [2048] * 4, 2048)["staged"] == 8      # 73 us against 90
-
-
-def test_chunks_over_long_prefixes_cut_the_keys_into_chains(core):
-    """Fewer workgroups than fill the chip, each with a long chain of key blocks: 64-wide heads
-    in three chains (2,048 tokens over 30,720: 347 us against 500 in the 16-row kernel; 4,096
-    tokens: 63 against 92), 128-wide in two (1,024 over 3,072, 28 heads: 92 against 133)."""
-    assert plan(core, 14, 2, 64, [2048], 2048 + 30720)["staged"] == 24
-    assert plan(core, 14, 2, 64, [4096], 4096)["staged"] == 24
-    assert plan(core, 28, 4, 128, [1024], 4096)["staged"] == 16
-    # too few workgroups for either: the 16-row kernel, more of them (512 over 7,680: 71 against 93)
-    assert plan(core, 14, 2, 64, [512], 8192)["staged"] in (1, 2, 4)
-
-
-def test_head_sizes_the_32_row_kernel_does_not_take(core):
-    p = plan(core, 8, 2, 96, [8192], 8192)
-    assert p["mfma"] and p["staged"] == 0 and p["rows"] in (16, 32)
-    p = plan(core, 8, 2, 256, [8192], 8192)
-    assert p["mfma"] and p["staged"] == 0 and p["rows"] == 16
-    assert not plan(core, 8, 2, 48, [64], 64)["mfma"]        # no matrix-core kernel of that size
-
-
-def test_mixed_steps_use_the_prompt_kernel_when_a_portion_is_long(core):
-    """A portion of 512 tokens beside 63 decoded ones: the prompt kernel for all of them."""
-    p = plan(core, 14, 2, 64, [512] + [1] * 63, 4096)
-    assert p["staged"] in (1, 2, 4) and p["splits"] == 1
-
-
-def test_the_qkv_projection_is_one_kernel_where_that_is_faster(core):
-    """Projection, bias, rotation and cache write in one kernel: the skinny one for few rows of
-    a small matrix (1152 x 896 at 8 rows: 6.0 us against 10.6 as partial sums and a finishing
-    kernel), the tiled one for many rows.  A matrix of 24 MB or more at up to 256 rows goes as
-    K-split partial sums and a finishing kernel (4608 x 3584 at 8..64 rows: 14.0..16.5 us
-    against 15.2..30.7 in the one skinny kernel)."""
-    skinny, tiled, partials, unfused = 0, 1, 2, 3
-    for rows, want in ((1, skinny), (8, skinny), (16, skinny), (64, tiled), (2048, tiled)):
-        assert core.choose_qkv(BF16, BF16, rows, 1152, 896, 64, 64, 16, True) == want
-    for rows, want in ((1, partials), (8, partials), (64, partials), (256, partials), (2048, tiled)):
-        assert core.choose_qkv(BF16, BF16, rows, 4608, 3584, 128, 128, 16, True) == want
-        assert core.choose_qkv(BF16, BF16, rows, 7168, 5120, 128, 128, 16, True) == want
-    # what the fused kernels do not take: heads that are no multiple of 32 wide, a rotation
-    # over part of the head, interleaved pairs
-    assert core.choose_qkv(BF16, BF16, 8, 18 * 48, 168, 48, 48, 16, True) in (partials, unfused)
-    assert core.choose_qkv(BF16, BF16, 8, 1152, 896, 64, 32, 16, True) == unfused
-    assert core.choose_qkv(BF16, BF16, 8, 1152, 896, 64, 64, 16, False) == unfused
-
-
-def test_projections_into_the_residual_stream(core):
-    """Few rows: K in slices with partial sums where the matrix is large enough for bandwidth
-    to matter (the 0.5B down projection, 8.7 MB, at 8 rows: 5.2 us in 8 slices against 9.5
-    whole), all of K in one workgroup where latency is the cost (the 0.5B o projection, 1.6 MB);
-    the skinny kernel up to 16 rows of a matrix under 20 MB, tiles beyond."""
-    by_skinny, slices = core.plan_partials(8, 896, 4864)
-    assert by_skinny and slices == 8
-    by_skinny, slices = core.plan_partials(8, 3584, 18944)
-    assert not by_skinny and slices >= 2          # 136 MB: tiles stream it faster
-    by_skinny, slices = core.plan_partials(64, 3584, 18944)
-    assert not by_skinny and slices >= 2
-    generic, skinny, skinny_acc, tiled = 0, 1, 2, 3
-    F32 = 0
-    assert core.choose_linear(BF16, 8, 896, 896, False, True, F32, 0) == skinny_acc
-    assert core.choose_linear(BF16, 2048, 896, 896, False, True, F32, 0) == tiled
-    assert core.choose_linear(BF16, 1, 151936, 896, False, False, F32, 0) == skinny      # the head
-    assert core.choose_linear(BF16, 8, 151936, 896, False, False, F32, 0) == tiled
-    assert core.choose_linear(BF16, 8, 896, 900, False, True, F32, 0) == generic         # K % 8
-    assert core.choose_linear(F32, 8, 896, 896, False, True, F32, 0) == generic
+    # the q/k/v projection: one skinny kernel for few rows of a small matrix (1152 x 896 at 8
+    # rows: 6.0 us against 10.6 as partial sums and a finishing kernel), partial sums for a
+    # matrix of 24 MB or more (4608 x 3584 at 8..64 rows: 14.0..16.5 us against 15.2..30.7)
+    assert core.choose_qkv(BF16, BF16, 8, 1152, 896, 64, 64, 16, True) == 0
+    assert core.choose_qkv(BF16, BF16, 8, 4608, 3584, 128, 128, 16, True) == 2
+    # the head: the skinny kernel below 8 rows, tiles from there (152064 x 3584: 188 / 204 us
+    # skinny at 1 / 8 rows, 187 / 191 tiled)
+    assert core.choose_linear(BF16, 1, 151936, 896, False, False, F32, 0) == 1
+    assert core.choose_linear(BF16, 8, 151936, 896, False, False, F32, 0) == 3

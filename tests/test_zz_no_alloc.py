@@ -25,7 +25,11 @@ def test_argmax_without_allocation_equals_argmax_with_a_buffer():
 
     device = torch.device("cuda:0")
     stream = torch.cuda.current_stream(device).cuda_stream
-    for rows, vocab, seed in ((64, 151_936, 1), (5, 20_011, 2), (3, 1_003, 3)):
+    # the address of the library's array, resolved before any call that might be captured
+    assert lib.mk_argmax_static_init() == 0, lib.mk_last_error()
+    # the first case fills the array to its stated limit (the last row's parts lie in its last
+    # slots); the following, smaller ones run over what it left there
+    for rows, vocab, seed in ((limit, 16_384, 4), (64, 151_936, 1), (5, 20_011, 2), (3, 1_003, 3)):
         g = torch.Generator().manual_seed(seed)
         logits = torch.randn(rows, vocab, generator=g).to(device)
         logits[0, vocab - 1] = 50.0                     # the very last place
