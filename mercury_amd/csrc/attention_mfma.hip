@@ -1206,14 +1206,14 @@ static void launch_merge(const AttnParams& p, hipStream_t stream) {
 }
 
 template <int D>
-static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stream) {
+static void launch_attn(const AttnParams& p, int rows_per_tile, bool merge, hipStream_t stream) {
   if constexpr (D <= 128) {
     if (attn_grouped(rows_per_tile, p.num_splits)) {
       AttnParams g = p;
       g.num_splits = p.num_splits / ATTN_WAVES;
       const dim3 grid(g.num_tiles, g.n_kv, g.num_splits);
       attn_mfma_kernel<D, 1, ATTN_AHEAD_16, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(g);
-      launch_merge<D>(g, stream);
+      if (merge) launch_merge<D>(g, stream);
       return;
     }
   }
@@ -1228,7 +1228,7 @@ static void launch_attn(const AttnParams& p, int rows_per_tile, hipStream_t stre
     // 64 rows: only instantiated where the accumulators fit the register file
     if constexpr (D <= 64) attn_mfma_kernel<D, 4, ATTN_AHEAD_64><<<grid, threads, 0, stream>>>(p);
   }
-  launch_merge<D>(p, stream);
+  if (merge) launch_merge<D>(p, stream);
 }
 
 // The most rows (16, 32 or 64) one wavefront can take for this head size.
@@ -1295,13 +1295,13 @@ extern "C" int mk_attention_mfma_check(int q_stride, int out_stride, int num_til
   return 0;
 }
 
-extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
-                                 const void* k_cache, const void* v_cache, const int* tile_seq,
-                                 const int* tile_row0, int num_tiles, const int* cu_q,
-                                 const int* kv_len, const int* block_table, int table_stride,
-                                 int page_size, int n_q, int n_kv, int d, float scale, int window,
-                                 int rows_per_tile, int staged, int num_splits, int split_blocks,
-                                 float* part_o, float* part_ml, hipStream_t stream) {
+static int attention_mfma(const void* q, int q_stride, void* out, int out_stride,
+                          const void* k_cache, const void* v_cache, const int* tile_seq,
+                          const int* tile_row0, int num_tiles, const int* cu_q, const int* kv_len,
+                          const int* block_table, int table_stride, int page_size, int n_q,
+                          int n_kv, int d, float scale, int window, int rows_per_tile, int staged,
+                          int num_splits, int split_blocks, float* part_o, float* part_ml,
+                          bool merge, hipStream_t stream) {
   if (int code = mk_attention_mfma_check(q_stride, out_stride, num_tiles, page_size, n_q, n_kv, d,
                                          scale, window, rows_per_tile, staged, num_splits,
                                          split_blocks, part_o && part_ml)) {
@@ -1341,13 +1341,47 @@ extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out
     return 0;
   }
   switch (d) {
-    case 32: staged ? launch_staged<32>(p, rows_per_tile, staged, stream) : launch_attn<32>(p, rows_per_tile, stream); break;
-    case 64: staged ? launch_staged<64>(p, rows_per_tile, staged, stream) : launch_attn<64>(p, rows_per_tile, stream); break;
-    case 96: staged ? launch_staged<96>(p, rows_per_tile, staged, stream) : launch_attn<96>(p, rows_per_tile, stream); break;
-    case 128: staged ? launch_staged<128>(p, rows_per_tile, staged, stream) : launch_attn<128>(p, rows_per_tile, stream); break;
-    case 192: staged ? launch_staged<192>(p, rows_per_tile, staged, stream) : launch_attn<192>(p, rows_per_tile, stream); break;
-    case 256: staged ? launch_staged<256>(p, rows_per_tile, staged, stream) : launch_attn<256>(p, rows_per_tile, stream); break;
+    case 32: staged ? launch_staged<32>(p, rows_per_tile, staged, stream) : launch_attn<32>(p, rows_per_tile, merge, stream); break;
+    case 64: staged ? launch_staged<64>(p, rows_per_tile, staged, stream) : launch_attn<64>(p, rows_per_tile, merge, stream); break;
+    case 96: staged ? launch_staged<96>(p, rows_per_tile, staged, stream) : launch_attn<96>(p, rows_per_tile, merge, stream); break;
+    case 128: staged ? launch_staged<128>(p, rows_per_tile, staged, stream) : launch_attn<128>(p, rows_per_tile, merge, stream); break;
+    case 192: staged ? launch_staged<192>(p, rows_per_tile, staged, stream) : launch_attn<192>(p, rows_per_tile, merge, stream); break;
+    case 256: staged ? launch_staged<256>(p, rows_per_tile, staged, stream) : launch_attn<256>(p, rows_per_tile, merge, stream); break;
   }
   MK_LAUNCH_CHECK("attention_mfma");
   return 0;
+}
+
+extern "C" int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
+                                 const void* k_cache, const void* v_cache, const int* tile_seq,
+                                 const int* tile_row0, int num_tiles, const int* cu_q,
+                                 const int* kv_len, const int* block_table, int table_stride,
+                                 int page_size, int n_q, int n_kv, int d, float scale, int window,
+                                 int rows_per_tile, int staged, int num_splits, int split_blocks,
+                                 float* part_o, float* part_ml, hipStream_t stream) {
+  return attention_mfma(q, q_stride, out, out_stride, k_cache, v_cache, tile_seq, tile_row0,
+                        num_tiles, cu_q, kv_len, block_table, table_stride, page_size, n_q, n_kv, d,
+                        scale, window, rows_per_tile, staged, num_splits, split_blocks, part_o,
+                        part_ml, true, stream);
+}
+
+extern "C" int mk_attention_mfma_parts_written(int rows_per_tile, int num_splits, int d) {
+  return d <= 128 && attn_grouped(rows_per_tile, num_splits) ? num_splits / ATTN_WAVES : num_splits;
+}
+
+extern "C" int mk_attention_mfma_parts(const void* q, int q_stride, const void* k_cache,
+                                       const void* v_cache, const int* tile_seq,
+                                       const int* tile_row0, int num_tiles, const int* cu_q,
+                                       const int* kv_len, const int* block_table,
+                                       int table_stride, int page_size, int n_q, int n_kv, int d,
+                                       float scale, int window, int rows_per_tile, int num_splits,
+                                       int split_blocks, float* part_o, float* part_ml,
+                                       hipStream_t stream) {
+  // (four parts that one workgroup's wavefronts add up are one result, written to `out`)
+  MK_REQUIRE(num_splits > 1 && mk_attention_mfma_parts_written(rows_per_tile, num_splits, d) > 1,
+             "attention: partial results are left only where the keys are split over workgroups");
+  return attention_mfma(q, q_stride, nullptr, n_q * d, k_cache, v_cache, tile_seq, tile_row0,
+                        num_tiles, cu_q, kv_len, block_table, table_stride, page_size, n_q, n_kv, d,
+                        scale, window, rows_per_tile, 0, num_splits, split_blocks, part_o, part_ml,
+                        false, stream);
 }

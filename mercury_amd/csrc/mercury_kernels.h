@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 14
+#define MK_ABI_VERSION 15
 
 #ifdef __cplusplus
 extern "C" {
@@ -178,6 +178,29 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
                       int d, float scale, int window, int rows_per_tile, int staged,
                       int num_splits, int split_blocks, float* part_o, float* part_ml,
                       hipStream_t stream);
+
+// Decoding with split keys, in two kernels instead of three.  mk_attention_mfma_parts is
+// mk_attention_mfma without the merge of the key splits: the partial results stay in part_o /
+// part_ml, mk_attention_mfma_parts_written(...) of them per (tile, kv head) (a workgroup's four
+// wavefronts may have added four parts up already).  mk_attention_out then merges them and
+// multiplies by the output matrix w_o [N, n_q d] in one kernel, for steps of one token per
+// sequence (tile = token, M of them): out[slice, M, N] are float32 partial sums over slices of
+// heads_per_slice query heads each (mk_attention_out_heads_per_slice: how many, 0 where the
+// sizes are not taken; mk_attention_out_max_parts: the most partial results per (tile, kv head)
+// it takes), to be added up by whoever consumes the projection.  wide: 128 rows of w_o per
+// workgroup instead of 64.
+int mk_attention_mfma_parts_written(int rows_per_tile, int num_splits, int d);
+int mk_attention_mfma_parts(const void* q, int q_stride, const void* k_cache, const void* v_cache,
+                            const int* tile_seq, const int* tile_row0, int num_tiles,
+                            const int* cu_q, const int* kv_len, const int* block_table,
+                            int table_stride, int page_size, int n_q, int n_kv, int d, float scale,
+                            int window, int rows_per_tile, int num_splits, int split_blocks,
+                            float* part_o, float* part_ml, hipStream_t stream);
+int mk_attention_out_heads_per_slice(int n_q, int n_kv, int d, int M, int N);
+int mk_attention_out_max_parts(int M, int heads_per_slice);
+int mk_attention_out(const float* part_o, const float* part_ml, int parts, const void* w_o,
+                     float* out, int M, int N, int n_q, int n_kv, int d, int heads_per_slice,
+                     int wide, hipStream_t stream);
 
 // @library core
 

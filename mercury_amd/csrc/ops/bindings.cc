@@ -326,6 +326,44 @@ void bind_ops(py::module_& m) {
     });
     return (uintptr_t)q;
   });
+  m.def("launch_attention_project", [](uintptr_t q, int q_stride, int dtype, const py::dict& args,
+                                       const py::dict& arrays, const std::vector<int>& counts,
+                                       int max_q_len, int max_kv_len, const py::object& tiles,
+                                       uintptr_t w_o, uintptr_t b_o, int b_o_dtype, int hidden,
+                                       uintptr_t h, int fold, const py::object& alloc,
+                                       uintptr_t stream) {
+    const AttendArgs a = attend_from(args);
+    const StepArrays s = arrays_from(arrays);
+    mk_step_view view;
+    std::memset(&view, 0, sizeof view);
+    view.num_seqs = (int)counts.size();
+    view.counts = counts.data();
+    for (int c : counts) view.num_tokens += c;
+    view.max_q_len = max_q_len;
+    view.max_kv_len = max_kv_len;
+    const AttentionPlan plan = plan_for(dtype, a, view);
+    mk_tile_list list;
+    std::memset(&list, 0, sizeof list);
+    if (plan.mfma) {
+      const py::tuple t = tiles(a.n_q / a.n_kv, plan.tile_rows);
+      list.group = a.n_q / a.n_kv;
+      list.tile_rows = plan.tile_rows;
+      list.seq = as_ptr<const int>(py::cast<uintptr_t>(t[0]));
+      list.row0 = as_ptr<const int>(py::cast<uintptr_t>(t[1]));
+      list.count = py::cast<int>(t[2]);
+      view.num_tile_lists = 1;
+      view.tile_lists = &list;
+    }
+    const float* pending = nullptr;
+    int count = 0;
+    with_scratch(dtype, stream, alloc, [&](Launch& l) {
+      attend_and_project(l, Queries{as_ptr<const void>(q), q_stride}, a, s, view,
+                         as_ptr<const void>(w_o), as_ptr<const void>(b_o), b_o_dtype, hidden,
+                         as_ptr<float>(h), pending, count, AttendForce{}, fold);
+      return 0;
+    });
+    return py::make_tuple((uintptr_t)pending, count);
+  }, "The attention and its output projection into h; (address, count) of partial sums left.");
   m.def("launch_attention", [](uintptr_t q, int q_stride, int dtype, const py::dict& args,
                                const py::dict& arrays, const std::vector<int>& counts,
                                int max_q_len, int max_kv_len, const py::dict& force_in,

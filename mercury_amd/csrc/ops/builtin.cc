@@ -81,9 +81,8 @@ int run_attention(const void* params, mk_op_context* ctx) {
     Launch l(ctx);
     const StepArrays arrays = arrays_of(s, p.group);
     const Queries q = qkv_project(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, arrays);
-    const void* attended = attend(l, q, attend_args(p), arrays, s);
-    project_into_stream(l, attended, s.num_tokens, p.w_o, ctx->hidden, p.qkv.n_q * p.qkv.head_dim,
-                        p.b_o, p.b_o_dtype, ctx->h, ctx->out_pending, ctx->out_pending_count);
+    attend_and_project(l, q, attend_args(p), arrays, s, p.w_o, p.b_o, p.b_o_dtype, ctx->hidden,
+                       ctx->h, ctx->out_pending, ctx->out_pending_count);
   });
 }
 

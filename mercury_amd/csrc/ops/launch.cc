@@ -220,6 +220,66 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
   return out;
 }
 
+namespace {
+// The merge of the key splits folded into the output projection repeats the merge once per
+// 64 (or 128) rows of w_o; it pays while that repetition stays small beside what the two
+// kernels it replaces cost (measured at 8 and 64 decoded tokens: see DESIGN's kernel notes).
+constexpr long long kFoldMaxRepeatedBytes = 48ll << 20;
+constexpr int kFoldWideFromHidden = 2048;
+}  // namespace
+
+void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
+                        const mk_step_view& step, const void* w_o, const void* b_o, int b_o_dtype,
+                        int hidden, float* h, const float*& pending, int& pending_count,
+                        AttendForce force, int fold) {
+  const int m = step.num_tokens, d = a.head_dim;
+  pending = nullptr;
+  pending_count = 0;
+  const AttentionPlan plan = plan_for(l.dtype(), a, step, force);
+  int heads_per_slice = 0, written = 0;
+  bool wide = false;
+  if (fold != 0 && plan.mfma && plan.splits > 1 && !plan.staged && plan.rows == 16 &&
+      step.max_q_len == 1 && plan.num_tiles == m && !b_o && a.n_q / a.n_kv <= 16) {
+    const KernelTable& t = need_mfma();
+    written = t.mk_attention_mfma_parts_written(plan.rows, plan.splits, d);
+    heads_per_slice = t.mk_attention_out_heads_per_slice(a.n_q, a.n_kv, d, m, hidden);
+    wide = hidden >= kFoldWideFromHidden;
+    if (heads_per_slice &&
+        (written < 2 || written > t.mk_attention_out_max_parts(m, heads_per_slice))) {
+      heads_per_slice = 0;
+    }
+    if (heads_per_slice && fold < 0) {
+      const long long part_bytes = (long long)m * a.n_q * written * (d * 4 + 8);
+      const long long repeats = (hidden + (wide ? 127 : 63)) / (wide ? 128 : 64);
+      if (part_bytes * repeats > kFoldMaxRepeatedBytes) heads_per_slice = 0;
+    }
+  }
+  if (!heads_per_slice) {
+    if (fold > 0) throw KernelError("attention: these sizes do not take the folded merge");
+    const void* attended = attend(l, q, a, s, step, force);
+    project_into_stream(l, attended, m, w_o, hidden, a.n_q * d, b_o, b_o_dtype, h, pending,
+                        pending_count);
+    return;
+  }
+  const size_t rows = (size_t)plan.num_tiles * a.n_kv * plan.splits * plan.rows;
+  float* part_o = (float*)l.alloc(rows * d * 4);
+  float* part_ml = (float*)l.alloc(rows * 2 * 4);
+  const int slices = a.n_q / heads_per_slice;
+  float* out = (float*)l.alloc((size_t)slices * m * hidden * 4);
+  pending = out;
+  pending_count = slices;
+  if (l.dry() || m == 0) return;
+  const KernelTable& t = need_mfma();
+  const mk_tile_list& tiles = tiles_for(step, a.n_q / a.n_kv, plan.tile_rows);
+  check_mfma(t.mk_attention_mfma_parts(q.q, q.stride, a.k_cache, a.v_cache, tiles.seq, tiles.row0,
+                                       tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride,
+                                       a.page_size, a.n_q, a.n_kv, d, a.scale, a.window, plan.rows,
+                                       plan.splits, plan.split_blocks, part_o, part_ml, l.stream()),
+             "attention");
+  check_mfma(t.mk_attention_out(part_o, part_ml, written, w_o, out, m, hidden, a.n_q, a.n_kv, d,
+                                heads_per_slice, wide ? 1 : 0, l.stream()), "attention_out");
+}
+
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
             int tile_config) {
   if (fuses_gating(l.dtype(), l.dtype(), m, k, 2 * inter)) {

@@ -132,6 +132,16 @@ AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
 void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
              const mk_step_view& step, AttendForce force = {}, void* out = nullptr);
 
+// The attention and its output projection into the residual stream h [m, hidden] (+ bias), as
+// project_into_stream does it (pending / pending_count: partial sums left for the next norm).
+// Decoding with the keys split over workgroups takes two kernels instead of three: the
+// attention leaves its partial results, and one kernel merges them and multiplies by w_o
+// (`fold`: -1 where the sizes allow and it pays, 0 never, 1 wherever the sizes allow).
+void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
+                        const mk_step_view& step, const void* w_o, const void* b_o, int b_o_dtype,
+                        int hidden, float* h, const float*& pending, int& pending_count,
+                        AttendForce force = {}, int fold = -1);
+
 // act = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, k].  tile_config: -2 by the
 // sizes, else the tiled kernel with that configuration (-1: its own choice).
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,

@@ -37,6 +37,7 @@ LIBRARIES = {
     "mfma": [
         "host_support.hip",
         "attention_mfma.hip",
+        "attention_out.hip",
         "gemm_mfma.hip",
     ],
 }

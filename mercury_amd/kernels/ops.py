@@ -536,6 +536,40 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     return scratch.view(address, (tokens, n_q * head_dim), q.dtype)
 
 
+def attention_project(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                      step, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int,
+                      scale: float, window: int | None, w_o: torch.Tensor,
+                      b_o: torch.Tensor | None, h: torch.Tensor, fold: bool | None = None):
+    """`attention` followed by the output projection into the float32 stream h [T, H], the way
+    a step's program runs the two: h += attended W_o^T (+ b_o), or float32 partial sums
+    [P, T, H] returned for the next norm to add.  Decoding with split keys merges the splits
+    inside the projection's kernel where that pays (`fold`: None by the sizes, False never,
+    True wherever the sizes allow)."""
+    _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, w_o, b_o, h)
+    tokens, hidden = step.num_tokens, w_o.shape[0]
+    if h.dtype != torch.float32 or h.shape != (tokens, hidden) or w_o.shape[1] != n_q * head_dim:
+        raise KernelArgumentError("attention_project: shapes do not match the float32 stream")
+    page_size = _check_caches("attention", k_cache, v_cache, n_kv, head_dim, q.dtype)
+    counts = [count for _first, count, _start in step.spans]
+    args = dict(n_q=n_q, n_kv=n_kv, head_dim=head_dim, page_size=page_size,
+                window=int(window or 0), scale=float(scale), k_cache=_ptr(k_cache),
+                v_cache=_ptr(v_cache))
+
+    def tiles(group, rows):
+        seq, row0, count = step.tiles(group, rows)
+        return _ptr(seq), _ptr(row0), count
+
+    scratch = Scratch(q.device)
+    address, count = _ensure(q).launch_attention_project(
+        _ptr(q), int(q_stride), dtype_code(q.dtype), args,
+        _arrays("attention", tokens, step.positions, step.token_seq, block_table, step.cu_q,
+                step.kv_len),
+        counts, step.max_q_len, step.max_kv_len, tiles, _ptr(w_o), _ptr(b_o),
+        dtype_code(b_o.dtype) if b_o is not None else F32, hidden, _ptr(h),
+        -1 if fold is None else int(bool(fold)), scratch, _stream())
+    return scratch.view(address, (count, tokens, hidden), torch.float32) if count else None
+
+
 # ----------------------------------------------------------------------------------- sampling
 
 

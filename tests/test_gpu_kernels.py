@@ -850,6 +850,62 @@ def test_attention_decode_with_split_keys(batch, context):
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("n_q,n_kv,d,hidden,batch,context", [
+    (14, 2, 64, 896, 8, 4096), (14, 2, 64, 896, 1, 700), (14, 2, 64, 896, 64, 1100),
+    (8, 2, 128, 1024, 3, 2000), (28, 4, 128, 200, 17, 900), (6, 3, 64, 1000, 33, 520),
+    (40, 8, 128, 264, 2, 3000)])
+def test_decode_attention_with_the_merge_folded_into_the_output_projection(n_q, n_kv, d, hidden,
+                                                                          batch, context):
+    """Decoding with split keys as two kernels (attention leaving its partial results; their
+    merge inside the output projection) gives what the three kernels give, and what the plain
+    attention followed by the library product gives: partial sums per slice of heads, or
+    nothing left over when the step is not one the folded kernel takes."""
+    page = 16
+    lens = [context - 13 * i for i in range(batch)]
+    per = -(-context // page)
+    bf = torch.bfloat16
+    qs = [rounded(rnd(1, n_q, d, seed=200 + i), bf) for i in range(batch)]
+    ks = [rounded(rnd(n, n_kv, d, seed=300 + i), bf) for i, n in enumerate(lens)]
+    vs = [rounded(rnd(n, n_kv, d, seed=400 + i), bf) for i, n in enumerate(lens)]
+    w_o = rounded(rnd(hidden, n_q * d, seed=9, scale=0.05), bf)
+    k_cache = torch.zeros(batch * per, n_kv, page, d, dtype=bf)
+    v_cache = torch.zeros_like(k_cache)
+    table = torch.zeros((batch, per), dtype=torch.int32)
+    for s in range(batch):
+        table[s] = torch.arange(s * per, (s + 1) * per, dtype=torch.int32)
+        for pos in range(lens[s]):
+            k_cache[s * per + pos // page, :, pos % page] = ks[s][pos].to(bf)
+            v_cache[s * per + pos // page, :, pos % page] = vs[s][pos].to(bf)
+    v_cache = v_cache.transpose(2, 3).contiguous()
+    from tests.helpers import context_from_spans
+
+    step = context_from_spans([(1, n - 1) for n in lens], DEV)
+    q_flat = torch.cat([q.reshape(1, n_q * d) for q in qs]).to(bf).to(DEV)
+    attended = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, n - 1)
+                          for q, k, v, n in zip(qs, ks, vs, lens)]).reshape(batch, n_q * d)
+    start = rnd(batch, hidden, seed=77)
+    want = start + rounded(attended, bf) @ w_o.T
+    results = {}
+    for fold in (True, False):
+        h = start.clone().to(DEV)
+        left = ops().attention_project(q_flat, n_q * d, k_cache.to(DEV), v_cache.to(DEV), step,
+                                       table.to(DEV), n_q, n_kv, d, d ** -0.5, None,
+                                       w_o.to(bf).to(DEV), None, h, fold=fold)
+        if fold:
+            assert left is not None and left.shape[1:] == (batch, hidden) and 1 < left.shape[0] <= 16
+        results[fold] = (h + (left.sum(0) if left is not None else 0)).cpu()
+    torch.testing.assert_close(results[True], want, atol=2e-2, rtol=2e-2)
+    torch.testing.assert_close(results[False], want, atol=2e-2, rtol=2e-2)
+    # the two paths round the merged rows to bfloat16 alike and differ in the order of sums only
+    torch.testing.assert_close(results[True], results[False], atol=2e-3, rtol=2e-3)
+    # steps the folded kernel does not take are refused when it is asked for by name
+    prompt = context_from_spans([(5, 100)], DEV)
+    with pytest.raises(RuntimeError, match="do not take the folded merge"):
+        ops().attention_project(q_flat[:5].contiguous(), n_q * d, k_cache.to(DEV), v_cache.to(DEV),
+                                prompt, table[:1].to(DEV), n_q, n_kv, d, d ** -0.5, None,
+                                w_o.to(bf).to(DEV), None, torch.zeros(5, hidden, device=DEV), fold=True)
+
+
 @pytest.mark.parametrize("dtype,kernel", [(torch.float32, "generic"), (torch.bfloat16, "mfma")])
 @pytest.mark.parametrize("q_len", [1, 40])
 def test_attention_over_a_very_long_context(dtype, kernel, q_len):
