@@ -241,22 +241,36 @@ __global__ void rmsnorm_vec_kernel(float* __restrict__ h, const float* __restric
       if (idx >= chunks) continue;
       const float4* p4 = (const float4*)(partials + (size_t)in_row * hidden) + idx;
       const size_t stride4 = partial_stride >> 2;
+      // Up to sixteen slices' loads are in flight at once (a decode step's norm is a chain of
+      // round trips to the L2 and little else); the additions keep their order: groups of
+      // four as (a + b) + (c + d), group after group, then what is left one by one.
       float4 t = make_float4(0.f, 0.f, 0.f, 0.f);
-      int k = 0;
-      for (; k + 4 <= num_partials; k += 4) {
-        const float4 a = p4[(size_t)k * stride4], b = p4[(size_t)(k + 1) * stride4];
-        const float4 cc = p4[(size_t)(k + 2) * stride4], d = p4[(size_t)(k + 3) * stride4];
-        t.x += (a.x + b.x) + (cc.x + d.x);
-        t.y += (a.y + b.y) + (cc.y + d.y);
-        t.z += (a.z + b.z) + (cc.z + d.z);
-        t.w += (a.w + b.w) + (cc.w + d.w);
-      }
-      for (; k < num_partials; ++k) {
-        const float4 a = p4[(size_t)k * stride4];
-        t.x += a.x;
-        t.y += a.y;
-        t.z += a.z;
-        t.w += a.w;
+      for (int k0 = 0; k0 < num_partials; k0 += 16) {
+        float4 part[16];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+          part[j] = k0 + j < num_partials ? p4[(size_t)(k0 + j) * stride4]
+                                          : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 16; j += 4) {
+          if (k0 + j + 4 <= num_partials) {
+            t.x += (part[j].x + part[j + 1].x) + (part[j + 2].x + part[j + 3].x);
+            t.y += (part[j].y + part[j + 1].y) + (part[j + 2].y + part[j + 3].y);
+            t.z += (part[j].z + part[j + 1].z) + (part[j + 2].z + part[j + 3].z);
+            t.w += (part[j].w + part[j + 1].w) + (part[j + 2].w + part[j + 3].w);
+          } else {
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+              if (k0 + j + i < num_partials) {
+                t.x += part[j + i].x;
+                t.y += part[j + i].y;
+                t.z += part[j + i].z;
+                t.w += part[j + i].w;
+              }
+            }
+          }
+        }
       }
       v[c] = make_float4(v[c].x + t.x, v[c].y + t.y, v[c].z + t.z, v[c].w + t.w);
       x4[idx] = v[c];
