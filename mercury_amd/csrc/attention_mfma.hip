@@ -1252,6 +1252,23 @@ extern "C" int mk_attention_mfma_wide(int head_dim) {
   return head_dim == 64 ? 0b101 : (head_dim == 128 ? 0b011 : 0);
 }
 
+// From how many workgroups of 128 rows on the kernel of 32-row wavefronts measured faster
+// than the 16-row kernels, for the instantiation of this head size with `chains` key groups
+// (0: no such instantiation).  The numbers belong to the instantiations, which is why they
+// stand here and not with the planner:
+//   64-wide heads, one chain: 14 heads in 2 groups at 2,048 tokens, 224 workgroups, 34 us
+//   against 30; 4 x 2,048, 896: 73 against 90; 8,192: 202 against 288.  Three chains: 2,048
+//   tokens, 224 workgroups, 30.6 us against 30.2; 4,096, 448: 64 against 89; 2,048 over 6,144:
+//   102 against 139; 512 over 1,536, 56: 28 against 22.
+//   128-wide heads, one chain: 28 heads in 4 groups at 2,048 tokens, 448 workgroups: 85
+//   against 96; 8,192: 752 against 969.  Two chains: 512 tokens over 1,536, 112: 54 against
+//   41; 40 heads in 8 groups there, 160: 54 against 67.
+extern "C" int mk_attention_mfma_wide_from(int head_dim, int chains) {
+  if (head_dim == 64) return chains == 1 ? 512 : (chains == 3 ? 192 : 0);
+  if (head_dim == 128) return chains == 1 ? 256 : (chains == 2 ? 128 : 0);
+  return 0;
+}
+
 extern "C" int mk_attention_mfma_supported(int head_dim, int page_size) {
   const bool d_ok = head_dim == 32 || head_dim == 64 || head_dim == 96 || head_dim == 128 ||
                     head_dim == 192 || head_dim == 256;

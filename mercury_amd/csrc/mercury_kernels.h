@@ -168,6 +168,9 @@ int mk_attention_mfma_max_rows(int head_dim);
 // without the launch (0: it would take them; else mk_last_error() says why not).
 int mk_attention_mfma_staged(int head_dim, int rows_per_tile);
 int mk_attention_mfma_wide(int head_dim);
+// From how many workgroups of 128 rows on the kernel of 32-row wavefronts with `chains` key
+// groups is the faster one at this head size (0: no such instantiation).
+int mk_attention_mfma_wide_from(int head_dim, int chains);
 int mk_attention_mfma_check(int q_stride, int out_stride, int num_tiles, int page_size, int n_q,
                             int n_kv, int d, float scale, int window, int rows_per_tile,
                             int staged, int num_splits, int split_blocks, int has_workspace);

@@ -27,19 +27,6 @@ constexpr int kFusedQkvMinWorkgroups = 128;
 
 constexpr int kAttentionTargetWaves = 1024;
 constexpr int kAttentionStagedWorkgroups = 64;
-// workgroups of 128 rows from which the kernel of 32-row wavefronts wins over the 16-row one
-// (14 heads of 64 in 2 groups: 2,048 tokens, 224 workgroups, 34 us against 30; 4 x 2,048, 896:
-// 73 against 90; 8,192: 202 against 288.  28 heads of 128 in 4 groups: 2,048 tokens, 448: 85
-// against 96; 8,192: 752 against 969; 512 tokens over 1,536, 112: 54 against 41; 40 heads in 8
-// groups there, 160: 54 with two key groups against 67; 14 heads of 64 at 4,096 tokens, 448
-// workgroups: 97 against 91 with four key groups)
-constexpr int kAttentionWideWorkgroups64 = 512;
-constexpr int kAttentionWideWorkgroups128 = 256;
-constexpr int kAttentionWideSplitWorkgroups128 = 128;
-// 14 heads of 64 with the keys in three chains: 2,048 tokens, 224 workgroups, 30.6 us against
-// 30.2; 4,096, 448: 64 against 89; 2,048 over 6,144: 102 against 139; 512 over 1,536, 56: 28
-// against 22
-constexpr int kAttentionWideSplitWorkgroups64 = 192;
 constexpr int kAttentionStagedMaxWaves = 16384;
 constexpr int kAttentionWideTileWaves = 400;
 constexpr int kAttentionMinBlocksPerSplit = 2;
@@ -153,11 +140,12 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   if (staged < 0 && !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 128) {
     const int chains = t.mk_attention_mfma_wide(head_dim);   // bit n - 1: n chains exist
     const long long workgroups = (total_rows / 128) * n_kv;
-    const long long full = head_dim == 64 ? kAttentionWideWorkgroups64 : kAttentionWideWorkgroups128;
-    const long long few = head_dim == 64 ? kAttentionWideSplitWorkgroups64 : kAttentionWideSplitWorkgroups128;
     const int most = (chains & 4) ? 3 : ((chains & 2) ? 2 : 1);
+    // the counts from which each instantiation measured faster are the kernel library's
+    const long long full = t.mk_attention_mfma_wide_from(head_dim, 1);
+    const long long few = most > 1 ? t.mk_attention_mfma_wide_from(head_dim, most) : 0;
     if ((chains & 1) && (workgroups >= full ||
-                         (head_dim == 64 && workgroups >= 3 * full / 4 && blocks < 32 * most))) {
+                         (most > 2 && workgroups >= 3 * full / 4 && blocks < 32 * most))) {
       // (three quarters of that many with chains too short to cut: 28 heads of 64, 2,048
       // tokens, 448 workgroups: 44 us against 47 in the 16-row kernel)
       staged = 8;
