@@ -10,6 +10,9 @@
 //
 // Scores, softmax and the weighted sum are float32 (reference formulas:
 // mercury/model/attention.py:9-32 and :87-101, scale = head_dim^-0.5 passed by the caller).
+// Two modifications of the score the reference does not have, for mixers that want them:
+// score_cap > 0 bounds it to cap * tanh(score / cap), and distance_slopes [n_q] subtracts
+// slope[head] * (query position - key position), a position encoding that lives in the score.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -21,7 +24,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
     const T* __restrict__ k_cache, const T* __restrict__ v_cache,
     const int* __restrict__ positions, const int* __restrict__ token_seq,
     const int* __restrict__ block_table, int table_stride, int page_shift, int n_q, int n_kv,
-    int d, float scale, int window) {
+    int d, float scale, int window, float score_cap, const float* __restrict__ distance_slopes) {
   __shared__ float qs[AG_MAX_D];
   __shared__ float probs[MK_WAVE];
   const int t = blockIdx.x, head = blockIdx.y, lane = threadIdx.x;
@@ -30,6 +33,7 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
   const int* table = block_table + (size_t)token_seq[t] * table_stride;
   const int page_size = 1 << page_shift, page_mask = page_size - 1;
   const int first = window > 0 ? max(0, pos - window + 1) : 0;
+  const float slope = distance_slopes ? distance_slopes[head] : 0.f;
 
   for (int i = lane; i < d; i += MK_WAVE)
     qs[i] = Elem<T>::load(q + (size_t)t * q_stride + head * d + i);
@@ -50,6 +54,10 @@ __global__ __launch_bounds__(64) void attention_generic_kernel(
       float dot = 0.f;
       for (int i = 0; i < d; ++i) dot = fmaf(qs[i], Elem<T>::load(krow + i), dot);
       score = dot * scale;
+      // a smooth bound on the score, then a penalty that grows with the distance: both leave
+      // the order of the sums alone
+      if (score_cap > 0.f) score = score_cap * tanhf(score / score_cap);
+      score -= slope * (float)(pos - j);
     }
     const float m_new = fmaxf(m, wave_max(score));
     const float p = j <= pos ? expf(score - m_new) : 0.f;
@@ -91,7 +99,8 @@ extern "C" int mk_attention_generic(const void* q, int q_stride, void* out, int 
                                     const int* positions, const int* token_seq,
                                     const int* block_table, int table_stride, int page_size,
                                     int n_q, int n_kv, int d, float scale, int window,
-                                    int tokens, hipStream_t stream) {
+                                    float score_cap, const float* distance_slopes, int tokens,
+                                    hipStream_t stream) {
   MK_REQUIRE(tokens >= 0 && n_q > 0 && n_kv > 0 && d > 0, "attention: bad sizes");
   MK_REQUIRE(n_q % n_kv == 0, "attention: %d query heads are not a multiple of %d kv heads",
              n_q, n_kv);
@@ -100,18 +109,19 @@ extern "C" int mk_attention_generic(const void* q, int q_stride, void* out, int 
   MK_REQUIRE(mk_is_pow2(page_size), "attention: page size %d is not a power of two", page_size);
   MK_REQUIRE(n_q <= 65535, "attention: too many heads (%d)", n_q);
   MK_REQUIRE(window >= 0, "attention: negative window");
+  MK_REQUIRE(score_cap >= 0.f, "attention: negative score cap");
   if (tokens == 0) return 0;
   dim3 grid(tokens, n_q);
   if (dtype == MK_F32)
     attention_generic_kernel<float><<<grid, MK_WAVE, 0, stream>>>(
         (const float*)q, q_stride, (float*)out, out_stride, (const float*)k_cache,
         (const float*)v_cache, positions, token_seq, block_table, table_stride,
-        mk_log2(page_size), n_q, n_kv, d, scale, window);
+        mk_log2(page_size), n_q, n_kv, d, scale, window, score_cap, distance_slopes);
   else if (dtype == MK_BF16)
     attention_generic_kernel<bf16_t><<<grid, MK_WAVE, 0, stream>>>(
         (const bf16_t*)q, q_stride, (bf16_t*)out, out_stride, (const bf16_t*)k_cache,
         (const bf16_t*)v_cache, positions, token_seq, block_table, table_stride,
-        mk_log2(page_size), n_q, n_kv, d, scale, window);
+        mk_log2(page_size), n_q, n_kv, d, scale, window, score_cap, distance_slopes);
   else
     MK_REQUIRE(false, "attention: unknown dtype %d", dtype);
   MK_LAUNCH_CHECK("attention_generic");

@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 15
+#define MK_ABI_VERSION 16
 
 #ifdef __cplusplus
 extern "C" {
@@ -65,12 +65,15 @@ int mk_linear_generic(const void* x, const void* w, int dtype, const void* bias,
                       int ldo, hipStream_t stream);
 
 // Causal grouped-query attention over the paged cache for any mix of prompt portions and
-// decoded tokens; window = 0 means all earlier keys.
+// decoded tokens; window = 0 means all earlier keys.  score_cap > 0: the scaled score becomes
+// cap * tanh(score / cap); distance_slopes (float32 [n_q], or null): slope[head] * (query
+// position - key position) is subtracted from it.
 int mk_attention_generic(const void* q, int q_stride, void* out, int out_stride,
                          const void* k_cache, const void* v_cache, int dtype,
                          const int* positions, const int* token_seq, const int* block_table,
                          int table_stride, int page_size, int n_q, int n_kv, int d, float scale,
-                         int window, int tokens, hipStream_t stream);
+                         int window, float score_cap, const float* distance_slopes, int tokens,
+                         hipStream_t stream);
 
 // mk_rope_kv_write for a projection that arrives as float32 partial sums [p, T, width] of a
 // K-split product: the slices are added in order (with the bias) before the rotation; q goes

@@ -84,6 +84,8 @@ AttendArgs attend_from(const py::dict& d) {
   a.scale = get<float>(d, "scale", 0.f);
   a.k_cache = ptr_of<const void>(d, "k_cache");
   a.v_cache = ptr_of<const void>(d, "v_cache");
+  a.score_cap = get<float>(d, "score_cap", 0.f);
+  a.distance_slopes = ptr_of<const float>(d, "distance_slopes");
   return a;
 }
 
@@ -212,6 +214,8 @@ void bind_ops(py::module_& m) {
     p.group = get<int>(d, "group", 0);
     p.window = get<int>(d, "window", 0);
     p.scale = get<float>(d, "scale", 0.f);
+    p.score_cap = get<float>(d, "score_cap", 0.f);
+    p.distance_slopes = ptr_of<const float>(d, "distance_slopes");
     return blob(p);
   });
   m.def("gated_mlp_params", [](uintptr_t w_gate_up, uintptr_t w_down, int inter) {

@@ -70,6 +70,8 @@ AttendArgs attend_args(const AttentionParams& p) {
   a.scale = p.scale;
   a.k_cache = p.qkv.k_cache;
   a.v_cache = p.qkv.v_cache;
+  a.score_cap = p.score_cap;
+  a.distance_slopes = p.distance_slopes;
   return a;
 }
 

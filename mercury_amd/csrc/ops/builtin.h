@@ -32,6 +32,8 @@ struct AttentionParams {
   int group = 0;          // which of the step's block tables
   int window = 0;
   float scale = 0.f;
+  float score_cap = 0.f;                    // > 0: the score is bounded to cap * tanh(. / cap)
+  const float* distance_slopes = nullptr;   // [n_q]: slope * distance is subtracted from it
 };
 
 // "gated_mlp": h += (act(x Wg^T) * (x Wu^T)) Wd^T (or left as partial sums).

@@ -173,6 +173,12 @@ Queries qkv_project(Launch& l, const void* x, int m, int k, const QkvArgs& a, co
 
 AttentionPlan plan_for(int dtype, const AttendArgs& a, const mk_step_view& step,
                        const AttendForce& force) {
+  if (!a.plain_scores()) {
+    if (force.kernel == 2) {
+      throw KernelError("attention: the matrix-core kernels neither cap nor bias the score");
+    }
+    return AttentionPlan();     // the float32-arithmetic kernel
+  }
   const std::vector<int> counts(step.counts, step.counts + step.num_seqs);
   return plan_attention(dtype, a.head_dim, a.page_size, a.n_q, a.n_kv, a.window, counts,
                         step.max_q_len, step.max_kv_len, force.kernel, force.tile_rows, force.staged,
@@ -200,7 +206,7 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
       check_core(need_core().mk_attention_generic(
                      q.q, q.stride, out, a.n_q * d, a.k_cache, a.v_cache, l.dtype(), s.positions,
                      s.token_seq, s.table, s.table_stride, a.page_size, a.n_q, a.n_kv, d, a.scale,
-                     a.window, m, l.stream()), "attention");
+                     a.window, a.score_cap, a.distance_slopes, m, l.stream()), "attention");
     }
     return out;
   }

@@ -117,6 +117,12 @@ struct AttendArgs {
   int n_q = 0, n_kv = 0, head_dim = 0, page_size = 0, window = 0;
   float scale = 0.f;
   const void *k_cache = nullptr, *v_cache = nullptr;
+  // What only the float32-arithmetic kernel computes: a bound cap * tanh(score / cap) on the
+  // score, and a penalty slope[head] * distance subtracted from it.  With either, that kernel
+  // runs whatever the dtype.
+  float score_cap = 0.f;
+  const float* distance_slopes = nullptr;
+  bool plain_scores() const { return score_cap <= 0.f && distance_slopes == nullptr; }
 };
 
 struct AttendForce {

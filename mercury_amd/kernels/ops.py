@@ -488,7 +488,9 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
               step, block_table: torch.Tensor, n_q: int, n_kv: int, head_dim: int, scale: float,
               window: int | None = None, out: torch.Tensor | None = None,
               kernel: str = "auto", tile_rows: int | None = None,
-              split_override: tuple | None = None, staged: bool | None = None) -> torch.Tensor:
+              split_override: tuple | None = None, staged: bool | None = None,
+              score_cap: float | None = None,
+              distance_slopes: torch.Tensor | None = None) -> torch.Tensor:
     """Causal grouped-query attention of every token of the step over its sequence's cached
     keys; q is read from rows of `q` with stride `q_stride` (the fused qkv buffer).
     `step` describes the batch (positions, token_seq, cu_q, kv_len, spans, tiles());
@@ -501,8 +503,14 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
     (False, or 1, 2 or 4 groups of wavefronts that split a workgroup's keys among them)
     whether workgroups of four wavefronts share the keys and values of one sequence's rows
     through LDS; by default the step's size decides all three.
+    score_cap bounds the scaled score to cap * tanh(score / cap); distance_slopes (float32
+    [n_q]) subtracts slope[head] * (query position - key position) from it.  With either the
+    float32-arithmetic kernel runs, whatever the dtype.
     """
-    _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out)
+    _dev(q, k_cache, v_cache, step.positions, step.token_seq, block_table, out, distance_slopes)
+    if distance_slopes is not None and (distance_slopes.dtype != torch.float32
+                                        or distance_slopes.shape != (n_q,)):
+        raise KernelArgumentError(f"attention: distance_slopes must be float32 [{n_q}]")
     tokens = step.num_tokens
     if q.numel() < (tokens - 1) * q_stride + n_q * head_dim and tokens:
         raise KernelArgumentError("attention: q buffer too small")
@@ -519,7 +527,8 @@ def attention(q: torch.Tensor, q_stride: int, k_cache: torch.Tensor, v_cache: to
                  split_blocks=split_override[1] if split_override is not None else 0)
     args = dict(n_q=n_q, n_kv=n_kv, head_dim=head_dim, page_size=page_size,
                 window=int(window or 0), scale=float(scale), k_cache=_ptr(k_cache),
-                v_cache=_ptr(v_cache))
+                v_cache=_ptr(v_cache), score_cap=float(score_cap or 0.0),
+                distance_slopes=_ptr(distance_slopes))
 
     def tiles(group, rows):
         seq, row0, count = step.tiles(group, rows)

@@ -23,6 +23,9 @@ class Attention(Mixer):
     keys j <= p, and with a window only j > p - window
     (reference: mercury/model/qwen2.py:45-69, mercury/model/attention.py:9-32, :87-101).
     `names` maps q, k, v, o to the stored tensors' leaf names (default ``q_proj`` ...).
+    `score_cap` bounds the scaled score to cap * tanh(score / cap); a position encoding may
+    bring a penalty on the distance in the score (`PositionDescriptor.distance_slopes`).  The
+    reference has neither; with either the float32-arithmetic attention kernel runs.
     """
 
     graph_safe = True   # forward launches kernels only: a decode step may be captured in a graph
@@ -30,7 +33,7 @@ class Attention(Mixer):
     def __init__(self, hidden: int, n_q: int, n_kv: int, head_dim: int,
                  position: PositionEncoding, qkv_bias: bool = True, o_bias: bool = False,
                  scale: float | None = None, window: int | None = None,
-                 names: dict | None = None):
+                 names: dict | None = None, score_cap: float | None = None):
         if n_q % n_kv:
             raise ValueError(f"{n_q} query heads are not a multiple of {n_kv} key/value heads")
         self.hidden, self.n_q, self.n_kv, self.head_dim = int(hidden), int(n_q), int(n_kv), int(head_dim)
@@ -38,6 +41,7 @@ class Attention(Mixer):
         self.qkv_bias, self.o_bias = bool(qkv_bias), bool(o_bias)
         self.scale = float(scale) if scale is not None else self.head_dim ** -0.5
         self.window = int(window) if window else None
+        self.score_cap = float(score_cap) if score_cap else 0.0
         self.names = {**DEFAULT_NAMES, **(names or {})}
         self.w_qkv = self.b_qkv = self.w_o = self.b_o = None
         self._alone: dict = {}
@@ -120,7 +124,8 @@ class Attention(Mixer):
             table_positions=0 if pos.cos is None else pos.cos.shape[0],
             interleaved=pos.interleaved, k_cache=cache.k.data_ptr(), v_cache=cache.v.data_ptr(),
             group=cache.group, page_size=cache.page_size, scale=self.scale,
-            window=self.window or 0, writes=cache.writes))
+            window=self.window or 0, writes=cache.writes, score_cap=self.score_cap,
+            distance_slopes=ptr(pos.distance_slopes)))
 
     def forward(self, x, step, cache, state, accum):
         if self.position.describe() is not None:
@@ -148,5 +153,5 @@ class Attention(Mixer):
         ops.rope_kv_write(q, None, None, step.positions, step.token_seq, table, k_cache,
                           v_cache, n_q, heads_kv, d, 0, cache.writes)
         attended = ops.attention(q, q.shape[1], cache.k, cache.v, step, table, n_q, n_kv, d,
-                                 self.scale, self.window)
+                                 self.scale, self.window, score_cap=self.score_cap)
         return ops.project_into_stream(attended, self.w_o, self.b_o, accum)

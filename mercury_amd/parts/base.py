@@ -122,12 +122,16 @@ class PositionDescriptor:
     """A position encoding as the kernels understand it: the first `rotary_dim` dims of every
     query and key head are turned by the angle tables `cos` / `sin` ([positions, rotary_dim/2],
     float32), pair j being dims (j, j + rotary_dim/2) of the head, or (2j, 2j + 1) when
-    `interleaved`.  rotary_dim 0: queries and keys stay as projected."""
+    `interleaved`.  rotary_dim 0: queries and keys stay as projected.  `distance_slopes`
+    (float32 [query heads]): an encoding that lives in the score, slope[head] * (query position
+    - key position) being subtracted from it (the float32-arithmetic attention kernel computes
+    that; the matrix-core kernels do not)."""
 
     rotary_dim: int = 0
     cos: torch.Tensor | None = None
     sin: torch.Tensor | None = None
     interleaved: bool = False
+    distance_slopes: torch.Tensor | None = None
 
 
 class Part:

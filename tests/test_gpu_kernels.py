@@ -927,6 +927,64 @@ def test_attention_over_a_very_long_context(dtype, kernel, q_len):
     assert got[-1, 0].mean() > 6.0                       # the far value dominates that head
 
 
+def slow_attention_with_score_terms(q, k, v, scale, cap, slopes):
+    """q [n_q, d] at the last position of k, v [S, n_kv, d]: softmax over
+    cap * tanh(score / cap) - slope[head] * distance, written out."""
+    n_q, n_kv = q.shape[0], k.shape[1]
+    group = n_q // n_kv
+    last = k.shape[0] - 1
+    out = torch.zeros_like(q)
+    for head in range(n_q):
+        scores = (k[:, head // group] @ q[head]) * scale
+        if cap:
+            scores = cap * torch.tanh(scores / cap)
+        if slopes is not None:
+            scores = scores - slopes[head] * (last - torch.arange(k.shape[0])).float()
+        out[head] = torch.softmax(scores, dim=0) @ v[:, head // group]
+    return out
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("cap,with_slopes", [(5.0, False), (None, True), (3.0, True)])
+def test_attention_with_a_capped_score_and_a_distance_penalty(dtype, cap, with_slopes):
+    """What the reference's attention does not have and another mixer may want: the score
+    bounded by cap * tanh(. / cap), and slope[head] * distance subtracted from it (a position
+    encoding that lives in the score).  The float32-arithmetic kernel computes both, in
+    either dtype; the matrix-core kernel refuses them."""
+    n_q, n_kv, d, page = 6, 2, 32, 16
+    lens = [70, 33, 5]
+    slopes = torch.tensor([0.5 ** (i + 1) for i in range(n_q)]) if with_slopes else None
+    qs = [rounded(rnd(1, n_q, d, seed=20 + i, scale=2.0), dtype) for i in range(len(lens))]
+    ks = [rounded(rnd(n, n_kv, d, seed=30 + i, scale=2.0), dtype) for i, n in enumerate(lens)]
+    vs = [rounded(rnd(n, n_kv, d, seed=40 + i), dtype) for i, n in enumerate(lens)]
+    per = -(-max(lens) // page)
+    k_cache = torch.zeros(len(lens) * per, n_kv, page, d, dtype=dtype)
+    v_cache = torch.zeros_like(k_cache)
+    table = torch.zeros((len(lens), per), dtype=torch.int32)
+    for s, n in enumerate(lens):
+        table[s] = torch.arange(s * per, (s + 1) * per, dtype=torch.int32)
+        for pos in range(n):
+            k_cache[s * per + pos // page, :, pos % page] = ks[s][pos].to(dtype)
+            v_cache[s * per + pos // page, :, pos % page] = vs[s][pos].to(dtype)
+    from tests.helpers import context_from_spans
+
+    step = context_from_spans([(1, n - 1) for n in lens], DEV)
+    q_flat = torch.cat([q.reshape(1, n_q * d) for q in qs]).to(dtype).to(DEV)
+    args = (q_flat, n_q * d, k_cache.to(DEV), v_cache.transpose(2, 3).contiguous().to(DEV), step,
+            table.to(DEV), n_q, n_kv, d, d ** -0.5, None)
+    got = ops().attention(*args, score_cap=cap,
+                          distance_slopes=None if slopes is None else slopes.to(DEV))
+    want = torch.stack([slow_attention_with_score_terms(q[0], k, v, d ** -0.5, cap, slopes)
+                        for q, k, v in zip(qs, ks, vs)])
+    torch.testing.assert_close(got.float().cpu().view(-1, n_q, d), want, **tol(dtype))
+    # the terms matter: without them the result is another
+    bare = ops().attention(*args).float().cpu().view(-1, n_q, d)
+    assert float((bare - want).abs().max()) > 10 * tol(dtype)["atol"]
+    if dtype == torch.bfloat16:
+        with pytest.raises(RuntimeError, match="neither cap nor bias"):
+            ops().attention(*args, score_cap=cap or 1.0, kernel="mfma")
+
+
 def test_attention_gqa_equals_mha_with_repeated_heads():
     n_q, n_kv, d, page, s = 6, 2, 16, 16, 37
     q, k, v = (rnd(s, h, d, seed=90 + i) for i, h in enumerate((n_q, n_kv, n_kv)))

@@ -272,6 +272,93 @@ def test_embedding_scale_head_bias_and_cap_change_the_logits(tmp_path):
     assert math.isclose(SCALE, 3.0)
 
 
+def test_a_position_encoding_that_lives_in_the_score(tmp_path):
+    """Another position encoding, registered from outside: no rotation, but a penalty
+    slope[head] * distance in the score (and a cap on the score beside it).  It describes
+    itself to the kernels, so its layers stay inside the program; the slow version is written
+    out here.  Only distances enter, so shifting all positions changes nothing."""
+    from mercury_amd.config import Qwen2Config, register_architecture
+    from mercury_amd.engine.replay import ReplaySession
+    from mercury_amd.parts import (Attention, DecoderModel, GatedMLP, PositionDescriptor,
+                                   PositionEncoding, PreNormBlock, RMSNorm, register_position)
+    from mercury_amd.weights import write_random_model
+
+    cap = 4.0
+
+    @register_position("test_distance_penalty")
+    class DistancePenalty(PositionEncoding):
+        def __init__(self, heads):
+            self.values = [2.0 ** -(i + 1) for i in range(heads)]
+            self.slopes = None
+
+        def prepare(self, max_positions, device):
+            self.slopes = torch.tensor(self.values, dtype=torch.float32, device=device)
+
+        def describe(self):
+            return PositionDescriptor(distance_slopes=self.slopes)
+
+    @register_architecture("TestDistanceLM", Qwen2Config)
+    def build(cfg):
+        h, eps = cfg.hidden_size, cfg.rms_norm_eps
+        layers = [PreNormBlock(
+            Attention(h, cfg.num_attention_heads, cfg.num_key_value_heads, cfg.head_dim,
+                      DistancePenalty(cfg.num_attention_heads), qkv_bias=False, score_cap=cap),
+            GatedMLP(h, cfg.intermediate_size), RMSNorm(h, eps), RMSNorm(h, eps),
+            {"mixer": "self_attn.", "ffn": "mlp.", "norm_mixer": "input_layernorm.",
+             "norm_ffn": "post_attention_layernorm."}) for _ in range(cfg.num_hidden_layers)]
+        return DecoderModel(cfg.vocab_size, h, layers, RMSNorm(h, eps), tied_head=True,
+                            max_positions=cfg.max_position_embeddings, config=cfg)
+
+    config = {**helpers.TINY_A, "architectures": ["TestDistanceLM"], "hidden_size": 96,
+              "num_attention_heads": 3, "num_key_value_heads": 1, "head_dim": 32,
+              "intermediate_size": 136, "vocab_size": 301}
+    folder = write_random_model(tmp_path / "distance", config, seed=6, std=0.15, dtype=torch.float32)
+    w, cfg = helpers.plain_model(folder)
+    tokens = helpers.random_tokens(301, 50, 5)
+
+    def slow(tokens, w):
+        """In the weights' own dtype, scores and softmax in float32, the stream in float32."""
+        n_q, n_kv, d, eps = 3, 1, 32, cfg["rms_norm_eps"]
+        dtype = w["model.embed_tokens.weight"].dtype
+        slopes = torch.tensor([2.0 ** -(i + 1) for i in range(n_q)])
+        h = w["model.embed_tokens.weight"][torch.tensor(tokens)].float()
+        positions = torch.arange(len(tokens))
+        distance = (positions[:, None] - positions[None, :]).float()
+        for i in range(cfg["num_hidden_layers"]):
+            p = f"model.layers.{i}."
+            x = plain.rms_norm(h.to(dtype), w[p + "input_layernorm.weight"], eps)[0]
+            q = (x @ w[p + "self_attn.q_proj.weight"].T).view(-1, n_q, d).float()
+            k = (x @ w[p + "self_attn.k_proj.weight"].T).view(-1, n_kv, d).float()
+            v = (x @ w[p + "self_attn.v_proj.weight"].T).view(-1, n_kv, d).float()
+            scores = torch.einsum("qhd,kd->hqk", q, k[:, 0]) * d ** -0.5
+            scores = cap * torch.tanh(scores / cap) - slopes[:, None, None] * distance[None]
+            scores = scores.masked_fill(distance[None] < 0, float("-inf"))
+            attended = torch.einsum("hqk,kd->qhd", torch.softmax(scores, -1), v[:, 0]).to(dtype)
+            h = h + (attended.reshape(len(tokens), -1) @ w[p + "self_attn.o_proj.weight"].T).float()
+            x = plain.rms_norm(h.to(dtype), w[p + "post_attention_layernorm.weight"], eps)[0]
+            h = h + plain.gated_mlp(x, w[p + "mlp.gate_proj.weight"], w[p + "mlp.up_proj.weight"],
+                                    w[p + "mlp.down_proj.weight"]).float()
+        x = plain.rms_norm(h.to(dtype), w["model.norm.weight"], eps)[0]
+        return (x @ w["model.embed_tokens.weight"].T).float()
+
+    want = slow(tokens, w)
+    # what bfloat16 costs the slow version itself, times the slack the replay tests use
+    cost = float((slow(tokens, {n: t.bfloat16() for n, t in w.items()}) - want).abs().max())
+    for dtype, tol in (("float32", dict(atol=2e-5, rtol=1e-4)),
+                       ("bfloat16", dict(atol=1.5 * cost, rtol=0))):
+        s = ReplaySession(folder, dtype, 128)
+        assert "host" not in s.runner.program.kinds
+        whole = s.step([{"id": "a", "tokens": tokens, "want": list(range(50))}], ["a"])
+        torch.testing.assert_close(whole, want, **tol)
+        rows = [s.step([{"id": "b", "tokens": tokens[:31], "want": list(range(31))}], [])]
+        for i in range(31, 50):
+            rows.append(s.step([{"id": "b", "tokens": tokens[i:i + 1], "want": [0]}],
+                               ["b"] if i == 49 else []))
+        torch.testing.assert_close(torch.cat(rows), want, **tol)
+        if dtype == "float32":
+            assert torch.equal(torch.cat(rows), whole)     # the order of sums is the position's own
+
+
 def test_a_subclass_that_overrides_forward_is_not_lowered():
     """`lower` describes the base class's work.  A subclass with a `forward` of its own must
     run through that `forward`, as a step the caller runs; one that also brings its own
