@@ -719,30 +719,32 @@ struct WideLane {
 };
 
 template <int D>
-__device__ __forceinline__ WideLane wide_lane(int page_size, int lane, int wave) {
+__device__ __forceinline__ WideLane wide_lane(int page_size, int lane, int load) {
   constexpr int KEYS_PER_LOAD = 512 / D, CH = D / 8;
-  const int key = wave * KEYS_PER_LOAD + lane / CH;      // of load j = 0; load j is 4 j loads on
+  const int key = load * KEYS_PER_LOAD + lane / CH;      // only key % 16 and load % (D / 64) count
   const int slot = lane % CH;
   const int chunk = wide_chunk_swizzle<D>(key, slot);    // the chunk that lies at the lane's slot
-  const int dim = ((wave % (D / 64)) * 64 + lane) % D;
+  const int dim = ((load % (D / 64)) * 64 + lane) % D;
   WideLane out;
   out.k_at = (uint32_t)(key & 15) * (uint32_t)(D * 2) + (uint32_t)chunk * 16u;
   out.v_at = (uint32_t)dim * (uint32_t)(page_size * 2);
   return out;
 }
 
-// The loads of one block by one wavefront, D / 32 of keys and as many of values, into the
-// ring buffer at LDS byte address `dst`.  Load j of the keys brings 1024 bytes of rows
-// (8 keys at D = 64, 4 at D = 128), load j of the values 64 dims of one piece of 8 keys; both
-// lie in the stretch of 16 keys number (wave / 2) + 2 j (D = 64) or j (D = 128) of the
-// block, so the page is looked up once for the pair, everything but the lane's own offset is
-// the wavefront's (scalar) arithmetic, and the load takes that base and a 32-bit offset.
-// Keys outside what the workgroup's rows see (or past the group's last block) are fetched
-// from page 0, which always exists, and masked in the scores.
-template <int D>
+// The loads of one block by one of the GW wavefronts that share it, D / (8 GW) of keys and as
+// many of values, into the ring buffer at LDS byte address `dst`.  Load number n of the keys
+// brings 1024 bytes of rows (8 keys at D = 64, 4 at D = 128), load n of the values 64 dims of
+// one piece of 8 keys; both lie in the same stretch of 16 keys of the block, so the page is
+// looked up once for the pair, everything but the lane's own offset is the wavefront's
+// (scalar) arithmetic, and the load takes that base and a 32-bit offset.  The wavefront's
+// loads are numbers wave, wave + GW, ...: a lane's offset is the same for all of them where
+// GW loads are a whole number of 16-key stretches, and alternates between two otherwise
+// (`mine[j % 2]`).  Keys outside what the workgroup's rows see (or past the group's last
+// block) are fetched from page 0, which always exists, and masked in the scores.
+template <int D, int GW>
 __device__ __forceinline__ void wide_fetch(const AttnParams& p, TableWindow& tw, int b, int b_end,
                                            int kmin, int kmax, int kvh, int lane, int wave,
-                                           unsigned int dst, const WideLane& mine) {
+                                           unsigned int dst, const WideLane (&mine)[2]) {
   constexpr int KEYS_PER_LOAD = 512 / D;
   const int ps = 1 << p.page_shift;
   const uint32_t head_bytes = (uint32_t)ps * D * 2;
@@ -750,8 +752,9 @@ __device__ __forceinline__ void wide_fetch(const AttnParams& p, TableWindow& tw,
   const uint32_t head_at = (uint32_t)kvh * head_bytes;
   auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
 #pragma unroll
-  for (int j = 0; j < D / 32; ++j) {
-    const int load = wave + 4 * j;
+  for (int j = 0; j < D / (8 * GW); ++j) {
+    const int load = wave + GW * j;
+    const WideLane& at = mine[(GW * KEYS_PER_LOAD) % 16 == 0 ? 0 : j % 2];
     const int stretch = (load * KEYS_PER_LOAD) >> 4;       // 16 keys, within one page
     const int piece = load / (D / 64);                      // the values' piece of 8 keys
     const int kh = uniform((b << 6) + stretch * 16);
@@ -770,9 +773,9 @@ __device__ __forceinline__ void wide_fetch(const AttnParams& p, TableWindow& tw,
     const unsigned int k_to = dst + (unsigned int)load * 1024u;
     const unsigned int v_to = dst + (unsigned int)(64 * D * 2) + (unsigned int)load * 1024u;
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 : : "s"(k_to), "v"(mine.k_at), "s"(k_from) : "memory", "m0");
+                 : : "s"(k_to), "v"(at.k_at), "s"(k_from) : "memory", "m0");
     asm volatile("s_mov_b32 m0, %0\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %1, %2"
-                 : : "s"(v_to), "v"(mine.v_at), "s"(v_from) : "memory", "m0");
+                 : : "s"(v_to), "v"(at.v_at), "s"(v_from) : "memory", "m0");
   }
 }
 
@@ -887,26 +890,42 @@ __device__ __forceinline__ void wide_block(const Frag (&qf)[D / 16], f32x16 (&ac
 // bits 3:0 and 15:14; the other counters are left alone).
 #define WIDE_WAIT(loads) (((loads) & 15) | (((loads) >> 4) << 14) | (7 << 4) | (15 << 8))
 
-template <int D, int KG, int NB>
-__global__ __launch_bounds__(256 * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D <= 256 ? 2 : 1))) void attn_wide_kernel(AttnParams p) {
+// GW wavefronts of 32 rows each make a key group, a tile of 32 GW rows: four, or two where
+// tiles of 128 rows would be fewer than fill the chip.
+template <int D, int KG, int NB, int GW = 4>
+__global__ __launch_bounds__(64 * GW * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D <= 256 ? 2 : 1))) void attn_wide_kernel(AttnParams p) {
   constexpr int BUFFER = 2 * 64 * D * 2;                   // bytes of a block's keys and values
-  constexpr int LOADS = D / 16;                            // load instructions per wavefront and block
+  constexpr int LOADS = D / (4 * GW);                      // load instructions per wavefront and block
   constexpr int MERGE = D / 2 + 2;                         // floats a thread hands over
-  static_assert(KG == 1 || (KG - 1) * MERGE * 256 * 4 <= KG * NB * BUFFER, "merge space fits the rings");
+  constexpr int GROUP_THREADS = 64 * GW, ROWS = 32 * GW;
+  static_assert(GW == 2 || GW == 4, "two or four wavefronts a key group");
+  static_assert(KG == 1 || (KG - 1) * MERGE * GROUP_THREADS * 4 <= KG * NB * BUFFER, "merge space fits the rings");
   static_assert((NB - 1) * LOADS < 64, "the loads in flight fit the counter");
   __shared__ __attribute__((aligned(1024))) unsigned char lds[KG * NB * BUFFER];
-  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) & 3;
-  const int kgroup = __builtin_amdgcn_readfirstlane((int)(threadIdx.x >> 8));
+  const int lane = threadIdx.x & 63, wave = (threadIdx.x >> 6) % GW;
+  const int kgroup = __builtin_amdgcn_readfirstlane((int)(threadIdx.x / GROUP_THREADS));
   const int wave_u = __builtin_amdgcn_readfirstlane(wave);
   unsigned char* const ring = lds + kgroup * (NB * BUFFER);
   const unsigned int ring_at = (unsigned int)(uintptr_t)(__attribute__((address_space(3))) void*)ring;
   const int n = lane & 31, hh = lane >> 5;
-  const int tile = p.num_tiles - 1 - (int)blockIdx.x;     // the longest work first
   const int kvh = blockIdx.y;
+  const int G = p.group;
+  const WideLane mine[2] = {wide_lane<D>(1 << p.page_shift, lane, wave_u),
+                            wide_lane<D>(1 << p.page_shift, lane, wave_u + GW)};
+  Frag ones[2];
+  {
+    const uint32_t pair = 0x3F803F80u;                    // two bfloat16 ones
+    const uint32_t even = (lane & 16) ? 0u : pair, odd = (lane & 16) ? pair : 0u;
+    ones[0].u = make_uint4(even, even, even, even);
+    ones[1].u = make_uint4(odd, odd, odd, odd);
+  }
+  auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
+  const float c = p.scale * 1.44269504088896340736f;
+
+  const int tile = p.num_tiles - 1 - (int)blockIdx.x;     // the longest work first
   const int seq = p.tile_seq[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
   const int pos0 = p.kv_len[seq] - q_len;
-  const int G = p.group;
   const int rows_total = q_len * G;
   const int wg_row0 = p.tile_row0[tile];
   const int row0 = wg_row0 + wave * 32;
@@ -919,7 +938,7 @@ __global__ __launch_bounds__(256 * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D
   const int pos = pos0 + tok;
   const int lo = p.window > 0 ? max(0, pos - p.window + 1) : 0;
 
-  const int wg_last = min(wg_row0 + 127, rows_total - 1);
+  const int wg_last = min(wg_row0 + ROWS - 1, rows_total - 1);
   const int wg_kmax = pos0 + wg_last / G;
   const int wg_kmin = p.window > 0 ? max(0, pos0 + wg_row0 / G - p.window + 1) : 0;
   const int b0 = wg_kmin >> 6, b1 = (wg_kmax >> 6) + 1;
@@ -927,12 +946,11 @@ __global__ __launch_bounds__(256 * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D
   const int iterations = __builtin_amdgcn_readfirstlane((b1 - b0 + KG - 1) / KG);   // the same for every group
 
   // The ring starts to fill before anything else is asked of memory.
-  const WideLane mine = wide_lane<D>(1 << p.page_shift, lane, wave_u);
   TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
 #pragma unroll
   for (int i = 0; i < NB - 1; ++i)
-    wide_fetch<D>(p, tw, first + i * KG, b1, wg_kmin, wg_kmax, kvh, lane, wave_u,
-                  ring_at + (unsigned int)(i * BUFFER), mine);
+    wide_fetch<D, GW>(p, tw, first + i * KG, b1, wg_kmin, wg_kmax, kvh, lane, wave_u,
+                      ring_at + (unsigned int)(i * BUFFER), mine);
 
   Frag qf[D / 16];
   {
@@ -950,21 +968,12 @@ __global__ __launch_bounds__(256 * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D
   // Sums of weights per row, kept by the matrix cores (see wide_block): rowsum[h][.] on lane l
   // is the sum of row 16 h + l % 16, both halves' keys included.
   f32x4 rowsum[2] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
-  Frag ones[2];
-  {
-    const uint32_t pair = 0x3F803F80u;                    // two bfloat16 ones
-    const uint32_t even = (lane & 16) ? 0u : pair, odd = (lane & 16) ? pair : 0u;
-    ones[0].u = make_uint4(even, even, even, even);
-    ones[1].u = make_uint4(odd, odd, odd, odd);
-  }
 
-  auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
   const int last_flat = min(row0 + 31, rows_total - 1);
   const int kmax = uniform(wave_has_rows ? pos0 + last_flat / G : -1);
   const int kmin = uniform(p.window > 0 ? max(0, pos0 + row0 / G - p.window + 1) : 0);
   const int see_upto = uniform(pos0 + row0 / G);       // every valid row of the wavefront sees up to here
   const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
-  const float c = p.scale * 1.44269504088896340736f;
   // the queries were asked for after the ring's first loads: all of them have to be there
   // before the counting below starts
   __builtin_amdgcn_s_waitcnt(WIDE_WAIT(0));
@@ -981,8 +990,8 @@ __global__ __launch_bounds__(256 * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D
     const int b = first + i * KG;                                                                \
     __builtin_amdgcn_s_waitcnt(WIDE_WAIT((NB - 2) * LOADS));                                     \
     __syncthreads();                                                                             \
-    wide_fetch<D>(p, tw, b + (NB - 1) * KG, b1, wg_kmin, wg_kmax, kvh, lane, wave_u,             \
-                  ring_at + (unsigned int)(((i + NB - 1) % NB) * BUFFER), mine);                 \
+    wide_fetch<D, GW>(p, tw, b + (NB - 1) * KG, b1, wg_kmin, wg_kmax, kvh, lane, wave_u,         \
+                      ring_at + (unsigned int)(((i + NB - 1) % NB) * BUFFER), mine);             \
     const uint4* lds_k = (const uint4*)(ring + (i % NB) * BUFFER);                               \
     const uint2* lds_v = (const uint2*)(ring + (i % NB) * BUFFER + 64 * D * 2);                  \
     const int key0 = b << 6;                                                                     \
@@ -1016,47 +1025,49 @@ __global__ __launch_bounds__(256 * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB * D
     // wavefront-in-group holds the same rows and dims in every group.
     __syncthreads();                                    // the rings are free now
     float* const merge = (float*)lds;
-    const int slot = threadIdx.x & 255;
+    const int slot = threadIdx.x % GROUP_THREADS;
     if (kgroup > 0) {
-      float* mine = merge + (size_t)(kgroup - 1) * MERGE * 256 + slot;
+      float* mine_out = merge + (size_t)(kgroup - 1) * MERGE * GROUP_THREADS + slot;
       int e = 0;
-      mine[256 * e++] = m;
-      mine[256 * e++] = lsum;
+      mine_out[GROUP_THREADS * e++] = m;
+      mine_out[GROUP_THREADS * e++] = lsum;
 #pragma unroll
       for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) mine[256 * e++] = acc[db][i];
+        for (int i = 0; i < 16; ++i) mine_out[GROUP_THREADS * e++] = acc[db][i];
     }
     __syncthreads();
-    if (kgroup > 0) return;
+    if (kgroup == 0) {
 #pragma unroll
-    for (int g = 1; g < KG; ++g) {
-      const float* theirs = merge + (size_t)(g - 1) * MERGE * 256 + slot;
-      int e = 0;
-      const float m_g = theirs[256 * e++], l_g = theirs[256 * e++];
-      const float m_new = fmaxf(m, m_g);
-      const float c_own = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
-      const float c_g = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_g - m_new);
-      m = m_new;
-      lsum = lsum * c_own + l_g * c_g;
+      for (int g = 1; g < KG; ++g) {
+        const float* theirs = merge + (size_t)(g - 1) * MERGE * GROUP_THREADS + slot;
+        int e = 0;
+        const float m_g = theirs[GROUP_THREADS * e++], l_g = theirs[GROUP_THREADS * e++];
+        const float m_new = fmaxf(m, m_g);
+        const float c_own = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m - m_new);
+        const float c_g = m_new == -INFINITY ? 0.f : __builtin_amdgcn_exp2f(m_g - m_new);
+        m = m_new;
+        lsum = lsum * c_own + l_g * c_g;
 #pragma unroll
-      for (int db = 0; db < D / 32; ++db)
+        for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-        for (int i = 0; i < 16; ++i) acc[db][i] = acc[db][i] * c_own + theirs[256 * e++] * c_g;
+          for (int i = 0; i < 16; ++i) acc[db][i] = acc[db][i] * c_own + theirs[GROUP_THREADS * e++] * c_g;
+      }
     }
   }
 
-  if (!row_ok) return;
-  const float inv = 1.f / lsum;
-  // acc[db][i] is O^T[dim = db * 32 + 8 (i / 4) + 4 hh + i % 4][row n].
-  bf16_t* dst = p.out + (size_t)(q0 + tok) * p.out_stride + head * D + 4 * hh;
+  if (row_ok && kgroup == 0) {
+    const float inv = 1.f / lsum;
+    // acc[db][i] is O^T[dim = db * 32 + 8 (i / 4) + 4 hh + i % 4][row n].
+    bf16_t* dst = p.out + (size_t)(q0 + tok) * p.out_stride + head * D + 4 * hh;
 #pragma unroll
-  for (int db = 0; db < D / 32; ++db)
+    for (int db = 0; db < D / 32; ++db)
 #pragma unroll
-    for (int q4 = 0; q4 < 4; ++q4)
-      *(uint2*)(dst + db * 32 + 8 * q4) =
-          make_uint2(pack_bf16x2(acc[db][4 * q4] * inv, acc[db][4 * q4 + 1] * inv),
-                     pack_bf16x2(acc[db][4 * q4 + 2] * inv, acc[db][4 * q4 + 3] * inv));
+      for (int q4 = 0; q4 < 4; ++q4)
+        *(uint2*)(dst + db * 32 + 8 * q4) =
+            make_uint2(pack_bf16x2(acc[db][4 * q4] * inv, acc[db][4 * q4 + 1] * inv),
+                       pack_bf16x2(acc[db][4 * q4 + 2] * inv, acc[db][4 * q4 + 3] * inv));
+  }
 }
 
 // Merge the key splits of one (tile, kv head, row) per workgroup: the maximum of the running
@@ -1177,14 +1188,23 @@ static void launch_staged(const AttnParams& p, int rows_per_tile, int key_groups
 // 128-wide heads two workgroups with two buffers (8,192 tokens, 28 heads: 752 us against 1256
 // with three buffers and one workgroup).  Key groups: as many as keep three (64) or two (128)
 // wavefronts a SIMD in one workgroup, for launches of fewer workgroups than fill the chip.
+// Tiles of 64 rows (64-wide heads): four key groups with two buffers each (128 KB, eight
+// wavefronts, one workgroup a compute unit) or two (64 KB, two workgroups a unit).
 template <int D>
-static void launch_wide(const AttnParams& p, int key_groups, hipStream_t stream) {
+static void launch_wide(const AttnParams& p, int staged, hipStream_t stream) {
   const dim3 grid(p.num_tiles, p.n_kv);
+  const int chains = staged / 8;
   if constexpr (D == 64) {
-    if (key_groups == 3) attn_wide_kernel<D, 3, 3><<<grid, 768, 0, stream>>>(p);
-    else attn_wide_kernel<D, 1, 3><<<grid, 256, 0, stream>>>(p);
+    if (staged % 8) {   // tiles of 64 rows, two wavefronts a key group
+      if (chains == 4) attn_wide_kernel<D, 4, 2, 2><<<grid, 512, 0, stream>>>(p);
+      else attn_wide_kernel<D, 2, 2, 2><<<grid, 256, 0, stream>>>(p);
+    } else if (chains == 3) {
+      attn_wide_kernel<D, 3, 3><<<grid, 768, 0, stream>>>(p);
+    } else {
+      attn_wide_kernel<D, 1, 3><<<grid, 256, 0, stream>>>(p);
+    }
   } else {
-    if (key_groups == 2) attn_wide_kernel<D, 2, 2><<<grid, 512, 0, stream>>>(p);
+    if (chains == 2) attn_wide_kernel<D, 2, 2><<<grid, 512, 0, stream>>>(p);
     else attn_wide_kernel<D, 1, 2><<<grid, 256, 0, stream>>>(p);
   }
 }
@@ -1252,6 +1272,10 @@ extern "C" int mk_attention_mfma_wide(int head_dim) {
   return head_dim == 64 ? 0b101 : (head_dim == 128 ? 0b011 : 0);
 }
 
+// The same for its workgroups of 64 rows, two wavefronts a key group (`staged` = 8 times the
+// number of chains, plus 4; tile list in steps of 64 rows): 64-wide heads in two or four chains.
+extern "C" int mk_attention_mfma_wide_half(int head_dim) { return head_dim == 64 ? 0b1010 : 0; }
+
 // From how many workgroups of 128 rows on the kernel of 32-row wavefronts measured faster
 // than the 16-row kernels, for the instantiation of this head size with `chains` key groups
 // (0: no such instantiation).  The numbers belong to the instantiations, which is why they
@@ -1266,6 +1290,31 @@ extern "C" int mk_attention_mfma_wide(int head_dim) {
 extern "C" int mk_attention_mfma_wide_from(int head_dim, int chains) {
   if (head_dim == 64) return chains == 1 ? 512 : (chains == 3 ? 192 : 0);
   if (head_dim == 128) return chains == 1 ? 256 : (chains == 2 ? 128 : 0);
+  return 0;
+}
+
+// Whether the 64-row instantiation with `chains` key groups measured faster than whatever
+// else takes a step of `workgroups` tiles of 64 rows (kv heads counted), whose longest
+// sequence is `blocks` blocks of 64 keys, with `n_kv` key/value heads.  Measured, us against
+// the best of the other kernels, 64-wide heads:
+//   four chains, 112 to 256 workgroups, chains of 12 blocks and more: 512 tokens over 3,584,
+//   14 heads in 2 groups (112): 35.1 against 40.7, 32 in 8 (256): 39.8 against 47.5; 1,024
+//   tokens, 14 in 2 (224): 13.9 against 14.8; 256 over 1,792, 28 in 4 (112): 20.3 against 22.2
+//   (128 over 4,000, 28 workgroups: 35 against 19).  With one or two key/value heads up to
+//   448: 2,048 tokens, 14 in 2: 27.7 against 29.2; two of 1,024 over 1,024: 37.3 against 41.4.
+//   two chains, 257 to 512 workgroups, four key/value heads or more, or chains of 8 blocks at
+//   most: 1,024 tokens, 28 in 4 (448): 19.6 against 22.9, 32 in 8 (512): 21.3 against 27.1;
+//   2,048 tokens, 16 in 8 (512): 37.3 against 45.0; four prompts of 512, 14 in 2 (448): 13.6
+//   against 18.0 (one of 2,048, 14 in 2: 33.2 against 29.2; 3,072 tokens, 28 in 4, 1,344
+//   workgroups: 86 against 82).
+extern "C" int mk_attention_mfma_wide_half_wins(int head_dim, int chains, int workgroups,
+                                                int blocks, int n_kv) {
+  if (head_dim != 64) return 0;
+  if (chains == 4) {
+    return (workgroups >= 112 && workgroups <= 256 && blocks >= 12) ||
+           (n_kv <= 2 && workgroups > 256 && workgroups <= 448 && blocks > 8);
+  }
+  if (chains == 2) return workgroups > 256 && workgroups <= 512 && (n_kv >= 4 || blocks <= 8);
   return 0;
 }
 
@@ -1297,14 +1346,17 @@ extern "C" int mk_attention_mfma_check(int q_stride, int out_stride, int num_til
   MK_REQUIRE(rows_per_tile <= mk_attention_mfma_max_rows(d),
              "attention: %d rows per tile are too many for head size %d", rows_per_tile, d);
   MK_REQUIRE(split_blocks >= 0, "attention: negative split size");
-  MK_REQUIRE(staged == 0 || staged == 1 || staged == 2 || staged == 4 || staged == 8 ||
-                 staged == 16 || staged == 24,
-             "attention: %d key groups (0, 1, 2 or 4; 8, 16 and 24 for the kernel of 32-row "
-             "wavefronts with one, two and three)", staged);
+  const int wide_chains = staged >= 8 ? staged / 8 : 0;
+  MK_REQUIRE(staged == 0 || staged == 1 || staged == 2 || staged == 4 ||
+                 (staged >= 8 && wide_chains <= 4 && (staged % 8 == 0 || staged % 8 == 4)),
+             "attention: %d key groups (0, 1, 2 or 4; 8 times one to four for the kernel of "
+             "32-row wavefronts, plus 4 for its tiles of 64 rows)", staged);
   MK_REQUIRE(staged < 8 || (num_splits == 1 && rows_per_tile == 32 &&
-                            ((mk_attention_mfma_wide(d) >> (staged / 8 - 1)) & 1)),
+                            (((staged % 8 ? mk_attention_mfma_wide_half(d) : mk_attention_mfma_wide(d)) >>
+                              (wide_chains - 1)) & 1)),
              "attention: the kernel of 32-row wavefronts takes unsplit keys, 32 rows per "
-             "wavefront and head sizes 64 (one or three key groups) and 128 (one or two)");
+             "wavefront and head sizes 64 (one or three key groups, two or four with tiles of "
+             "64 rows) and 128 (one or two)");
   MK_REQUIRE(!staged || staged >= 8 ||
                  (num_splits == 1 && staged <= mk_attention_mfma_staged(d, rows_per_tile)),
              "attention: staging in LDS takes unsplit keys, head sizes 64 and 128 and 16 or 32 "
@@ -1353,7 +1405,7 @@ static int attention_mfma(const void* q, int q_stride, void* out, int out_stride
   // of 8 key/value heads: 10 us unfolded, 16 folded; 64 tokens: 194 and 186)
   p.kv_fold = num_tiles < 32 ? 1 : (n_kv % 4 == 0 ? 4 : (n_kv % 2 == 0 ? 2 : 1));
   if (staged >= 8) {
-    if (d == 64) launch_wide<64>(p, staged / 8, stream); else launch_wide<128>(p, staged / 8, stream);
+    if (d == 64) launch_wide<64>(p, staged, stream); else launch_wide<128>(p, staged, stream);
     MK_LAUNCH_CHECK("attention_mfma");
     return 0;
   }

@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 16
+#define MK_ABI_VERSION 17
 
 #ifdef __cplusplus
 extern "C" {
@@ -174,6 +174,12 @@ int mk_attention_mfma_wide(int head_dim);
 // From how many workgroups of 128 rows on the kernel of 32-row wavefronts with `chains` key
 // groups is the faster one at this head size (0: no such instantiation).
 int mk_attention_mfma_wide_from(int head_dim, int chains);
+// The same kernel on tiles of 64 rows (two wavefronts a key group; staged = 8 * chains + 4):
+// which numbers of chains exist at this head size (bit n - 1), and whether the instantiation
+// with `chains` of them is the faster one for a step of `workgroups` such tiles (key/value
+// heads counted) whose longest sequence is `blocks` blocks of 64 keys.
+int mk_attention_mfma_wide_half(int head_dim);
+int mk_attention_mfma_wide_half_wins(int head_dim, int chains, int workgroups, int blocks, int n_kv);
 int mk_attention_mfma_check(int q_stride, int out_stride, int num_tiles, int page_size, int n_q,
                             int n_kv, int d, float scale, int window, int rows_per_tile,
                             int staged, int num_splits, int split_blocks, int has_workspace);

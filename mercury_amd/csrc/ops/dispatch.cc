@@ -154,6 +154,18 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
       // of 64 is a tie (30.6 against 30.2 us) and stays with the 16-row kernel
       staged = 8 * most;
     }
+    // its tiles of 64 rows, for steps of fewer workgroups than fill the chip twice
+    if (staged < 0 && (long long)max_q_len * group >= 64) {
+      const int half = t.mk_attention_mfma_wide_half(head_dim);
+      const long long tiles = (total_rows / 64) * n_kv;
+      const int blocks64 = (span + 63) / 64;
+      for (int n = 4; n >= 1 && staged < 0 && tiles < (1 << 20); --n) {
+        if (((half >> (n - 1)) & 1) &&
+            t.mk_attention_mfma_wide_half_wins(head_dim, n, (int)tiles, blocks64, n_kv)) {
+          staged = 8 * n + 4;
+        }
+      }
+    }
     if (staged >= 8) rows = 32;
   }
   if (staged < 0) {
@@ -166,7 +178,7 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
     if (yes) rows = 16;
   }
   plan.rows = rows;
-  plan.tile_rows = staged ? rows * 4 : rows;
+  plan.tile_rows = staged >= 8 && staged % 8 ? rows * 2 : (staged ? rows * 4 : rows);
   plan.num_tiles = count_tiles(counts, group, plan.tile_rows);
   if (staged == -1) {
     // A workgroup's chain of key blocks is cut into 2 or 4 chains side by side while that

@@ -55,10 +55,11 @@ struct AttentionPlan {
   bool mfma = false;
   int rows = 16;          // rows per wavefront tile
   int staged = 0;         // 0, or how many groups of four wavefronts share a workgroup's keys;
-                          // 8, 16, 24: the kernel of 32-row wavefronts with one, two, three groups
+                          // 8, 16, 24: the kernel of 32-row wavefronts with one, two, three groups;
+                          // 20, 36: the same on tiles of 64 rows with two and four groups
   int splits = 1;
   int split_blocks = 0;
-  int tile_rows = 16;     // rows per entry of the tile list: rows, or 4 * rows when staged
+  int tile_rows = 16;     // rows per entry of the tile list: rows, 4 * rows when staged, 2 * rows for 20 and 36
   int num_tiles = 0;
 };
 

@@ -784,13 +784,14 @@ def test_attention_through_lds_for_prompts(tile_rows, d, n_q, n_kv, page, groups
 
 
 @pytest.mark.parametrize("d,n_q,n_kv,page,groups", [
-    (64, 14, 2, 16, 8), (128, 6, 2, 16, 8), (128, 6, 2, 64, 16), (64, 6, 2, 32, 24)])
+    (64, 14, 2, 16, 8), (128, 6, 2, 16, 8), (128, 6, 2, 64, 16), (64, 6, 2, 32, 24),
+    (64, 14, 2, 16, 36), (64, 6, 2, 32, 20)])
 @pytest.mark.parametrize("window", [None, 200, 700])
 def test_attention_of_32_row_wavefronts_over_long_prompts(d, n_q, n_kv, page, groups, window):
     """The prompt kernel of 32-row wavefronts walks its key blocks in three stretches: blocks
     that a window's far edge cuts, blocks that every row sees whole, blocks that the diagonal
     cuts.  Long sequences give each stretch several blocks, with one and with two chains of
-    blocks side by side; in each sequence one far key carries a score that stands out for the
+    blocks side by side, in tiles of 128 rows and (groups 20 and 36) of 64; in each sequence one far key carries a score that stands out for the
     rows that may see it, so a block dropped or taken twice shows."""
     lens, q_lens = [1500, 700, 260], [1500, 300, 129]
     qs, ks, vs = [], [], []
@@ -825,7 +826,7 @@ def test_attention_through_lds_is_refused_where_it_does_not_fit():
         run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
                       kernel="mfma", staged=True)
     # two chains of key blocks exist for 128-wide heads only, three for 64-wide only
-    for d, groups in ((64, 16), (128, 24)):
+    for d, groups in ((64, 16), (128, 24), (128, 20), (64, 28), (64, 12)):
         q = rounded(rnd(40, 2, d, seed=1), torch.bfloat16)
         with pytest.raises((KernelArgumentError, RuntimeError)):
             run_attention([q], [q], [q], torch.bfloat16, [[0, 1, 2]], 16, 4, [40], [40], 0.1,
