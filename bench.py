@@ -224,7 +224,7 @@ class Bench:
             out["gemm_flops"] = round(2.0 * n ** 3 / gemm_s, -9)
         return out
 
-    def prefill(self, tokens: int, repeats: int = 5) -> dict:
+    def prefill(self, tokens: int, repeats: int = 9) -> dict:
         from mercury_amd import SamplingParams
 
         times = []

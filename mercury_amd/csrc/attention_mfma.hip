@@ -908,7 +908,6 @@ __global__ __launch_bounds__(64 * GW * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB
   unsigned char* const ring = lds + kgroup * (NB * BUFFER);
   const unsigned int ring_at = (unsigned int)(uintptr_t)(__attribute__((address_space(3))) void*)ring;
   const int n = lane & 31, hh = lane >> 5;
-  const int kvh = blockIdx.y;
   const int G = p.group;
   const WideLane mine[2] = {wide_lane<D>(1 << p.page_shift, lane, wave_u),
                             wide_lane<D>(1 << p.page_shift, lane, wave_u + GW)};
@@ -922,7 +921,27 @@ __global__ __launch_bounds__(64 * GW * KG, KG > 1 ? 1 : (NB * D <= 192 ? 3 : (NB
   auto uniform = [](int v) { return __builtin_amdgcn_readfirstlane(v); };
   const float c = p.scale * 1.44269504088896340736f;
 
-  const int tile = p.num_tiles - 1 - (int)blockIdx.x;     // the longest work first
+  // The order of work.  Workgroups are handed out in the order of their index, to the compute
+  // units in turn, and stay until their chain of key blocks is done; the length of a chain
+  // grows with the tile's number within its sequence.  So the index counts the (tile, kv
+  // head) pairs from the longest down, kv heads side by side, and of the stretches of 256
+  // that are resident from the start (as many as a unit holds workgroups) every second one
+  // runs backwards: the unit that took the longest of one stretch takes the shortest of the
+  // next, and what is resident on a unit adds up to about the same everywhere (8,192 tokens
+  // of 14 heads of 64: 211 us against 227; 16,384: 641 against 683; 28 heads of 128: 610
+  // against 634).  What follows the residents goes to whichever unit is free first, the
+  // longest first.
+  constexpr int RESIDENT = KG > 1 ? (GW == 2 && KG == 2 ? 2 : 1) : (NB * D <= 192 ? 3 : (NB * D <= 256 ? 2 : 1));
+  int tile, kvh_x;
+  {
+    const int total = gridDim.x * gridDim.y, id = blockIdx.y * gridDim.x + blockIdx.x;
+    const int stretch = id / 256, size = min(256, total - stretch * 256), at = id - stretch * 256;
+    const bool backwards = (stretch & 1) && stretch < RESIDENT;
+    const int rank = stretch * 256 + (backwards ? size - 1 - at : at);
+    kvh_x = rank % (int)gridDim.y;
+    tile = p.num_tiles - 1 - rank / (int)gridDim.y;
+  }
+  const int kvh = kvh_x;
   const int seq = p.tile_seq[tile];
   const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
   const int pos0 = p.kv_len[seq] - q_len;
@@ -1276,45 +1295,42 @@ extern "C" int mk_attention_mfma_wide(int head_dim) {
 // number of chains, plus 4; tile list in steps of 64 rows): 64-wide heads in two or four chains.
 extern "C" int mk_attention_mfma_wide_half(int head_dim) { return head_dim == 64 ? 0b1010 : 0; }
 
-// From how many workgroups of 128 rows on the kernel of 32-row wavefronts measured faster
-// than the 16-row kernels, for the instantiation of this head size with `chains` key groups
-// (0: no such instantiation).  The numbers belong to the instantiations, which is why they
-// stand here and not with the planner:
-//   64-wide heads, one chain: 14 heads in 2 groups at 2,048 tokens, 224 workgroups, 34 us
-//   against 30; 4 x 2,048, 896: 73 against 90; 8,192: 202 against 288.  Three chains: 2,048
-//   tokens, 224 workgroups, 30.6 us against 30.2; 4,096, 448: 64 against 89; 2,048 over 6,144:
-//   102 against 139; 512 over 1,536, 56: 28 against 22.
-//   128-wide heads, one chain: 28 heads in 4 groups at 2,048 tokens, 448 workgroups: 85
-//   against 96; 8,192: 752 against 969.  Two chains: 512 tokens over 1,536, 112: 54 against
-//   41; 40 heads in 8 groups there, 160: 54 against 67.
-extern "C" int mk_attention_mfma_wide_from(int head_dim, int chains) {
-  if (head_dim == 64) return chains == 1 ? 512 : (chains == 3 ? 192 : 0);
-  if (head_dim == 128) return chains == 1 ? 256 : (chains == 2 ? 128 : 0);
-  return 0;
-}
-
-// Whether the 64-row instantiation with `chains` key groups measured faster than whatever
-// else takes a step of `workgroups` tiles of 64 rows (kv heads counted), whose longest
-// sequence is `blocks` blocks of 64 keys, with `n_kv` key/value heads.  Measured, us against
-// the best of the other kernels, 64-wide heads:
-//   four chains, 112 to 256 workgroups, chains of 12 blocks and more: 512 tokens over 3,584,
-//   14 heads in 2 groups (112): 35.1 against 40.7, 32 in 8 (256): 39.8 against 47.5; 1,024
-//   tokens, 14 in 2 (224): 13.9 against 14.8; 256 over 1,792, 28 in 4 (112): 20.3 against 22.2
-//   (128 over 4,000, 28 workgroups: 35 against 19).  With one or two key/value heads up to
-//   448: 2,048 tokens, 14 in 2: 27.7 against 29.2; two of 1,024 over 1,024: 37.3 against 41.4.
-//   two chains, 257 to 512 workgroups, four key/value heads or more, or chains of 8 blocks at
-//   most: 1,024 tokens, 28 in 4 (448): 19.6 against 22.9, 32 in 8 (512): 21.3 against 27.1;
-//   2,048 tokens, 16 in 8 (512): 37.3 against 45.0; four prompts of 512, 14 in 2 (448): 13.6
-//   against 18.0 (one of 2,048, 14 in 2: 33.2 against 29.2; 3,072 tokens, 28 in 4, 1,344
-//   workgroups: 86 against 82).
-extern "C" int mk_attention_mfma_wide_half_wins(int head_dim, int chains, int workgroups,
-                                                int blocks, int n_kv) {
-  if (head_dim != 64) return 0;
-  if (chains == 4) {
-    return (workgroups >= 112 && workgroups <= 256 && blocks >= 12) ||
-           (n_kv <= 2 && workgroups > 256 && workgroups <= 448 && blocks > 8);
+// Which instantiation of the kernel of 32-row wavefronts, as its `staged` code (0: none, the
+// 16-row kernels are the faster ones), for a step of `wg128` workgroups of 128 rows or
+// `wg64` of 64 (key/value heads counted) whose longest sequence is `blocks32` blocks of 32
+// keys; `fresh`: most of the longest sequence's keys are this step's own (a prompt from its
+// start rather than a portion over a long prefix).  The numbers belong to the instantiations,
+// which is why they stand here and not with the planner.  Measured, us, against the best
+// of the rest (each line: heads in groups, tokens (over a prefix), then the candidates):
+//  64-wide heads (codes 8: one chain of key blocks, 24: three; tiles of 64 rows 36: four, 20: two)
+//   14 in 2, 1,024: 16-row 15.7, 8 23.2, 24 19.5, 36 15.2    2,048: 29.5, 39.7, 29.0, 36 28.0
+//   14 in 2, 3,072: 16-row 55.9, 8 57.2, 24 39.7, 36 50.9    6,144: 151, 8 117, 24 115
+//   14 in 2, 512 over 3,584: 16-row 40.7, 24 48.2, 36 36.4   two of 1,024 over 1,024: 42.5, 8 40.3, 24 30.2, 36 35.8
+//   28 in 4, 1,024: 16-row 23.8, 8 23.3, 24 19.8, 20 19.0    1,536: 36.5, 8 32.1, 24 25.9, 20 27.1
+//   28 in 4, 2,048: 8 41.0, 24 35.8, 20 40.9    3,072: 8 62.6, 24 68.7    four of 512: 8 17.2, 24 24.4, 20 22.7
+//   16 in 8, 1,536: 16-row 32.6, 24 24.1, 36 21.9    4,096: 8 76.0, 24 60.4    four of 512: 8 15.4, 20 14.0
+//   32 in 8, 768: 16-row 20.5, 8 19.1, 20 15.8    2,048: 8 42.0, 24 38.7    3,072: 8 65.7, 24 74.8
+//  128-wide heads (codes 8: one chain, 16: two)
+//   28 in 4, 512: 16-row 15.9, 16 19.8    1,024: 37.5, 8 36.6, 16 30.6    2,048: 8 67.9, 16 58.3    3,072: 8 103, 16 116
+//   28 in 4, 1,024 over 3,072: 16-row 137, 8 121, 16 91.7    four of 512: 8 28.0, 16 35.2    two of 1,024 over 1,024: 8 77.8, 16 81.5
+//   40 in 8, 768: 16-row 30.2, 8 29.4, 16 25.9    1,536: 8 53.4, 16 49.8    2,048: 8 73.2, 16 84.9
+//   16 in 8, 1,024: 16-row 25.3, 16 29.3    2,048: 8 62.8, 16 49.9    4,096: 8 127, 16 105    6,144: 8 207, 16 228
+extern "C" int mk_attention_mfma_wide_choice(int head_dim, int wg128, int wg64, int blocks32,
+                                             int fresh) {
+  if (head_dim == 64) {
+    if (wg128 >= 192 && wg128 <= 512 && blocks32 >= 48 && !(fresh && wg64 <= 512)) return 24;
+    if (wg128 >= 512 || (wg128 >= 384 && blocks32 < 48)) return 8;
+    if (wg64 >= 112 && wg64 <= 256 && blocks32 >= 24) return 36;
+    if (wg64 > 256 && wg64 <= 512) return blocks32 >= 48 ? 36 : 20;
+    return 0;
   }
-  if (chains == 2) return workgroups > 256 && workgroups <= 512 && (n_kv >= 4 || blocks <= 8);
+  if (head_dim == 128) {
+    if ((wg128 >= 160 && wg128 <= 384 && blocks32 >= 16) ||
+        (wg128 > 384 && wg128 <= 512 && blocks32 >= 24 && fresh)) {
+      return 16;
+    }
+    return wg128 >= 256 ? 8 : 0;
+  }
   return 0;
 }
 

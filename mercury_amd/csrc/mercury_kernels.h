@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 17
+#define MK_ABI_VERSION 18
 
 #ifdef __cplusplus
 extern "C" {
@@ -171,15 +171,14 @@ int mk_attention_mfma_max_rows(int head_dim);
 // without the launch (0: it would take them; else mk_last_error() says why not).
 int mk_attention_mfma_staged(int head_dim, int rows_per_tile);
 int mk_attention_mfma_wide(int head_dim);
-// From how many workgroups of 128 rows on the kernel of 32-row wavefronts with `chains` key
-// groups is the faster one at this head size (0: no such instantiation).
-int mk_attention_mfma_wide_from(int head_dim, int chains);
 // The same kernel on tiles of 64 rows (two wavefronts a key group; staged = 8 * chains + 4):
-// which numbers of chains exist at this head size (bit n - 1), and whether the instantiation
-// with `chains` of them is the faster one for a step of `workgroups` such tiles (key/value
-// heads counted) whose longest sequence is `blocks` blocks of 64 keys.
+// which numbers of chains exist at this head size (bit n - 1).
 int mk_attention_mfma_wide_half(int head_dim);
-int mk_attention_mfma_wide_half_wins(int head_dim, int chains, int workgroups, int blocks, int n_kv);
+// Which of these instantiations, as its `staged` code, measured fastest for a step of `wg128`
+// workgroups of 128 rows or `wg64` of 64 (key/value heads counted) whose longest sequence is
+// `blocks32` blocks of 32 keys, most of them this step's own or not (`fresh`); 0: none, the
+// 16-row kernels are faster.
+int mk_attention_mfma_wide_choice(int head_dim, int wg128, int wg64, int blocks32, int fresh);
 int mk_attention_mfma_check(int q_stride, int out_stride, int num_tiles, int page_size, int n_q,
                             int n_kv, int d, float scale, int window, int rows_per_tile,
                             int staged, int num_splits, int split_blocks, int has_workspace);

@@ -134,36 +134,19 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   int staged = staged_in;
   const bool split_forced = splits_in > 0;
   if (staged >= 8) rows = 32;
-  // Long prompts of a head size it takes go to the kernel of 32-row wavefronts and 64-key
-  // blocks (`staged` 8, or 16 with the keys in two chains): workgroups of 128 rows of one
-  // sequence, chosen from the number of such workgroups at which it measured faster.
-  if (staged < 0 && !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 128) {
-    const int chains = t.mk_attention_mfma_wide(head_dim);   // bit n - 1: n chains exist
-    const long long workgroups = (total_rows / 128) * n_kv;
-    const int most = (chains & 4) ? 3 : ((chains & 2) ? 2 : 1);
-    // the counts from which each instantiation measured faster are the kernel library's
-    const long long full = t.mk_attention_mfma_wide_from(head_dim, 1);
-    const long long few = most > 1 ? t.mk_attention_mfma_wide_from(head_dim, most) : 0;
-    if ((chains & 1) && (workgroups >= full ||
-                         (most > 2 && workgroups >= 3 * full / 4 && blocks < 32 * most))) {
-      // (three quarters of that many with chains too short to cut: 28 heads of 64, 2,048
-      // tokens, 448 workgroups: 44 us against 47 in the 16-row kernel)
-      staged = 8;
-    } else if (most > 1 && workgroups >= few && blocks >= 32 * most) {
-      // chains of at least 16 blocks of 64 keys each: a single 2,048-token prompt of 14 heads
-      // of 64 is a tie (30.6 against 30.2 us) and stays with the 16-row kernel
-      staged = 8 * most;
-    }
-    // its tiles of 64 rows, for steps of fewer workgroups than fill the chip twice
-    if (staged < 0 && (long long)max_q_len * group >= 64) {
-      const int half = t.mk_attention_mfma_wide_half(head_dim);
-      const long long tiles = (total_rows / 64) * n_kv;
-      const int blocks64 = (span + 63) / 64;
-      for (int n = 4; n >= 1 && staged < 0 && tiles < (1 << 20); --n) {
-        if (((half >> (n - 1)) & 1) &&
-            t.mk_attention_mfma_wide_half_wins(head_dim, n, (int)tiles, blocks64, n_kv)) {
-          staged = 8 * n + 4;
-        }
+  // Prompts of a head size it takes go to the kernel of 32-row wavefronts and 64-key blocks,
+  // in workgroups of 128 rows of one sequence or of 64, the keys in one to four chains:
+  // whichever instantiation the kernel library measured fastest for a step of this many
+  // workgroups and blocks (`staged` 8, 16, 24; 20, 36 for the tiles of 64 rows).
+  if (staged < 0 && !split_forced && tile_rows <= 0 && (long long)max_q_len * group >= 64) {
+    const long long wg128 = (total_rows / 128) * n_kv, wg64 = (total_rows / 64) * n_kv;
+    if (wg64 < (1 << 24)) {
+      const int code = t.mk_attention_mfma_wide_choice(head_dim, (int)wg128, (int)wg64, blocks,
+                                                       2 * max_q_len > max_kv_len);
+      const bool half = code % 8 != 0;
+      const int exists = half ? t.mk_attention_mfma_wide_half(head_dim) : t.mk_attention_mfma_wide(head_dim);
+      if (code >= 8 && ((exists >> (code / 8 - 1)) & 1) && (half || (long long)max_q_len * group >= 128)) {
+        staged = code;
       }
     }
     if (staged >= 8) rows = 32;

@@ -44,7 +44,7 @@ def random_step(rng):
     if kind < 0.35:          # decoding
         counts = [1] * rng.choice((1, 2, 7, 8, 33, 64, 200, 256))
     elif kind < 0.6:         # one prompt, short to very long
-        counts = [rng.choice((2, 17, 64, 100, 512, 2048, 4700, 8192, 30000))]
+        counts = [rng.choice((2, 17, 64, 100, 200, 300, 512, 2048, 4700, 8192, 30000))]
     else:                    # portions beside decoded tokens
         counts = [rng.choice((1, 1, 1, 2, 16, 100, 512, 2048)) for _ in range(rng.randint(1, 40))]
     longest = max(counts) + rng.choice((0, 0, 5, 300, 4000, 30000))
@@ -171,15 +171,19 @@ def test_pinned_choices_of_the_benchmark_shapes(core):
     for heads, kv_heads, size in ((14, 2, 64), (28, 4, 128), (40, 8, 128)):
         p = plan(core, heads, kv_heads, size, [8192], 8192)
         assert (p["staged"], p["rows"]) == (8, 32)
-    # prompts of fewer workgroups than fill the chip twice: the same kernel on tiles of 64 rows,
-    # in four chains of key blocks (0.5B, 2,048 tokens: 27.7 us against 29.2; 512 tokens over
-    # 3,584: 35.1 against 40.7) or in two (1,024 tokens of 28 heads in 4 groups: 19.6 against
-    # 22.9); with 128-wide heads it does not exist
+    # shorter prompts: the same kernel with the keys in several chains, or on tiles of 64 rows
+    # where 128-row workgroups would be too few (0.5B, 2,048 tokens: four chains on 64-row
+    # tiles, 28.0 us against 29.5 in the 16-row kernel; 512 tokens over 3,584: 36.4 against
+    # 40.7; 1,024 tokens of 28 heads in 4 groups: two chains, 19.0 against 23.8; 3,072 tokens
+    # of 14 heads: three chains on 128-row tiles, 39.7 against 55.9), and two chains for
+    # 128-wide heads (7B, 2,048 tokens: 58.3 against 67.9 in one)
     assert plan(core, 14, 2, 64, [2048], 2048)["staged"] == 36
     p = plan(core, 14, 2, 64, [512], 4096)
     assert (p["staged"], p["rows"], p["tile_rows"]) == (36, 32, 64)
     assert plan(core, 28, 4, 64, [1024], 1024)["staged"] == 20
-    assert plan(core, 28, 4, 128, [1024], 1024)["staged"] < 8
+    assert plan(core, 14, 2, 64, [3072], 3072)["staged"] == 24
+    assert plan(core, 28, 4, 128, [2048], 2048)["staged"] == 16
+    assert plan(core, 28, 4, 128, [512], 512)["staged"] < 8
     # the q/k/v projection: one skinny kernel for few rows of a small matrix (1152 x 896 at 8
     # rows: 6.0 us against 10.6 as partial sums and a finishing kernel), partial sums for a
     # matrix of 24 MB or more (4608 x 3584 at 8..64 rows: 14.0..16.5 us against 15.2..30.7)

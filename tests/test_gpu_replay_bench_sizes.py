@@ -101,7 +101,7 @@ def exact_logits(folder, cfg, tokens):
              "f32_cost": float((single.double() - exact).abs().max())}
     return exact.float(), costs
 
-LONG = [("S64", 4736, 16), ("S128", 2432, 32)]
+LONG = [("S64", 4736, 16), ("S128", 2624, 32)]
 
 
 @pytest.fixture(scope="module", params=LONG, ids=[f"{n}-{t}" for n, t, _ in LONG])
