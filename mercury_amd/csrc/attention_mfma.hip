@@ -58,6 +58,7 @@ struct AttnParams {
   int split_blocks;  // key blocks per split; 0: each tile's range divided evenly
   int tile_rows;     // rows per tile: 16, 32 or 64
   int kv_fold;       // key/value heads per workgroup of the unstaged kernel: 1, 2 or 4
+  int direct;        // no tile list: tile t is the one new token of sequence t
 };
 
 #define ATTN_WAVES 4
@@ -127,6 +128,63 @@ __device__ __forceinline__ void load_key_block(KeyBlock<D>& blk, const AttnParam
     for (int h = 0; h < 2; ++h)
       blk.vf[dt].u2[h] = *(const uint2*)(vbase[h] + (v_lane + (uint32_t)(dt * 32 * ps)));
 }
+
+// The same loads for a block whose two halves' pages are known (wavefront-uniform), live or
+// not: addresses are valid either way, and what is not live is masked in the scores.
+template <int D>
+__device__ __forceinline__ void load_key_block_at(KeyBlock<D>& blk, const AttnParams& p, int b,
+                                                  int page_lo, int page_hi, bool live, int kvh,
+                                                  int lane) {
+  const int r = lane & 15, g4 = lane >> 4;
+  const int ps = 1 << p.page_shift;
+  const uint32_t k_lane = (uint32_t)(r * D + g4 * 8) * 2u;   // bytes
+  const uint32_t v_lane = (uint32_t)(r * ps + g4 * 4) * 2u;
+  const char* kbase[2];
+  const char* vbase[2];
+#pragma unroll
+  for (int h = 0; h < 2; ++h) {
+    const int kh = (b << 5) + h * 16;
+    blk.live[h] = live;
+    const int page = h ? page_hi : page_lo;
+    const int off = kh & (ps - 1);
+    const size_t head_bytes = ((size_t)page * p.n_kv + kvh) * ((size_t)ps * D * 2);
+    kbase[h] = (const char*)p.k_cache + head_bytes + (size_t)off * D * 2;
+    vbase[h] = (const char*)p.v_cache + head_bytes + (size_t)off * 2;
+  }
+#pragma unroll
+  for (int h = 0; h < 2; ++h)
+#pragma unroll
+    for (int c = 0; c < D / 32; ++c)
+      blk.kf[h][c].u = *(const uint4*)(kbase[h] + (k_lane + (uint32_t)c * 64u));
+#pragma unroll
+  for (int dt = 0; dt < D / 16; ++dt)
+#pragma unroll
+    for (int h = 0; h < 2; ++h)
+      blk.vf[dt].u2[h] = *(const uint2*)(vbase[h] + (v_lane + (uint32_t)(dt * 32 * ps)));
+}
+
+// A wavefront's view of the pages of every `stride`-th block of its sequence from `first` on:
+// lane l holds the two pages of block first + (base + l) * stride (a block of 32 keys lies in
+// one page or, with pages of 16, in two), 64 blocks at a time.
+struct StridedPages {
+  const int* table;
+  int width, first, stride, base, lo, hi;
+  __device__ __forceinline__ void fetch(int from, int page_shift, int lane) {
+    base = from;
+    const int key = (first + (from + lane) * stride) << 5;
+    const int a = key >> page_shift, b = (key + 16) >> page_shift;
+    // (entries past a sequence's pages are -1: page 0 stands in, its keys are masked)
+    lo = a < width ? max(table[a], 0) : 0;
+    hi = b < width ? max(table[b], 0) : 0;
+    __builtin_amdgcn_s_waitcnt(0x0F70);      // vmcnt(0), here and not before every readlane
+  }
+  // the pages of the wavefront's j-th block (j never decreases)
+  __device__ __forceinline__ void pages(int j, int page_shift, int lane, int& page_lo, int& page_hi) {
+    if (j >= base + 64) fetch(j, page_shift, lane);
+    page_lo = __builtin_amdgcn_readlane(lo, j - base);
+    page_hi = __builtin_amdgcn_readlane(hi, j - base);
+  }
+};
 
 // The running state of RT tiles of 16 rows: this lane's row of each tile.
 template <int D, int RT>
@@ -223,9 +281,20 @@ __device__ __forceinline__ void attend(TileState<D, RT>& st, const KeyBlock<D>& 
 // before anything is written: a quarter of the partial results for the merge, or none at all
 // when the workgroup has the tile's whole range.  p.num_splits then counts workgroups per
 // tile, each of ATTN_WAVES parts.
-template <int D, int RT, int AHEAD, bool GROUPED = false>
+//
+// DIRECT (decoding: every sequence brings one token, whose heads are one tile): tile t is
+// sequence t, so nothing has to be looked up before the block table and the queries are asked
+// for; and part s of S takes the blocks s, s + S, s + 2 S, ... of the keys, so a wavefront
+// knows its first block, and where in the table its blocks' pages stand, without the
+// sequence's length: table, queries and length travel together, the first block's keys and
+// values follow, and the length is there when the scores are masked.  Two trips to memory
+// before the first product instead of four, and parts that are equal for every sequence
+// whatever its length.  (A first block past a sequence's end is read from whatever page the
+// table names there, which exists, and masked.)
+template <int D, int RT, int AHEAD, bool GROUPED = false, bool DIRECT = false>
 __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) void attn_mfma_kernel(AttnParams p) {
   static_assert(!GROUPED || (RT == 1 && D <= 128), "grouped parts: one tile, heads up to 128");
+  static_assert(!DIRECT || (RT == 1 && AHEAD == 1), "direct: one tile, one block ahead");
   const int lane = threadIdx.x & 63;
   // Tiles are taken from the last: under a causal mask the later tiles of a prompt read the
   // most keys, and the longest work should start first.
@@ -238,9 +307,9 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
   const int kvh = GROUPED ? blockIdx.y : blockIdx.y * fold + wave % fold;
   const int split = GROUPED ? blockIdx.z * ATTN_WAVES + wave : blockIdx.z;
   const int splits = GROUPED ? p.num_splits * ATTN_WAVES : p.num_splits;
-  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
-  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
-  const int pos0 = p.kv_len[seq] - q_len;  // position of the step's first token of the sequence
+  const int seq = DIRECT ? tile : p.tile_seq[tile], row0 = DIRECT ? 0 : p.tile_row0[tile];
+  const int q0 = DIRECT ? seq : p.cu_q[seq], q_len = DIRECT ? 1 : p.cu_q[seq + 1] - q0;
+  const int kv_len = p.kv_len[seq];      // (DIRECT: asked for here, first used after the loads below)
   const int G = p.group;
   const int rows_total = q_len * G;
   const int r = lane & 15, g4 = lane >> 4;
@@ -254,8 +323,6 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
     st.row_ok[t] = flat < rows_total;
     tok[t] = st.row_ok[t] ? flat / G : 0;
     head[t] = kvh * G + (st.row_ok[t] ? flat % G : 0);
-    st.pos[t] = pos0 + tok[t];
-    st.lo[t] = p.window > 0 ? max(0, st.pos[t] - p.window + 1) : 0;
     st.m[t] = -INFINITY;
     st.lsum[t] = 0.f;
     const bf16_t* qrow = p.q + (size_t)(q0 + tok[t]) * p.q_stride + head[t] * D + g4 * 8;
@@ -264,6 +331,23 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
       st.qf[t][c].u = st.row_ok[t] ? *(const uint4*)(qrow + c * 32) : make_uint4(0, 0, 0, 0);
 #pragma unroll
     for (int dt = 0; dt < D / 16; ++dt) st.acc[t][dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  }
+
+  TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
+  StridedPages sp = {tw.table, tw.width, split, splits, 0, 0, 0};
+  KeyBlock<D> first_block;
+  if constexpr (DIRECT) {
+    sp.fetch(0, p.page_shift, lane);          // (the wait inside is for the queries too)
+    int page_lo, page_hi;
+    sp.pages(0, p.page_shift, lane, page_lo, page_hi);
+    load_key_block_at<D>(first_block, p, split, page_lo, page_hi, true, kvh, lane);
+  }
+
+  const int pos0 = kv_len - q_len;  // position of the step's first token of the sequence
+#pragma unroll
+  for (int t = 0; t < RT; ++t) {
+    st.pos[t] = pos0 + tok[t];
+    st.lo[t] = p.window > 0 ? max(0, st.pos[t] - p.window + 1) : 0;
   }
 
   // Keys any row of the tiles can see, in blocks of 32, and this split's share of them.
@@ -278,7 +362,6 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
   const int see_from = p.window > 0 ? max(0, kmax - p.window + 1) : 0;
   const float c = p.scale * 1.44269504088896340736f;
 
-  TableWindow tw = {p.block_table + (size_t)seq * p.table_stride, p.table_stride, -64, 0};
   if (AHEAD == 0) {
     KeyBlock<D> blk;
     for (int b = b0; b < b1; ++b) {
@@ -287,6 +370,23 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
     }
   } else if (AHEAD == 1) {
     KeyBlock<D> x, y;
+    if constexpr (DIRECT) {
+      // blocks split, split + S, ...: the wavefront's j-th block is b
+      x = first_block;
+      int page_lo, page_hi;
+      for (int b = split, j = 0; b < blk_hi; b += 2 * splits, j += 2) {
+        const bool more = b + splits < blk_hi;
+        sp.pages(more ? j + 1 : j, p.page_shift, lane, page_lo, page_hi);
+        load_key_block_at<D>(y, p, b + splits, page_lo, page_hi, more, kvh, lane);
+        attend<D, RT>(st, x, b << 5, c, g4, see_upto, see_from);
+        if (more) {
+          const bool further = b + 2 * splits < blk_hi;
+          sp.pages(further ? j + 2 : j + 1, p.page_shift, lane, page_lo, page_hi);
+          load_key_block_at<D>(x, p, b + 2 * splits, page_lo, page_hi, further, kvh, lane);
+          attend<D, RT>(st, y, (b + splits) << 5, c, g4, see_upto, see_from);
+        }
+      }
+    } else {
     load_key_block<D>(x, p, tw, b0, b1, kmin, kmax, kvh, lane);
     for (int b = b0; b < b1; b += 2) {
       load_key_block<D>(y, p, tw, b + 1, b1, kmin, kmax, kvh, lane);
@@ -295,6 +395,7 @@ __global__ __launch_bounds__(64 * ATTN_WAVES, (RT == 1 && D <= 128 ? 2 : 1)) voi
         load_key_block<D>(x, p, tw, b + 2, b1, kmin, kmax, kvh, lane);
         attend<D, RT>(st, y, (b + 1) << 5, c, g4, see_upto, see_from);
       }
+    }
     }
   } else {
     KeyBlock<D> x, y, z;
@@ -1099,8 +1200,9 @@ __global__ __launch_bounds__(256) void attn_merge_kernel(AttnParams p) {
   __shared__ float group_sum[4][D];
   __shared__ float scratch[16];
   const int tile = blockIdx.x, kvh = blockIdx.y, r = blockIdx.z, R = p.tile_rows;
-  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
-  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  // (no tile list: tile t is the one new token of sequence t)
+  const int seq = p.direct ? tile : p.tile_seq[tile], row0 = p.direct ? 0 : p.tile_row0[tile];
+  const int q0 = p.direct ? seq : p.cu_q[seq], q_len = p.direct ? 1 : p.cu_q[seq + 1] - q0;
   const int G = p.group;
   const int flat = row0 + r;
   if (flat >= q_len * G) return;
@@ -1151,8 +1253,9 @@ template <int D>
 __global__ __launch_bounds__(256) void attn_merge_rows_kernel(AttnParams p) {
   constexpr int PER = D / 16;
   const int tile = blockIdx.x, kvh = blockIdx.y, R = p.tile_rows, S = p.num_splits;
-  const int seq = p.tile_seq[tile], row0 = p.tile_row0[tile];
-  const int q0 = p.cu_q[seq], q_len = p.cu_q[seq + 1] - q0;
+  // (no tile list: tile t is the one new token of sequence t)
+  const int seq = p.direct ? tile : p.tile_seq[tile], row0 = p.direct ? 0 : p.tile_row0[tile];
+  const int q0 = p.direct ? seq : p.cu_q[seq], q_len = p.direct ? 1 : p.cu_q[seq + 1] - q0;
   const int G = p.group;
   const size_t base = ((size_t)tile * p.n_kv + kvh) * S;
   const int sub = threadIdx.x & 15;
@@ -1251,7 +1354,8 @@ static void launch_attn(const AttnParams& p, int rows_per_tile, bool merge, hipS
       AttnParams g = p;
       g.num_splits = p.num_splits / ATTN_WAVES;
       const dim3 grid(g.num_tiles, g.n_kv, g.num_splits);
-      attn_mfma_kernel<D, 1, ATTN_AHEAD_16, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(g);
+      if (g.direct) attn_mfma_kernel<D, 1, ATTN_AHEAD_16, true, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(g);
+      else attn_mfma_kernel<D, 1, ATTN_AHEAD_16, true><<<grid, 64 * ATTN_WAVES, 0, stream>>>(g);
       if (merge) launch_merge<D>(g, stream);
       return;
     }
@@ -1260,7 +1364,8 @@ static void launch_attn(const AttnParams& p, int rows_per_tile, bool merge, hipS
   dim3 grid((p.num_tiles + per - 1) / per, p.n_kv / p.kv_fold, p.num_splits);
   const int threads = 64 * ATTN_WAVES;
   if (rows_per_tile == 16) {
-    attn_mfma_kernel<D, 1, ATTN_AHEAD_16><<<grid, threads, 0, stream>>>(p);
+    if (p.direct) attn_mfma_kernel<D, 1, ATTN_AHEAD_16, false, true><<<grid, threads, 0, stream>>>(p);
+    else attn_mfma_kernel<D, 1, ATTN_AHEAD_16><<<grid, threads, 0, stream>>>(p);
   } else if (rows_per_tile == 32) {
     if constexpr (D <= 128) attn_mfma_kernel<D, 2, ATTN_AHEAD_32><<<grid, threads, 0, stream>>>(p);
   } else {
@@ -1393,6 +1498,14 @@ static int attention_mfma(const void* q, int q_stride, void* out, int out_stride
     return code;
   }
   if (num_tiles == 0) return 0;
+  // No tile list: tile t is the one new token of sequence t (see DIRECT).
+  const bool direct = tile_seq == nullptr;
+  MK_REQUIRE((tile_seq == nullptr) == (tile_row0 == nullptr), "attention: half a tile list");
+  MK_REQUIRE(!direct || (rows_per_tile == 16 && staged == 0 && window == 0 && n_q / n_kv <= 16 &&
+                         split_blocks == 0),
+             "attention: without a tile list every sequence brings one token of at most 16 heads "
+             "a group, in tiles of 16 rows, unwindowed (the parts of the keys are then every "
+             "num_splits-th block, not stretches of split_blocks)");
   AttnParams p;
   p.q = (const bf16_t*)q;
   p.q_stride = q_stride;
@@ -1420,6 +1533,7 @@ static int attention_mfma(const void* q, int q_stride, void* out, int out_stride
   // with few tiles the wavefronts are better spread over more workgroups (one decoded token
   // of 8 key/value heads: 10 us unfolded, 16 folded; 64 tokens: 194 and 186)
   p.kv_fold = num_tiles < 32 ? 1 : (n_kv % 4 == 0 ? 4 : (n_kv % 2 == 0 ? 2 : 1));
+  p.direct = direct;
   if (staged >= 8) {
     if (d == 64) launch_wide<64>(p, staged, stream); else launch_wide<128>(p, staged, stream);
     MK_LAUNCH_CHECK("attention_mfma");

@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 18
+#define MK_ABI_VERSION 19
 
 #ifdef __cplusplus
 extern "C" {
@@ -167,6 +167,10 @@ int mk_attention_mfma_max_rows(int head_dim);
 // four wavefronts taking the key blocks in turn; for many rows per sequence, keys unsplit.
 // staged = 8: the prompt kernel built on 32 x 32 x 16 products (wavefronts of 32 rows, blocks
 // of 64 keys; tiles of 128 rows, rows_per_tile = 32), where mk_attention_mfma_wide says so.
+// tile_seq = tile_row0 = null: no tile list, tile t is the one new token of sequence t
+// (decoding; tiles of 16 rows, at most 16 heads a group, no window, split_blocks 0): part s of
+// num_splits is then the blocks s, s + num_splits, ... of the keys, and the kernel asks for
+// nothing before the block table.
 // mk_attention_mfma_check: what mk_attention_mfma checks of its arguments before it launches,
 // without the launch (0: it would take them; else mk_last_error() says why not).
 int mk_attention_mfma_staged(int head_dim, int rows_per_tile);

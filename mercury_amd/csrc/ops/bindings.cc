@@ -43,6 +43,7 @@ py::dict plan_to_py(const AttentionPlan& p) {
   d["mfma"] = p.mfma;
   d["rows"] = p.rows;
   d["staged"] = p.staged;
+  d["direct"] = p.direct;
   d["splits"] = p.splits;
   d["split_blocks"] = p.split_blocks;
   d["tile_rows"] = p.tile_rows;
@@ -180,6 +181,7 @@ void bind_ops(py::module_& m) {
     p.mfma = py::cast<bool>(plan["mfma"]);
     p.rows = py::cast<int>(plan["rows"]);
     p.staged = py::cast<int>(plan["staged"]);
+    p.direct = plan.contains("direct") && py::cast<bool>(plan["direct"]);
     p.splits = py::cast<int>(plan["splits"]);
     p.split_blocks = py::cast<int>(plan["split_blocks"]);
     p.tile_rows = py::cast<int>(plan["tile_rows"]);

@@ -129,7 +129,12 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   total_rows *= group;
   // 64-row tiles exist but run at one wavefront per SIMD; 32 rows measured fastest
   const int max_rows = std::min(32, t.mk_attention_mfma_max_rows(head_dim));
-  while (rows < max_rows && (total_rows / (rows * 2)) * n_kv >= kAttentionWideTileWaves) rows *= 2;
+  // (never wider than the rows the longest sequence brings: a decoded token's heads are one
+  // tile of 16 however many sequences there are)
+  while (rows < max_rows && rows < (long long)max_q_len * group &&
+         (total_rows / (rows * 2)) * n_kv >= kAttentionWideTileWaves) {
+    rows *= 2;
+  }
   if (tile_rows > 0) rows = tile_rows;
   int staged = staged_in;
   const bool split_forced = splits_in > 0;
@@ -192,6 +197,13 @@ AttentionPlan plan_attention(int dtype, int head_dim, int page_size, int n_q, in
   if (split_forced) {
     plan.splits = splits_in;
     plan.split_blocks = split_blocks_in;
+  }
+  // Decoding (every sequence brings one token, whose heads are one tile): no tile list, the
+  // parts of the keys every splits-th block (the kernel then knows where a part starts before
+  // it knows the sequence's length).
+  if (!staged && !split_forced && tile_rows <= 0 && rows == 16 && max_q_len == 1 && window == 0 &&
+      group <= 16 && total_rows == (long long)counts.size() * group) {
+    plan.direct = true;
   }
   return plan;
 }

@@ -58,7 +58,9 @@ struct AttentionPlan {
                           // 8, 16, 24: the kernel of 32-row wavefronts with one, two, three groups;
                           // 20, 36: the same on tiles of 64 rows with two and four groups
   int splits = 1;
-  int split_blocks = 0;
+  int split_blocks = 0;   // key blocks (of 32) per part; 0: every tile's own range in equal parts
+  bool direct = false;    // decoding, one token per sequence: no tile list, part s of the keys is
+                          // every splits-th block from s
   int tile_rows = 16;     // rows per entry of the tile list: rows, 4 * rows when staged, 2 * rows for 20 and 36
   int num_tiles = 0;
 };

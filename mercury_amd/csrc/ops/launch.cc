@@ -219,7 +219,8 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
   if (l.dry() || m == 0) return out;
   const mk_tile_list& tiles = tiles_for(step, a.n_q / a.n_kv, plan.tile_rows);
   check_mfma(need_mfma().mk_attention_mfma(
-                 q.q, q.stride, out, a.n_q * d, a.k_cache, a.v_cache, tiles.seq, tiles.row0,
+                 q.q, q.stride, out, a.n_q * d, a.k_cache, a.v_cache,
+                 plan.direct ? nullptr : tiles.seq, plan.direct ? nullptr : tiles.row0,
                  tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride, a.page_size, a.n_q, a.n_kv,
                  d, a.scale, a.window, plan.rows, plan.staged, plan.splits, plan.split_blocks,
                  part_o, part_ml, l.stream()), "attention");
@@ -277,8 +278,9 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
   if (l.dry() || m == 0) return;
   const KernelTable& t = need_mfma();
   const mk_tile_list& tiles = tiles_for(step, a.n_q / a.n_kv, plan.tile_rows);
-  check_mfma(t.mk_attention_mfma_parts(q.q, q.stride, a.k_cache, a.v_cache, tiles.seq, tiles.row0,
-                                       tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride,
+  check_mfma(t.mk_attention_mfma_parts(q.q, q.stride, a.k_cache, a.v_cache,
+                                       plan.direct ? nullptr : tiles.seq,
+                                       plan.direct ? nullptr : tiles.row0, tiles.count, s.cu_q, s.kv_len, s.table, s.table_stride,
                                        a.page_size, a.n_q, a.n_kv, d, a.scale, a.window, plan.rows,
                                        plan.splits, plan.split_blocks, part_o, part_ml, l.stream()),
              "attention");

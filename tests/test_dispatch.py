@@ -79,6 +79,13 @@ def test_every_plan_is_one_the_kernel_accepts(core):
         assert 1 <= p["splits"] <= max(1, blocks // 2) or p["splits"] == 1, case
         if p["splits"] > 1:
             assert p["staged"] == 0 and (p["splits"] < 4 or p["splits"] % 4 == 0), case
+        # without a tile list: only where every sequence brings one token whose heads are one
+        # tile of 16 rows, unwindowed, the keys' parts every n-th block
+        if p["direct"]:
+            assert set(counts) == {1} and group <= 16 and not window and not p["staged"], case
+            assert p["rows"] == 16 and p["split_blocks"] == 0 and p["num_tiles"] == len(counts), case
+        elif set(counts) == {1} and group <= 16 and not window:
+            assert False, case      # a decode step that misses the direct kernel
         # the kernel of 32-row wavefronts: only where a sequence has at least 128 rows
         if p["staged"] >= 8:
             assert max(counts) * group >= (64 if half else 128) and p["rows"] == 32, case

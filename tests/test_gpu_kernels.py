@@ -851,6 +851,45 @@ def test_attention_decode_with_split_keys(batch, context):
     torch.testing.assert_close(got, want, **tol(torch.bfloat16))
 
 
+@pytest.mark.parametrize("n_q,n_kv,d,page,lens", [
+    (14, 2, 64, 16, [3000, 5, 70, 1, 33, 1024]), (8, 2, 128, 32, [2500, 1, 64, 31]),
+    (6, 3, 32, 64, [130, 4000, 2]), (4, 4, 96, 16, [700, 17])])
+def test_attention_decode_of_sequences_of_very_different_lengths(n_q, n_kv, d, page, lens):
+    """Decoding takes the parts of a sequence's keys as every n-th block and asks for a part's
+    first block before it knows the sequence's length: most parts of the short sequences here
+    start past their end, where the block table holds -1 (and the cache poison); one key far
+    back in each longer sequence carries a score that stands out, so a block that is skipped or
+    taken twice shows."""
+    bf = torch.bfloat16
+    batch = len(lens)
+    per = -(-max(lens) // page)
+    qs, ks, vs = [], [], []
+    for i, n in enumerate(lens):
+        k = rnd(n, n_kv, d, seed=330 + i)
+        q = rnd(1, n_q, d, seed=230 + i)
+        if n > 40:
+            far = n // 3
+            k[far] *= 3.0
+            q[0] += 6.0 / (9 * d ** 0.5) * k[far].repeat_interleave(n_q // n_kv, 0)
+        qs.append(rounded(q, bf))
+        ks.append(rounded(k, bf))
+        vs.append(rounded(rnd(n, n_kv, d, seed=430 + i), bf))
+    order = torch.randperm(batch * per + 3, generator=torch.Generator().manual_seed(5)).tolist()
+    pages, at = [], 0
+    for n in lens:
+        need = -(-n // page)
+        pages.append(order[at:at + need])
+        at += need
+    from mercury_amd.hostcore import core
+    plan = core.plan_attention(1, d, page, n_q, n_kv, 0, [1] * batch, 1, max(lens))
+    assert plan["mfma"] and plan["direct"] and plan["splits"] > 1, plan
+    got = run_attention(qs, ks, vs, bf, pages, page, batch * per + 3, lens, [1] * batch,
+                        d ** -0.5, poison=1e4, kernel="mfma")
+    want = torch.cat([plain.causal_attention(q, k, v, d ** -0.5, n - 1)
+                      for q, k, v, n in zip(qs, ks, vs, lens)])
+    torch.testing.assert_close(got, want, **tol(bf))
+
+
 @pytest.mark.parametrize("n_q,n_kv,d,hidden,batch,context", [
     (14, 2, 64, 896, 8, 4096), (14, 2, 64, 896, 1, 700), (14, 2, 64, 896, 64, 1100),
     (8, 2, 128, 1024, 3, 2000), (28, 4, 128, 200, 17, 900), (6, 3, 64, 1000, 33, 520),
