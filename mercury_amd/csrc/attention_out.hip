@@ -63,6 +63,34 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutParams p) {
     return (((size_t)tok * p.n_kv + kvh) * S) * 16 + j;
   };
 
+  // The parts' weighted values are asked for now as well, where a thread's share of them fits
+  // its registers (sixteen loads of four floats): they depend on nothing either, and asked
+  // for after the weights are known (below) they would be a second chain of trips to memory
+  // behind the first.  A thread's items are (pair, four dims) number threadIdx.x + 256 it.
+  constexpr int QUADS = D / 4;
+  constexpr int ITEMS = (16 * MT * HP * QUADS + 255) / 256;   // items per thread
+  constexpr int HELD = 16 / ITEMS;                            // parts per item a thread can hold
+  // (From 17 tokens on: with fewer the merge hides behind the weights' way from HBM either
+  // way, 1.010 against 1.013 ms a step of 8 tokens of the 0.5B shapes; 64 tokens: 1.634
+  // against 1.662.)
+  const bool ahead = MT >= 2 && ITEMS <= 4 && S <= HELD;
+  float4 held[MT >= 2 && ITEMS <= 4 ? ITEMS : 1][MT >= 2 && ITEMS <= 4 ? HELD : 1];
+  if constexpr (MT >= 2 && ITEMS <= 4) {
+    if (ahead) {
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int i = threadIdx.x + 256 * it;
+        const int pair = i / QUADS, quad = i - pair * QUADS;
+        const bool real = i < 16 * MT * HP * QUADS && pair / HP < p.M;
+        const float4* src = (const float4*)(p.part_o + base_of(real ? pair : 0) * D + quad * 4);
+#pragma unroll
+        for (int s2 = 0; s2 < HELD; ++s2) {
+          held[it][s2] = real && s2 < S ? src[(size_t)s2 * (16 * D / 4)] : make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+      }
+    }
+  }
+
   // Merge, step 1: every part's maximum and sum, all loads at once.
   for (int i = threadIdx.x; i < pairs * S; i += 256) {
     const int pair = i / S, part = i - pair * S;
@@ -88,38 +116,82 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutParams p) {
     for (int s2 = 0; s2 < S; ++s2) w[s2] *= inv;
   }
   __syncthreads();
-  // Step 3: a thread per four dims of a pair adds the weighted parts up in part order, four
-  // parts' loads in flight at a time, and leaves bfloat16 in LDS (what the attention would
-  // have written).
-  constexpr int QUADS = D / 4;
-  for (int i = threadIdx.x; i < 16 * MT * HP * QUADS; i += 256) {
-    const int pair = i / QUADS, quad = i - pair * QUADS;
-    const int tok = pair / HP, hh = pair - tok * HP;
-    uint2* dst = (uint2*)(merged + tok * STRIDE + hh * D + quad * 4);
-    if (tok >= p.M) {
-      *dst = make_uint2(0u, 0u);
-      continue;
+  // Step 3: a thread per four dims of a pair adds the weighted parts up in part order (in
+  // fours, then what is left one by one: the same sums whether the values were asked for
+  // ahead or are only now, four parts' loads in flight at a time) and leaves bfloat16 in LDS
+  // (what the attention would have written).
+  bool done = false;
+  if constexpr (MT >= 2 && ITEMS <= 4) {
+    if (ahead) {
+#pragma unroll
+      for (int it = 0; it < ITEMS; ++it) {
+        const int i = threadIdx.x + 256 * it;
+        if (i >= 16 * MT * HP * QUADS) continue;
+        const int pair = i / QUADS, quad = i - pair * QUADS;
+        const int tok = pair / HP, hh = pair - tok * HP;
+        uint2* dst = (uint2*)(merged + tok * STRIDE + hh * D + quad * 4);
+        if (tok >= p.M) {
+          *dst = make_uint2(0u, 0u);
+          continue;
+        }
+        const float* w = weight + pair * S;
+        float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+        for (int g = 0; g < HELD; g += 4) {       // (constant indices: the values are registers)
+          if (g + 4 <= HELD && g + 4 <= S) {
+            const float4 v0 = held[it][g], v1 = held[it][g + 1 < HELD ? g + 1 : 0];
+            const float4 v2 = held[it][g + 2 < HELD ? g + 2 : 0], v3 = held[it][g + 3 < HELD ? g + 3 : 0];
+            const float w0 = w[g], w1 = w[g + 1], w2 = w[g + 2], w3 = w[g + 3];
+            o.x += (v0.x * w0 + v1.x * w1) + (v2.x * w2 + v3.x * w3);
+            o.y += (v0.y * w0 + v1.y * w1) + (v2.y * w2 + v3.y * w3);
+            o.z += (v0.z * w0 + v1.z * w1) + (v2.z * w2 + v3.z * w3);
+            o.w += (v0.w * w0 + v1.w * w1) + (v2.w * w2 + v3.w * w3);
+          } else {
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+              if (g + k < HELD && g + k < S) {
+                const float4 v = held[it][g + k < HELD ? g + k : 0];
+                const float ws = w[g + k];
+                o.x += v.x * ws, o.y += v.y * ws, o.z += v.z * ws, o.w += v.w * ws;
+              }
+            }
+          }
+        }
+        *dst = make_uint2(pack_bf16x2(o.x, o.y), pack_bf16x2(o.z, o.w));
+      }
+      done = true;
     }
-    const float4* src = (const float4*)(p.part_o + base_of(pair) * D + quad * 4);
-    const size_t step = (size_t)16 * D / 4;
-    const float* w = weight + pair * S;
-    float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
-    int s2 = 0;
-    for (; s2 + 4 <= S; s2 += 4) {
-      const float4 v0 = src[(size_t)s2 * step], v1 = src[(size_t)(s2 + 1) * step];
-      const float4 v2 = src[(size_t)(s2 + 2) * step], v3 = src[(size_t)(s2 + 3) * step];
-      const float w0 = w[s2], w1 = w[s2 + 1], w2 = w[s2 + 2], w3 = w[s2 + 3];
-      o.x += (v0.x * w0 + v1.x * w1) + (v2.x * w2 + v3.x * w3);
-      o.y += (v0.y * w0 + v1.y * w1) + (v2.y * w2 + v3.y * w3);
-      o.z += (v0.z * w0 + v1.z * w1) + (v2.z * w2 + v3.z * w3);
-      o.w += (v0.w * w0 + v1.w * w1) + (v2.w * w2 + v3.w * w3);
+  }
+  if (!done) {
+    for (int i = threadIdx.x; i < 16 * MT * HP * QUADS; i += 256) {
+      const int pair = i / QUADS, quad = i - pair * QUADS;
+      const int tok = pair / HP, hh = pair - tok * HP;
+      uint2* dst = (uint2*)(merged + tok * STRIDE + hh * D + quad * 4);
+      if (tok >= p.M) {
+        *dst = make_uint2(0u, 0u);
+        continue;
+      }
+      const float4* src = (const float4*)(p.part_o + base_of(pair) * D + quad * 4);
+      const size_t step = (size_t)16 * D / 4;
+      const float* w = weight + pair * S;
+      float4 o = make_float4(0.f, 0.f, 0.f, 0.f);
+      int s2 = 0;
+      for (; s2 + 4 <= S; s2 += 4) {
+        const float4 v0 = src[(size_t)s2 * step], v1 = src[(size_t)(s2 + 1) * step];
+        const float4 v2 = src[(size_t)(s2 + 2) * step], v3 = src[(size_t)(s2 + 3) * step];
+        const float w0 = w[s2], w1 = w[s2 + 1], w2 = w[s2 + 2], w3 = w[s2 + 3];
+        o.x += (v0.x * w0 + v1.x * w1) + (v2.x * w2 + v3.x * w3);
+        o.y += (v0.y * w0 + v1.y * w1) + (v2.y * w2 + v3.y * w3);
+        o.z += (v0.z * w0 + v1.z * w1) + (v2.z * w2 + v3.z * w3);
+        o.w += (v0.w * w0 + v1.w * w1) + (v2.w * w2 + v3.w * w3);
+      }
+      for (; s2 < S; ++s2) {
+        const float4 v = src[(size_t)s2 * step];
+        const float ws = w[s2];
+        o.x += v.x * ws, o.y += v.y * ws, o.z += v.z * ws, o.w += v.w * ws;
+      }
+      *dst = make_uint2(pack_bf16x2(o.x, o.y), pack_bf16x2(o.z, o.w));
     }
-    for (; s2 < S; ++s2) {
-      const float4 v = src[(size_t)s2 * step];
-      const float ws = w[s2];
-      o.x += v.x * ws, o.y += v.y * ws, o.z += v.z * ws, o.w += v.w * ws;
-    }
-    *dst = make_uint2(pack_bf16x2(o.x, o.y), pack_bf16x2(o.z, o.w));
   }
   __syncthreads();
 
