@@ -230,7 +230,8 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
 namespace {
 // The merge of the key splits folded into the output projection repeats the merge once per
 // 64 (or 128) rows of w_o; it pays while that repetition stays small beside what the two
-// kernels it replaces cost (measured at 8 and 64 decoded tokens: see DESIGN's kernel notes).
+// kernels it replaces cost (0.5B shapes, 8 decoded tokens: 11.5 us a layer against 14.6 as
+// three kernels; 32B shapes, 64 tokens: 247 against 204, 100 MB of parts repeated).
 constexpr long long kFoldMaxRepeatedBytes = 48ll << 20;
 constexpr int kFoldWideFromHidden = 2048;
 }  // namespace
