@@ -160,6 +160,28 @@ def test_long_request_whole_then_a_decoded_tail(long_case, dtype):
     assert s.manager.leaked_pages() == 0
 
 
+@pytest.mark.parametrize("length,code", [(1280, 20), (3072, 24)])
+def test_prompts_of_middle_lengths_through_the_other_attention_instantiations(length, code):
+    """Between the short prompts of the small cases and the long ones above, the planner takes
+    the 32-row attention kernel in two chains on tiles of 64 rows (1,280 tokens of 14 heads
+    of 64) and in three chains on tiles of 128 (3,072): whole prompts of those lengths through
+    the model, against the float64 run."""
+    from mercury_amd.hostcore import core
+    from mercury_amd.kernels import ops
+
+    folder = folder_for("S64", sharpen=3.0)
+    cfg = plain.read_config(folder)
+    plan = core.plan_attention(ops.BF16, cfg["head_dim"], 16, cfg["num_attention_heads"],
+                               cfg["num_key_value_heads"], 0, [length], length, length)
+    assert plan["mfma"] and plan["staged"] == code, plan
+    tokens = helpers.random_tokens(cfg["vocab_size"], length, seed=length)
+    want, cost = exact_logits(folder, cfg, tokens)
+    s = session(folder, "bfloat16", length, 16)
+    got = s.step([entry("x", tokens)], ["x"])
+    check(got, want, "bfloat16", f"S64, {length} tokens whole", **cost)
+    assert s.manager.leaked_pages() == 0
+
+
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
 def test_long_request_in_portions_beside_a_decoding_neighbour(long_case, dtype):
     """The benchmark's serving shape: portions of 512 tokens of a long prompt beside another
