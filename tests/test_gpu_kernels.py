@@ -853,7 +853,8 @@ def test_attention_decode_with_split_keys(batch, context):
 
 @pytest.mark.parametrize("n_q,n_kv,d,page,lens", [
     (14, 2, 64, 16, [3000, 5, 70, 1, 33, 1024]), (8, 2, 128, 32, [2500, 1, 64, 31]),
-    (6, 3, 32, 64, [130, 4000, 2]), (4, 4, 96, 16, [700, 17])])
+    (6, 3, 32, 64, [130, 4000, 2]), (4, 4, 96, 16, [700, 17]), (8, 1, 256, 64, [900, 3, 200]),
+    (6, 2, 192, 32, [1500, 40])])
 def test_attention_decode_of_sequences_of_very_different_lengths(n_q, n_kv, d, page, lens):
     """Decoding takes the parts of a sequence's keys as every n-th block and asks for a part's
     first block before it knows the sequence's length: most parts of the short sequences here
@@ -881,7 +882,9 @@ def test_attention_decode_of_sequences_of_very_different_lengths(n_q, n_kv, d, p
         pages.append(order[at:at + need])
         at += need
     from mercury_amd.hostcore import core
-    plan = core.plan_attention(1, d, page, n_q, n_kv, 0, [1] * batch, 1, max(lens))
+    from mercury_amd.kernels import lib
+    lib.load("core"), lib.load("mfma")
+    plan = core.plan_attention(ops().BF16, d, page, n_q, n_kv, 0, [1] * batch, 1, max(lens))
     assert plan["mfma"] and plan["direct"] and plan["splits"] > 1, plan
     got = run_attention(qs, ks, vs, bf, pages, page, batch * per + 3, lens, [1] * batch,
                         d ** -0.5, poison=1e4, kernel="mfma")
