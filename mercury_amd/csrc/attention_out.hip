@@ -7,9 +7,10 @@
 // the output matrix W [N, n_q D] and HP query heads (a slice of K): it first asks for its
 // weights, then merges its heads' parts for all M tokens into LDS (bfloat16, what the
 // attention would have written), multiplies, and writes a float32 partial sum
-// out[slice, M, N] that the next norm adds up in slice order.  Every workgroup of a slice
-// repeats the slice's merge (the parts come out of the L2); the host chooses this kernel
-// where that repetition is small beside the weights.
+// out[slice, M, N] that the next norm adds up in slice order, or adds its result into the
+// fixed-point residual stream.  Every workgroup of a slice repeats the slice's merge (the
+// parts come out of the L2); the host chooses this kernel where that repetition is small
+// beside the weights.
 #include "common.h"
 #include "mercury_kernels.h"
 
@@ -25,7 +26,8 @@ struct AttnOutParams {
   const float* part_o;   // [token, kv head, part, 16, D]
   const float* part_ml;  // [token, kv head, part, 16, 2]: base-2 running maximum, sum of weights
   const bf16_t* w;       // [N, n_q * D]
-  float* out;            // [n_q / HP, M, N]
+  float* out;            // [n_q / HP, M, N], or null and
+  fixed_t* fixed_out;    // [M, N]: the fixed-point residual stream the result is added into
   int M, N, n_kv, group, parts;
 };
 
@@ -216,6 +218,17 @@ __global__ __launch_bounds__(256) void attn_out_kernel(AttnOutParams p) {
   for (int tb = 0; tb < MT; ++tb) {
     const int m = tb * 16 + r;
     if (m >= p.M) continue;
+    if (p.fixed_out) {
+      fixed_t* sum = p.fixed_out + (size_t)m * p.N;
+#pragma unroll
+      for (int t = 0; t < NW; ++t) {
+        const int n = n0 + t * 16 + g4 * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          if (n + i < p.N) add_fixed(sum + n + i, acc[t][tb][i]);
+      }
+      continue;
+    }
     float* dst = p.out + ((size_t)slice * p.M + m) * p.N;
 #pragma unroll
     for (int t = 0; t < NW; ++t) {
@@ -259,8 +272,9 @@ static void launch_out(const AttnOutParams& p, int n_q, hipStream_t stream) {
 }
 
 extern "C" int mk_attention_out(const float* part_o, const float* part_ml, int parts,
-                                const void* w_o, float* out, int M, int N, int n_q, int n_kv, int d,
-                                int heads_per_slice, int wide, hipStream_t stream) {
+                                const void* w_o, float* out, long long* fixed_out, int M, int N,
+                                int n_q, int n_kv, int d, int heads_per_slice, int wide,
+                                hipStream_t stream) {
   MK_REQUIRE(parts >= 2 && parts <= mk_attention_out_max_parts(M, heads_per_slice),
              "attention_out: %d parts (2 to %d for %d tokens and %d heads per slice)", parts,
              mk_attention_out_max_parts(M, heads_per_slice), M, heads_per_slice);
@@ -268,13 +282,15 @@ extern "C" int mk_attention_out(const float* part_o, const float* part_ml, int p
                  heads_per_slice == mk_attention_out_heads_per_slice(n_q, n_kv, d, M, N),
              "attention_out: sizes not taken (head size 64 or 128, at most 64 tokens), or another "
              "number of heads per slice than mk_attention_out_heads_per_slice gives");
-  MK_REQUIRE(part_o && part_ml && w_o && out, "attention_out: null argument");
+  MK_REQUIRE(part_o && part_ml && w_o && (out != nullptr) != (fixed_out != nullptr),
+             "attention_out: null argument, or not exactly one of the two outputs");
   MK_REQUIRE(((n_q * d) & 7) == 0, "attention_out: rows of W must be 16-byte aligned");
   AttnOutParams p;
   p.part_o = part_o;
   p.part_ml = part_ml;
   p.w = (const bf16_t*)w_o;
   p.out = out;
+  p.fixed_out = (fixed_t*)fixed_out;
   p.M = M;
   p.N = N;
   p.n_kv = n_kv;

@@ -72,6 +72,27 @@ struct Elem<bf16_t> {
   static __device__ __forceinline__ float round(float v) { return bf16_to_f32(f32_to_bf16(v)); }
 };
 
+// ------------------------------------------------------- the residual stream in fixed point
+//
+// In steps of a few tokens the residual stream is kept as 64-bit integers in units of 2^-32
+// (range +-2^31, finer than float32 from 2^-8 up): projections add their results into it with
+// integer atomics, whose sum does not depend on the order they arrive in, so that partial
+// results over slices of K need neither a buffer nor a kernel that adds them up, and a value
+// is the same whichever workgroup finished first.
+typedef long long fixed_t;
+
+__device__ __forceinline__ fixed_t to_fixed(float y) {
+  return __float2ll_rn(fminf(fmaxf(y, -1.0e9f), 1.0e9f) * 4294967296.f);
+}
+
+__device__ __forceinline__ float from_fixed(fixed_t a) {
+  return __ll2float_rn(a) * 2.3283064365386963e-10f;
+}
+
+__device__ __forceinline__ void add_fixed(fixed_t* p, float y) {
+  atomicAdd((unsigned long long*)p, (unsigned long long)to_fixed(y));
+}
+
 // ------------------------------------------------------------------------------- reductions
 
 __device__ __forceinline__ float wave_sum(float v) {

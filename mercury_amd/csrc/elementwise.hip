@@ -64,6 +64,35 @@ extern "C" int mk_embed(const int* ids, const void* table, int dtype, float* out
   return 0;
 }
 
+// The same into the fixed-point residual stream of a step of few tokens.
+template <typename T>
+__global__ void embed_fixed_kernel(const int* __restrict__ ids, const T* __restrict__ table,
+                                   fixed_t* __restrict__ out, int hidden, int vocab, float scale) {
+  const int t = blockIdx.x;
+  int id = ids[t];
+  id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);
+  const T* row = table + (size_t)id * hidden;
+  fixed_t* dst = out + (size_t)t * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) dst[i] = to_fixed(Elem<T>::load(row + i) * scale);
+}
+
+extern "C" int mk_embed_fixed(const int* ids, const void* table, int dtype, long long* out,
+                              int tokens, int hidden, int vocab, float scale, hipStream_t stream) {
+  MK_REQUIRE(tokens >= 0 && hidden > 0 && vocab > 0, "embed: bad sizes T=%d H=%d V=%d", tokens,
+             hidden, vocab);
+  MK_REQUIRE(dtype == MK_F32 || dtype == MK_BF16, "embed: unknown dtype %d", dtype);
+  if (tokens == 0) return 0;
+  const int threads = hidden >= 1024 ? 1024 : (hidden + 63) / 64 * 64;
+  if (dtype == MK_F32)
+    embed_fixed_kernel<float><<<tokens, threads, 0, stream>>>(ids, (const float*)table,
+                                                              (fixed_t*)out, hidden, vocab, scale);
+  else
+    embed_fixed_kernel<bf16_t><<<tokens, threads, 0, stream>>>(ids, (const bf16_t*)table,
+                                                               (fixed_t*)out, hidden, vocab, scale);
+  MK_LAUNCH_CHECK("embed_fixed");
+  return 0;
+}
+
 // ------------------------------------------------------------------------------- logit cap
 
 // x <- cap * tanh(x / cap), in place: a smooth bound on the logits' size.  tanh from one
@@ -333,6 +362,72 @@ static int launch_rmsnorm(float* h, const float* partials, int num_partials,
   else
     rmsnorm_kernel<TO, bf16_t><<<out_rows, threads, 0, stream>>>(
         h, partials, num_partials, partial_stride, (const bf16_t*)weight, eps, rows, out, hidden);
+  return 0;
+}
+
+// RMSNorm of rows of the fixed-point residual stream: one block per output row, the row's
+// values two a thread and turn, the formula and the roundings of rmsnorm_kernel.
+template <typename TO>
+__global__ void rmsnorm_fixed_kernel(const fixed_t* __restrict__ h64, const void* __restrict__ weight,
+                                     int weight_bf16, float eps, const int* __restrict__ rows,
+                                     TO* __restrict__ out, int hidden) {
+  __shared__ float scratch[16];
+  const int out_row = blockIdx.x;
+  const int in_row = rows ? rows[out_row] : out_row;
+  const fixed_t* x = h64 + (size_t)in_row * hidden;
+  float sq = 0.f;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float v = from_fixed(x[i]);
+    sq += v * v;
+  }
+  const float total = block_sum(sq, scratch);
+  const float rstd = rsqrtf(total / (float)hidden + eps);
+  TO* dst = out + (size_t)out_row * hidden;
+  for (int i = threadIdx.x; i < hidden; i += blockDim.x) {
+    const float n = Elem<TO>::round(from_fixed(x[i]) * rstd);
+    const float w = weight_bf16 ? bf16_to_f32(((const bf16_t*)weight)[i]) : ((const float*)weight)[i];
+    Elem<TO>::store(dst + i, n * w);
+  }
+}
+
+extern "C" int mk_rmsnorm_fixed(const long long* h64, const void* weight, int weight_dtype,
+                                float eps, const int* rows, void* out, int out_dtype, int out_rows,
+                                int hidden, hipStream_t stream) {
+  MK_REQUIRE(out_rows >= 0 && hidden > 0, "rmsnorm: bad sizes rows=%d H=%d", out_rows, hidden);
+  MK_REQUIRE(weight_dtype == MK_F32 || weight_dtype == MK_BF16, "rmsnorm: weight dtype %d",
+             weight_dtype);
+  MK_REQUIRE(out_dtype == MK_F32 || out_dtype == MK_BF16, "rmsnorm: unknown out dtype %d", out_dtype);
+  if (out_rows == 0) return 0;
+  const int threads = hidden >= 1024 ? 1024 : (hidden + 63) / 64 * 64;
+  if (out_dtype == MK_F32)
+    rmsnorm_fixed_kernel<float><<<out_rows, threads, 0, stream>>>(
+        (const fixed_t*)h64, weight, weight_dtype == MK_BF16, eps, rows, (float*)out, hidden);
+  else
+    rmsnorm_fixed_kernel<bf16_t><<<out_rows, threads, 0, stream>>>(
+        (const fixed_t*)h64, weight, weight_dtype == MK_BF16, eps, rows, (bf16_t*)out, hidden);
+  MK_LAUNCH_CHECK("rmsnorm_fixed");
+  return 0;
+}
+
+// h64[i] += the sum of `count` float32 partial sums p[k * stride + i] (k in ascending order,
+// as sum_partials adds them), for i < n: what a projection that left partial sums owes the
+// fixed-point residual stream.
+__global__ void fixed_add_kernel(fixed_t* __restrict__ h64, const float* __restrict__ partials,
+                                 int count, size_t stride, long long n) {
+  const long long i = (long long)blockIdx.x * blockDim.x + threadIdx.x;
+  if (i >= n) return;
+  h64[i] += to_fixed(sum_partials(partials + i, count, stride));
+}
+
+extern "C" int mk_fixed_add(long long* h64, const float* partials, int count, long long stride,
+                            long long n, hipStream_t stream) {
+  MK_REQUIRE(count >= 1 && partials && h64 && n >= 0 && stride >= n, "fixed_add: bad arguments");
+  if (n == 0) return 0;
+  const long long blocks = (n + 255) / 256;
+  MK_REQUIRE(blocks < (1ll << 31), "fixed_add: %lld elements are too many for one launch", n);
+  fixed_add_kernel<<<(unsigned)blocks, 256, 0, stream>>>((fixed_t*)h64, partials, count,
+                                                         (size_t)stride, n);
+  MK_LAUNCH_CHECK("fixed_add");
   return 0;
 }
 

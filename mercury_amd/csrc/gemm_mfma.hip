@@ -52,7 +52,12 @@ __device__ __forceinline__ uint4 ld16(const bf16_t* p) { return *(const uint4*)p
 //               head's first half and tile 1 the same rows of its second half, so every lane
 //               holds both members of a rotation pair: bias, rounding, rotation by the token's
 //               position, q to `q_out`, k and v into the paged cache.  All of K.
-enum { SK_PARTIAL = 0, SK_GATED = 1, SK_ACC = 2, SK_QKV = 3 };
+//   SK_FIXED    rows n0.. of W, one slice of K each; y (+ bias, from slice 0) is added into
+//               the fixed-point residual stream out[m][n] with integer atomics.
+// NORMED (SK_GATED, SK_QKV, at most 16 rows): x is not read but made: the rows of the
+// fixed-point residual stream `h64`, RMS-normalised and weighted as the norm kernel would
+// have left them (reference: mercury/model/qwen2.py:27-31), each by one wavefront, into LDS.
+enum { SK_PARTIAL = 0, SK_GATED = 1, SK_ACC = 2, SK_QKV = 3, SK_FIXED = 4 };
 
 // Where the q/k/v projection's results go, and how they are rotated on the way.
 struct QkvTarget {
@@ -73,9 +78,18 @@ struct SkinnyArgs : QkvTarget {
   const bf16_t* w;
   void* out;
   int M, N, K, steps_per_slice;
-  const void* bias;  // SK_ACC, SK_QKV: [N] or null
+  const void* bias;  // SK_ACC, SK_QKV, SK_FIXED: [N] or null
   int bias_bf16;
+  // NORMED
+  const fixed_t* h64;   // [M, K]
+  const void* norm_w;   // [K]
+  int norm_bf16;
+  float norm_eps;
 };
+
+// The rows of x a NORMED workgroup makes for itself: [M][K + 8] bfloat16 (16 bytes of padding
+// a row against bank conflicts).
+extern __shared__ __align__(16) unsigned char skinny_rows[];
 
 // g * sigmoid(g) for a result that is rounded to bfloat16 next: the hardware's exponential
 // and reciprocal (an ulp or two of float32 each) in place of the library's, a dozen
@@ -186,9 +200,10 @@ __device__ __forceinline__ void qkv_store(const QkvTarget& p, const QkvPlace& pl
 // current step's products; the wavefronts' results are added through LDS in wave order.
 // Product j of a step takes k = step*128 + j*32 + g4*8 .. + 8 from a lane, so that one load
 // instruction reads 64 contiguous bytes of each of its 16 rows.
-template <int MT, int NT, int EPI, int WAVES>
+template <int MT, int NT, int EPI, int WAVES, bool NORMED = false>
 __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   static_assert((EPI != SK_GATED && EPI != SK_QKV) || NT == 2, "paired tiles");
+  static_assert(!NORMED || MT == 1, "rows made in LDS: at most 16");
   __shared__ float red[WAVES - 1][NT * MT * 4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g4 = lane >> 4;
   const int M = p.M, N = p.N, K = p.K;
@@ -213,7 +228,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   }
   const bf16_t* xrow[MT];
 #pragma unroll
-  for (int t = 0; t < MT; ++t) xrow[t] = p.x + (size_t)min(t * 16 + r, M - 1) * K;
+  for (int t = 0; t < MT; ++t) xrow[t] = NORMED ? nullptr : p.x + (size_t)min(t * 16 + r, M - 1) * K;
+  const bf16_t* made = (const bf16_t*)skinny_rows;   // NORMED
+  const int made_stride = K + 8, made_row = min(r, M - 1) * made_stride;
 
   constexpr int DEPTH = MT == 1 ? 3 : (MT == 2 ? 2 : 1);
   Frag a[DEPTH][NT][4], b[DEPTH][MT][4];
@@ -233,10 +250,46 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
     for (int j = 0; j < 4; ++j) {
       const bool ok = kk + j * 32 < K;
 #pragma unroll
-      for (int t = 0; t < MT; ++t)
-        b[buf][t][j].u = ok ? ld16(xrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
+      for (int t = 0; t < MT; ++t) {
+        if constexpr (NORMED) {
+          b[buf][t][j].u = ok ? *(const uint4*)(made + made_row + kk + j * 32) : make_uint4(0, 0, 0, 0);
+        } else {
+          b[buf][t][j].u = ok ? ld16(xrow[t] + kk + j * 32) : make_uint4(0, 0, 0, 0);
+        }
+      }
     }
   };
+
+  // NORMED: the norm's weights at this lane's places and the wavefront's first row of the
+  // residual stream are asked for before anything else, so that they are back (from the L2)
+  // and worked on while the first weights of W are still on their way from HBM.  (Loads at
+  // clamped places and values chosen afterwards: a load under a condition is a branch, and
+  // the compiler waits for it before the next.)
+  constexpr int HOLD = 8;
+  float g[NORMED ? HOLD : 1][2];
+  longlong2 v[NORMED ? HOLD : 1];
+  if constexpr (NORMED) {
+    if (wave < M) {
+      if (p.norm_bf16) {
+#pragma unroll
+        for (int i = 0; i < HOLD; ++i) {
+          const uint32_t u = *(const uint32_t*)((const bf16_t*)p.norm_w + min(i * 128 + lane * 2, K - 2));
+          g[i][0] = __uint_as_float(u << 16);
+          g[i][1] = __uint_as_float(u & 0xffff0000u);
+        }
+      } else {
+#pragma unroll
+        for (int i = 0; i < HOLD; ++i) {
+          const float2 u = *(const float2*)((const float*)p.norm_w + min(i * 128 + lane * 2, K - 2));
+          g[i][0] = u.x;
+          g[i][1] = u.y;
+        }
+      }
+#pragma unroll
+      for (int i = 0; i < HOLD; ++i)
+        v[i] = *(const longlong2*)(p.h64 + (size_t)wave * K + min(i * 128 + lane * 2, K - 2));
+    }
+  }
 
   int step = step_begin + wave;
   if (step < step_end) load_w(0, step);
@@ -257,6 +310,28 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
     }
   }
 
+  // SK_QKV: the bias of this lane's eight columns as well, in two loads (asked for one by one
+  // behind the products, each load waits for the one before it).
+  float bias_lo[4] = {0.f, 0.f, 0.f, 0.f}, bias_hi[4] = {0.f, 0.f, 0.f, 0.f};
+  if constexpr (EPI == SK_QKV) {
+    if (p.bias && wave == 0) {
+      const int at = n0 + g4 * 4, half = p.d / 2;
+      if (p.bias_bf16) {
+        const ushort4 l = *(const ushort4*)((const bf16_t*)p.bias + at);
+        const ushort4 h = *(const ushort4*)((const bf16_t*)p.bias + at + half);
+        bias_lo[0] = bf16_to_f32(l.x), bias_lo[1] = bf16_to_f32(l.y);
+        bias_lo[2] = bf16_to_f32(l.z), bias_lo[3] = bf16_to_f32(l.w);
+        bias_hi[0] = bf16_to_f32(h.x), bias_hi[1] = bf16_to_f32(h.y);
+        bias_hi[2] = bf16_to_f32(h.z), bias_hi[3] = bf16_to_f32(h.w);
+      } else {
+        const float4 l = *(const float4*)((const float*)p.bias + at);
+        const float4 h = *(const float4*)((const float*)p.bias + at + half);
+        bias_lo[0] = l.x, bias_lo[1] = l.y, bias_lo[2] = l.z, bias_lo[3] = l.w;
+        bias_hi[0] = h.x, bias_hi[1] = h.y, bias_hi[2] = h.z, bias_hi[3] = h.w;
+      }
+    }
+  }
+
   // SK_ACC: the values the result is added to are asked for now, by the wavefront that will
   // write them, so that the epilogue does not wait for them.
   const bool vec_out = (N & 3) == 0;
@@ -272,6 +347,45 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
                                              : make_float4(0.f, 0.f, 0.f, 0.f);
         }
     }
+  }
+
+  // NORMED: wavefront w makes rows w, w + WAVES, ...: a lane holds its two values of every
+  // 128 of the row (at most 1,024 wide: eight loads, all in flight at once; the norm's
+  // weights at the same places are shared by every row of the wavefront), adds up their
+  // squares, and leaves the normalised, weighted, rounded values in LDS.  The lane layout is
+  // the same whichever wavefront takes the row, so a row's x does not depend on the batch.
+  // The weights of W this wavefront multiplies first are on their way meanwhile.
+  if constexpr (NORMED) {
+#pragma unroll
+    for (int d = 1; d < DEPTH - 1; ++d)
+      if (step + d * WAVES < step_end) load_w(d, step + d * WAVES);
+    bf16_t* rows_out = (bf16_t*)skinny_rows;
+    for (int m = wave; m < M; m += WAVES) {
+      if (m != wave) {
+#pragma unroll
+        for (int i = 0; i < HOLD; ++i)
+          v[i] = *(const longlong2*)(p.h64 + (size_t)m * K + min(i * 128 + lane * 2, K - 2));
+      }
+      float f[HOLD][2], ss = 0.f;
+#pragma unroll
+      for (int i = 0; i < HOLD; ++i) {
+        const bool in = i * 128 + lane * 2 < K;
+        f[i][0] = in ? from_fixed(v[i].x) : 0.f;
+        f[i][1] = in ? from_fixed(v[i].y) : 0.f;
+        ss += f[i][0] * f[i][0] + f[i][1] * f[i][1];
+      }
+      const float rstd = rsqrtf(wave_sum(ss) / (float)K + p.norm_eps);
+#pragma unroll
+      for (int i = 0; i < HOLD; ++i) {
+        const int k0 = i * 128 + lane * 2;
+        if (k0 < K) {
+          *(uint32_t*)(rows_out + (size_t)m * made_stride + k0) =
+              pack_bf16x2(Elem<bf16_t>::round(f[i][0] * rstd) * g[i][0],
+                          Elem<bf16_t>::round(f[i][1] * rstd) * g[i][1]);
+        }
+      }
+    }
+    __syncthreads();
   }
 
   if (step < step_end) load_x(0, step);
@@ -307,7 +421,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
 #pragma unroll
     for (int d = 1; d < DEPTH - 1; ++d) {
       if (step + d * WAVES < step_end) {
-        load_w(d, step + d * WAVES);
+        if constexpr (!NORMED) load_w(d, step + d * WAVES);
         load_x(d, step + d * WAVES);
       }
     }
@@ -372,18 +486,27 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
       float lo[4], hi[4];
 #pragma unroll
       for (int i = 0; i < 4; ++i) {
-        lo[i] = acc[0][tb][i];
-        hi[i] = acc[1][tb][i];
-        if (p.bias) {
-          lo[i] += load_scalar(p.bias, p.bias_bf16, n0 + g4 * 4 + i);
-          hi[i] += load_scalar(p.bias, p.bias_bf16, n0 + half + g4 * 4 + i);
-        }
+        lo[i] = acc[0][tb][i] + bias_lo[i];
+        hi[i] = acc[1][tb][i] + bias_hi[i];
       }
       if constexpr (!EARLY_PLACE) {
         place[tb] = qkv_place(p, m);
         angles[tb] = qkv_angles(p, place[tb], head, dd);
       }
       qkv_store(p, place[tb], angles[tb], m, head, dd, lo, hi);
+    } else if constexpr (EPI == SK_FIXED) {
+      fixed_t* dst = (fixed_t*)p.out + (size_t)m * N;
+#pragma unroll
+      for (int ta = 0; ta < NT; ++ta) {
+        const int n = n0 + ta * 16 + g4 * 4;
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+          if (n + i >= N) continue;
+          float y = acc[ta][tb][i];
+          if (p.bias && slice == 0) y += load_scalar(p.bias, p.bias_bf16, n + i);
+          add_fixed(dst + n + i, y);
+        }
+      }
     } else {
       float* dst = (float*)p.out + ((size_t)(EPI == SK_PARTIAL ? slice : 0) * M + m) * N;
 #pragma unroll
@@ -462,16 +585,16 @@ extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
   return whole < 0.9 * split;
 }
 
-template <int NT, int EPI>
-static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream) {
+template <int NT, int EPI, bool NORMED = false, int WAVES = 0>
+static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream, size_t lds = 0) {
   // 8 wavefronts where the grid is small; with 3 or 4 tiles of x rows they would not fit
   // the register file.  More than 16 rows of x only for the q/k/v projection: the others
   // take the tiled kernel there.
-  constexpr int W = (EPI == SK_ACC || EPI == SK_QKV) ? 8 : SK_WAVES;
+  constexpr int W = WAVES ? WAVES : ((EPI == SK_ACC || EPI == SK_QKV || NORMED) ? 8 : SK_WAVES);
   const int tiles = (a.M + 15) / 16;
   if (tiles == 1) {
-    gemm_skinny_kernel<1, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a);
-  } else if constexpr (EPI == SK_QKV) {
+    gemm_skinny_kernel<1, NT, EPI, W, NORMED><<<grid, 64 * W, lds, stream>>>(a);
+  } else if constexpr (EPI == SK_QKV && !NORMED) {
     if (tiles == 2) gemm_skinny_kernel<2, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a);
     else if (tiles == 3) gemm_skinny_kernel<3, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a);
     else gemm_skinny_kernel<4, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a);
@@ -507,6 +630,29 @@ extern "C" int mk_linear_skinny(const void* x, const void* w, float* out, int M,
   return 0;
 }
 
+// h64[M, N] (the fixed-point residual stream) += x W^T (+ bias), 1 <= M <= 16, K in `slices`
+// slices as mk_linear_skinny takes them: no partial results are left, and the sum does not
+// depend on the order the slices finish in.
+extern "C" int mk_linear_skinny_fixed(const void* x, const void* w, const void* bias,
+                                      int bias_dtype, long long* h64, int M, int N, int K,
+                                      int slices, hipStream_t stream) {
+  MK_REQUIRE(M >= 1 && M <= 16, "skinny projection: M=%d outside 1..16", M);
+  MK_REQUIRE(N > 0 && K > 0 && K % 8 == 0, "skinny projection: K=%d must be a multiple of 8", K);
+  MK_REQUIRE(bias_dtype == MK_F32 || bias_dtype == MK_BF16, "skinny projection: bias dtype");
+  MK_REQUIRE(x && w && h64, "skinny projection: null argument");
+  const int steps = (K + 127) / 128;
+  MK_REQUIRE(slices >= 1 && slices <= steps && slices <= 65535,
+             "skinny projection: %d slices for %d steps", slices, steps);
+  const int per = (steps + slices - 1) / slices;
+  MK_REQUIRE((per * (slices - 1)) < steps, "skinny projection: an empty slice");
+  SkinnyArgs a = skinny_args(x, w, h64, M, N, K, per);
+  a.bias = bias;
+  a.bias_bf16 = bias_dtype == MK_BF16;
+  launch_skinny<2, SK_FIXED>(a, dim3((N + 31) / 32, slices), stream);
+  MK_LAUNCH_CHECK("linear_skinny_fixed");
+  return 0;
+}
+
 // out[M, N] (float32) += x W^T (+ bias), 1 <= M <= 16, all of K in each workgroup.
 extern "C" int mk_linear_skinny_acc(const void* x, const void* w, const void* bias,
                                     int bias_dtype, float* out, int M, int N, int K,
@@ -538,16 +684,56 @@ extern "C" int mk_gated_skinny(const void* x, const void* w, void* act, int M, i
   return 0;
 }
 
+// The widest row (K) the projections below take for M rows: the rows they make live in LDS.
+extern "C" int mk_skinny_normed_max_k(int M) {
+  if (M < 1 || M > 16) return 0;
+  const int fits = ((48 * 1024) / (2 * M) - 8) / 8 * 8;
+  return fits < 1024 ? fits : 1024;   // a lane holds its share of a row in registers
+}
+
+static int set_normed(SkinnyArgs& a, const long long* h64, const void* norm_w, int norm_dtype,
+                      float eps) {
+  MK_REQUIRE(h64 && norm_w, "normed projection: null argument");
+  MK_REQUIRE(norm_dtype == MK_F32 || norm_dtype == MK_BF16, "normed projection: weight dtype");
+  MK_REQUIRE(a.M >= 1 && a.M <= 16 && a.K <= mk_skinny_normed_max_k(a.M),
+             "normed projection: %d rows of %d are more than its workgroups hold (K <= %d)", a.M,
+             a.K, mk_skinny_normed_max_k(a.M));
+  a.h64 = (const fixed_t*)h64;
+  a.norm_w = norm_w;
+  a.norm_bf16 = norm_dtype == MK_BF16;
+  a.norm_eps = eps;
+  return 0;
+}
+
+static size_t normed_lds(const SkinnyArgs& a) { return (size_t)a.M * (a.K + 8) * 2; }
+
+// mk_gated_skinny on x = rmsnorm(h64) * norm_w, made by every workgroup for itself from the
+// fixed-point residual stream h64 [M, K].
+extern "C" int mk_gated_skinny_normed(const long long* h64, const void* norm_w, int norm_dtype,
+                                      float eps, const void* w, void* act, int M, int inter, int K,
+                                      hipStream_t stream) {
+  MK_REQUIRE(inter > 0 && K > 0 && K % 8 == 0, "gated projection: K=%d must be a multiple of 8",
+             K);
+  MK_REQUIRE(w && act, "gated projection: null argument");
+  SkinnyArgs a = skinny_args(nullptr, w, act, M, inter, K, (K + 127) / 128);
+  if (set_normed(a, h64, norm_w, norm_dtype, eps)) return 1;
+  if (M <= 4) launch_skinny<2, SK_GATED, true, 4>(a, dim3((inter + 15) / 16, 1), stream, normed_lds(a));
+  else launch_skinny<2, SK_GATED, true, 8>(a, dim3((inter + 15) / 16, 1), stream, normed_lds(a));
+  MK_LAUNCH_CHECK("gated_skinny_normed");
+  return 0;
+}
+
 // The q/k/v projection of 1 <= M <= 64 tokens with everything that follows it: bias, rotation
 // of q and k by the token's position (full head width, or none), q [M, n_q d] out, k and v
 // into the paged cache (n_kv = 0: queries only).  W is [(n_q + 2 n_kv) d, K].
 // Formulas: reference mercury/model/qwen2.py:57-64, mercury/model/rope.py:19-29.
-extern "C" int mk_qkv_skinny(const void* x, const void* w, const void* bias, int bias_dtype,
-                             void* q_out, const float* cos_table, const float* sin_table,
-                             int table_positions, const int* positions, const int* token_seq,
-                             const int* block_table, int table_stride, void* k_cache,
-                             void* v_cache, int page_size, int n_q, int n_kv, int d, int rotate,
-                             int M, int K, hipStream_t stream) {
+static int qkv_skinny_any(const void* x, const long long* h64, const void* norm_w, int norm_dtype,
+                          float eps, const void* w, const void* bias, int bias_dtype,
+                          void* q_out, const float* cos_table, const float* sin_table,
+                          int table_positions, const int* positions, const int* token_seq,
+                          const int* block_table, int table_stride, void* k_cache,
+                          void* v_cache, int page_size, int n_q, int n_kv, int d, int rotate,
+                          int M, int K, hipStream_t stream) {
   MK_REQUIRE(M >= 1 && M <= 64, "qkv projection: M=%d outside 1..64", M);
   MK_REQUIRE(n_q > 0 && n_kv >= 0 && d > 0 && d % 32 == 0,
              "qkv projection: head size %d is not a multiple of 32", d);
@@ -576,9 +762,44 @@ extern "C" int mk_qkv_skinny(const void* x, const void* w, const void* bias, int
   a.d = d;
   a.rotate = rotate;
   const dim3 grid((n_q + 2 * n_kv) * (d / 32), 1);
-  launch_skinny<2, SK_QKV>(a, grid, stream);
+  if (h64) {
+    if (set_normed(a, h64, norm_w, norm_dtype, eps)) return 1;
+    launch_skinny<2, SK_QKV, true>(a, grid, stream, normed_lds(a));
+  } else {
+    MK_REQUIRE(x, "qkv projection: null argument");
+    launch_skinny<2, SK_QKV>(a, grid, stream);
+  }
   MK_LAUNCH_CHECK("qkv_skinny");
   return 0;
+}
+
+extern "C" int mk_qkv_skinny(const void* x, const void* w, const void* bias, int bias_dtype,
+                             void* q_out, const float* cos_table, const float* sin_table,
+                             int table_positions, const int* positions, const int* token_seq,
+                             const int* block_table, int table_stride, void* k_cache,
+                             void* v_cache, int page_size, int n_q, int n_kv, int d, int rotate,
+                             int M, int K, hipStream_t stream) {
+  return qkv_skinny_any(x, nullptr, nullptr, MK_F32, 0.f, w, bias, bias_dtype, q_out, cos_table,
+                        sin_table, table_positions, positions, token_seq, block_table,
+                        table_stride, k_cache, v_cache, page_size, n_q, n_kv, d, rotate, M, K,
+                        stream);
+}
+
+// mk_qkv_skinny on x = rmsnorm(h64) * norm_w, made by every workgroup for itself from the
+// fixed-point residual stream h64 [M, K]; at most 16 tokens.
+extern "C" int mk_qkv_skinny_normed(const long long* h64, const void* norm_w, int norm_dtype,
+                                    float eps, const void* w, const void* bias, int bias_dtype,
+                                    void* q_out, const float* cos_table, const float* sin_table,
+                                    int table_positions, const int* positions,
+                                    const int* token_seq, const int* block_table,
+                                    int table_stride, void* k_cache, void* v_cache, int page_size,
+                                    int n_q, int n_kv, int d, int rotate, int M, int K,
+                                    hipStream_t stream) {
+  MK_REQUIRE(h64, "qkv projection: null argument");
+  return qkv_skinny_any(nullptr, h64, norm_w, norm_dtype, eps, w, bias, bias_dtype, q_out,
+                        cos_table, sin_table, table_positions, positions, token_seq, block_table,
+                        table_stride, k_cache, v_cache, page_size, n_q, n_kv, d, rotate, M, K,
+                        stream);
 }
 
 // ------------------------------------------------------------------------------- tiled
@@ -857,9 +1078,39 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
     }
     return;
   }
+  // The bias of this lane's columns, asked for in one go and at clamped places (a load under
+  // a condition is a branch that the compiler waits behind before the next load).
+  float col_bias[EPI == EPI_GATED ? 1 : TN][4];
+  if constexpr (EPI != EPI_GATED) {
+#pragma unroll
+    for (int tb = 0; tb < TN; ++tb)
+#pragma unroll
+      for (int i = 0; i < 4; ++i) col_bias[tb][i] = 0.f;
+    if (bias != nullptr) {
+#pragma unroll
+      for (int tb = 0; tb < TN; ++tb)
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+          col_bias[tb][i] = Elem<TBIAS>::load(bias + min(n0 + wn + tb * 16 + g4 * 4 + i, N - 1));
+    }
+  }
 #pragma unroll
   for (int ta = 0; ta < TM; ++ta) {
     const int m = m0 + wm + ta * 16 + r;
+    // EPI_ACC: the values a row tile's results are added to, all of the tile's loads in
+    // flight at once (one by one, each behind the store before it, a wavefront makes TM x TN
+    // trips to memory in a row).  Rows and columns past the end read a clamped place that
+    // nothing is made of.
+    float4 old[EPI == EPI_ACC ? TN : 1];
+    const bool old_held = EPI == EPI_ACC && (ldo & 3) == 0 && N >= 4;
+    if constexpr (EPI == EPI_ACC) {
+      if (old_held) {
+        const float* row = (const float*)out_ + (size_t)min(m, M - 1) * ldo;
+#pragma unroll
+        for (int tb = 0; tb < TN; ++tb)
+          old[tb] = *(const float4*)(row + min(n0 + wn + tb * 16 + g4 * 4, (N - 4) & ~3));
+      }
+    }
     if (m >= M) continue;
     if (EPI == EPI_GATED) {
 #pragma unroll
@@ -888,10 +1139,7 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
       const int n = n0 + wn + tb * 16 + g4 * 4;
       float v[4];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        v[i] = acc[ta][tb][i];
-        if (bias != nullptr && n + i < N) v[i] += Elem<TBIAS>::load(bias + n + i);
-      }
+      for (int i = 0; i < 4; ++i) v[i] = acc[ta][tb][i] + col_bias[tb][i];
       const bool whole = n + 3 < N && (ldo & 3) == 0;
       if (EPI == EPI_BF16) {
         bf16_t* dst = (bf16_t*)out_ + (size_t)m * ldo + n;
@@ -906,12 +1154,11 @@ __global__ __launch_bounds__(64 * WM * WN) void gemm_tiled_kernel(const bf16_t* 
         float* dst = (float*)out_ + (size_t)m * ldo + n;
         if (whole) {
           float4 o = make_float4(v[0], v[1], v[2], v[3]);
-          if (EPI == EPI_ACC) {
-            const float4 old = *(const float4*)dst;
-            o.x += old.x;
-            o.y += old.y;
-            o.z += old.z;
-            o.w += old.w;
+          if constexpr (EPI == EPI_ACC) {
+            o.x += old[tb].x;
+            o.y += old[tb].y;
+            o.z += old[tb].z;
+            o.w += old[tb].w;
           }
           *(float4*)dst = o;
         } else {

@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 19
+#define MK_ABI_VERSION 20
 
 #ifdef __cplusplus
 extern "C" {
@@ -24,6 +24,19 @@ int mk_abi_version();
 // out[t, :] = table[ids[t], :] * scale as float32 (the residual stream starts here).
 int mk_embed(const int* ids, const void* table, int dtype, float* out, int tokens, int hidden,
              int vocab, float scale, hipStream_t stream);
+
+// The residual stream of a step of few tokens in fixed point: 64-bit integers in units of
+// 2^-32, into which projections add their results with integer atomics (the sum is the same
+// in whatever order they arrive, and nothing has to add partial results up afterwards).
+// mk_embed_fixed starts it; mk_rmsnorm_fixed normalises rows of it as mk_rmsnorm does rows of
+// h; mk_fixed_add adds `count` float32 partial sums p[k * stride + i], i < n, into it.
+int mk_embed_fixed(const int* ids, const void* table, int dtype, long long* out, int tokens,
+                   int hidden, int vocab, float scale, hipStream_t stream);
+int mk_rmsnorm_fixed(const long long* h64, const void* weight, int weight_dtype, float eps,
+                     const int* rows, void* out, int out_dtype, int out_rows, int hidden,
+                     hipStream_t stream);
+int mk_fixed_add(long long* h64, const float* partials, int count, long long stride, long long n,
+                 hipStream_t stream);
 
 // logits[i] = cap * tanh(logits[i] / cap) for i < count, in place.
 int mk_logit_cap(float* logits, long long count, float cap, hipStream_t stream);
@@ -105,10 +118,28 @@ int mk_linear_skinny_unsplit(int M, int N, int K);
 int mk_linear_skinny_acc(const void* x, const void* w, const void* bias, int bias_dtype,
                          float* out, int M, int N, int K, hipStream_t stream);
 
+// h64[M, N] (the fixed-point residual stream, see mk_embed_fixed) += x W^T (+ bias) for
+// 1 <= M <= 16, K in `slices` slices as mk_linear_skinny takes them.
+int mk_linear_skinny_fixed(const void* x, const void* w, const void* bias, int bias_dtype,
+                           long long* h64, int M, int N, int K, int slices, hipStream_t stream);
+
 // act[M, inter] (bfloat16) = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, K],
 // 1 <= M <= 16.
 int mk_gated_skinny(const void* x, const void* w, void* act, int M, int inter, int K,
                     hipStream_t stream);
+
+// The gated and the q/k/v projection of at most 16 rows on x = rmsnorm(h64) * norm_w, which
+// every workgroup makes for itself from the fixed-point residual stream h64 [M, K] (the norm
+// needs no kernel of its own); K at most mk_skinny_normed_max_k(M).
+int mk_skinny_normed_max_k(int M);
+int mk_gated_skinny_normed(const long long* h64, const void* norm_w, int norm_dtype, float eps,
+                           const void* w, void* act, int M, int inter, int K, hipStream_t stream);
+int mk_qkv_skinny_normed(const long long* h64, const void* norm_w, int norm_dtype, float eps,
+                         const void* w, const void* bias, int bias_dtype, void* q_out,
+                         const float* cos_table, const float* sin_table, int table_positions,
+                         const int* positions, const int* token_seq, const int* block_table,
+                         int table_stride, void* k_cache, void* v_cache, int page_size, int n_q,
+                         int n_kv, int d, int rotate, int M, int K, hipStream_t stream);
 
 // The q/k/v projection of 1 <= M <= 64 tokens, w = [(n_q + 2 n_kv) d, K], with bias, rotation
 // of q and k over the whole head (rotate != 0), q [M, n_q d] out and k, v written to the
@@ -202,8 +233,9 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
 // sequence (tile = token, M of them): out[slice, M, N] are float32 partial sums over slices of
 // heads_per_slice query heads each (mk_attention_out_heads_per_slice: how many, 0 where the
 // sizes are not taken; mk_attention_out_max_parts: the most partial results per (tile, kv head)
-// it takes), to be added up by whoever consumes the projection.  wide: 128 rows of w_o per
-// workgroup instead of 64.
+// it takes), to be added up by whoever consumes the projection; or, with `out` null, the
+// result is added into the fixed-point residual stream fixed_out [M, N] (see mk_embed_fixed).
+// wide: 128 rows of w_o per workgroup instead of 64.
 int mk_attention_mfma_parts_written(int rows_per_tile, int num_splits, int d);
 int mk_attention_mfma_parts(const void* q, int q_stride, const void* k_cache, const void* v_cache,
                             const int* tile_seq, const int* tile_row0, int num_tiles,
@@ -214,8 +246,8 @@ int mk_attention_mfma_parts(const void* q, int q_stride, const void* k_cache, co
 int mk_attention_out_heads_per_slice(int n_q, int n_kv, int d, int M, int N);
 int mk_attention_out_max_parts(int M, int heads_per_slice);
 int mk_attention_out(const float* part_o, const float* part_ml, int parts, const void* w_o,
-                     float* out, int M, int N, int n_q, int n_kv, int d, int heads_per_slice,
-                     int wide, hipStream_t stream);
+                     float* out, long long* fixed_out, int M, int N, int n_q, int n_kv, int d,
+                     int heads_per_slice, int wide, hipStream_t stream);
 
 // @library core
 

@@ -285,7 +285,7 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
                                        a.page_size, a.n_q, a.n_kv, d, a.scale, a.window, plan.rows,
                                        plan.splits, plan.split_blocks, part_o, part_ml, l.stream()),
              "attention");
-  check_mfma(t.mk_attention_out(part_o, part_ml, written, w_o, out, m, hidden, a.n_q, a.n_kv, d,
+  check_mfma(t.mk_attention_out(part_o, part_ml, written, w_o, out, nullptr, m, hidden, a.n_q, a.n_kv, d,
                                 heads_per_slice, wide ? 1 : 0, l.stream()), "attention_out");
 }
 
