@@ -624,30 +624,64 @@ __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_pa
   const int width = (n_q + 2 * n_kv) * d;
   const int col0 = head0 * d;
   const float* row = partials + (size_t)t * width + col0;
-  if ((d & 3) == 0 && (partial_stride & 3) == 0) {
+  // Where the token's keys and values go, and by what this thread's first value turns: asked
+  // for now, beside the partial sums, and not in a chain of trips to memory behind them.
+  int page = -1, off = 0;
+  const int page_size = 1 << page_shift;
+  if (write_kv) {
+    page = block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)];
+    off = pos & (page_size - 1);
+  }
+  float first_c = 1.f, first_s = 0.f;
+  if (rot > 0) {
+    const int j = min((int)threadIdx.x, count - 1) % d;
+    const int jj = min(j < half ? j : j - half, half - 1);
+    first_c = cs[jj];
+    first_s = sn[jj];
+  }
+  if ((d & 3) == 0 && (partial_stride & 3) == 0 &&
+      (bias == nullptr || (uintptr_t)bias % 16 == 0)) {
     for (int i = threadIdx.x * 4; i < count; i += blockDim.x * 4) {
+      float o[4] = {0.f, 0.f, 0.f, 0.f};
+      if (bias) {
+        if constexpr (sizeof(TB) == 2) {
+          const ushort4 b = *(const ushort4*)(bias + col0 + i);
+          o[0] = bf16_to_f32(b.x), o[1] = bf16_to_f32(b.y), o[2] = bf16_to_f32(b.z), o[3] = bf16_to_f32(b.w);
+        } else {
+          const float4 b = *(const float4*)(bias + col0 + i);
+          o[0] = b.x, o[1] = b.y, o[2] = b.z, o[3] = b.w;
+        }
+      }
+      // Up to sixteen slices' loads in flight at once (at clamped places: a load under a
+      // condition is a branch the next load waits behind); the additions in the order of
+      // sum_partials: fours as (a + b) + (c + d), then what is left one by one.
       float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
-      int k = 0;   // the order of sum_partials, four values at a time
-      for (; k + 4 <= num_partials; k += 4) {
-        const float4 a = *(const float4*)(row + i + (size_t)k * partial_stride);
-        const float4 b = *(const float4*)(row + i + (size_t)(k + 1) * partial_stride);
-        const float4 c = *(const float4*)(row + i + (size_t)(k + 2) * partial_stride);
-        const float4 e = *(const float4*)(row + i + (size_t)(k + 3) * partial_stride);
-        v.x += (a.x + b.x) + (c.x + e.x);
-        v.y += (a.y + b.y) + (c.y + e.y);
-        v.z += (a.z + b.z) + (c.z + e.z);
-        v.w += (a.w + b.w) + (c.w + e.w);
-      }
-      for (; k < num_partials; ++k) {
-        const float4 a = *(const float4*)(row + i + (size_t)k * partial_stride);
-        v.x += a.x, v.y += a.y, v.z += a.z, v.w += a.w;
-      }
-      float o[4] = {v.x, v.y, v.z, v.w};
+      for (int k0 = 0; k0 < num_partials; k0 += 16) {
+        float4 part[16];
 #pragma unroll
-      for (int u = 0; u < 4; ++u) {
-        if (bias) o[u] += Elem<TB>::load(bias + col0 + i + u);
-        vals[i + u] = Elem<T>::round(o[u]);
+        for (int j = 0; j < 16; ++j)
+          part[j] = *(const float4*)(row + i + (size_t)min(k0 + j, num_partials - 1) * partial_stride);
+#pragma unroll
+        for (int j = 0; j < 16; j += 4) {
+          if (k0 + j + 4 <= num_partials) {
+            v.x += (part[j].x + part[j + 1].x) + (part[j + 2].x + part[j + 3].x);
+            v.y += (part[j].y + part[j + 1].y) + (part[j + 2].y + part[j + 3].y);
+            v.z += (part[j].z + part[j + 1].z) + (part[j + 2].z + part[j + 3].z);
+            v.w += (part[j].w + part[j + 1].w) + (part[j + 2].w + part[j + 3].w);
+          } else {
+#pragma unroll
+            for (int u = 0; u < 4; ++u) {
+              if (k0 + j + u < num_partials) {
+                v.x += part[j + u].x, v.y += part[j + u].y, v.z += part[j + u].z, v.w += part[j + u].w;
+              }
+            }
+          }
+        }
       }
+      vals[i] = Elem<T>::round(v.x + o[0]);
+      vals[i + 1] = Elem<T>::round(v.y + o[1]);
+      vals[i + 2] = Elem<T>::round(v.z + o[2]);
+      vals[i + 3] = Elem<T>::round(v.w + o[3]);
     }
   } else {
     for (int i = threadIdx.x; i < count; i += blockDim.x) {
@@ -658,26 +692,22 @@ __global__ void qkv_finish_kernel(const float* __restrict__ partials, int num_pa
   }
   __syncthreads();
 
-  auto rotated = [&](int base, int j) {
-    if (j < half) return vals[base + j] * cs[j] - vals[base + j + half] * sn[j];
-    if (j < rot) return vals[base + j] * cs[j - half] + vals[base + j - half] * sn[j - half];
-    return vals[base + j];
+  auto rotated = [&](int base, int j, bool first) {
+    if (j >= rot) return vals[base + j];
+    const int jj = j < half ? j : j - half;
+    const float c = first ? first_c : cs[jj], sine = first ? first_s : sn[jj];
+    if (j < half) return vals[base + j] * c - vals[base + j + half] * sine;
+    return vals[base + j] * c + vals[base + j - half] * sine;
   };
-  int page = -1, off = 0;
-  const int page_size = 1 << page_shift;
-  if (write_kv) {
-    page = block_table[(size_t)token_seq[t] * table_stride + (pos >> page_shift)];
-    off = pos & (page_size - 1);
-  }
   for (int i = threadIdx.x; i < count; i += blockDim.x) {
     const int local = i / d, j = i - local * d, head = head0 + local;
     if (head < n_q) {
-      Elem<T>::store(q_out + ((size_t)t * n_q + head) * d + j, rotated(local * d, j));
+      Elem<T>::store(q_out + ((size_t)t * n_q + head) * d + j, rotated(local * d, j, i == (int)threadIdx.x));
     } else if (page >= 0) {
       if (head < n_q + n_kv) {
         const int kh = head - n_q;
         Elem<T>::store(k_cache + (((size_t)page * n_kv + kh) * page_size + off) * d + j,
-                       rotated(local * d, j));
+                       rotated(local * d, j, i == (int)threadIdx.x));
       } else {
         const int vh = head - n_q - n_kv;
         Elem<T>::store(v_cache + (((size_t)page * n_kv + vh) * d + j) * page_size + off, vals[i]);
