@@ -694,6 +694,8 @@ extern "C" int mk_skinny_normed_max_k(int M) {
 static int set_normed(SkinnyArgs& a, const long long* h64, const void* norm_w, int norm_dtype,
                       float eps) {
   MK_REQUIRE(h64 && norm_w, "normed projection: null argument");
+  MK_REQUIRE((uintptr_t)h64 % 16 == 0 && (uintptr_t)norm_w % 8 == 0,
+             "normed projection: the residual stream must be 16-byte aligned, the norm's weights 8");
   MK_REQUIRE(norm_dtype == MK_F32 || norm_dtype == MK_BF16, "normed projection: weight dtype");
   MK_REQUIRE(a.M >= 1 && a.M <= 16 && a.K <= mk_skinny_normed_max_k(a.M),
              "normed projection: %d rows of %d are more than its workgroups hold (K <= %d)", a.M,
@@ -743,6 +745,7 @@ static int qkv_skinny_any(const void* x, const long long* h64, const void* norm_
   MK_REQUIRE(n_kv == 0 || (k_cache && v_cache && block_table && mk_is_pow2(page_size)),
              "qkv projection: the cache and a power-of-two page size are required");
   MK_REQUIRE(bias_dtype == MK_F32 || bias_dtype == MK_BF16, "qkv projection: bias dtype");
+  MK_REQUIRE((uintptr_t)bias % 16 == 0, "qkv projection: the bias must be 16-byte aligned");
   const int N = (n_q + 2 * n_kv) * d;
   SkinnyArgs a = skinny_args(x, w, nullptr, M, N, K, (K + 127) / 128);
   a.bias = bias;

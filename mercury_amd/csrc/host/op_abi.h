@@ -14,6 +14,12 @@
  *   pending  float32 [pending_count, T, hidden]  partial sums the previous operation left for
  *                                  this one to add into h
  *   logits   float32 [R, vocab]    the step's result; the operation that fills it says so
+ * A step of a few tokens may keep the residual stream in fixed point instead: `h` is then NULL
+ * and `h_fixed` holds it as 64-bit integers in units of 2^-32, into which operations add their
+ * results with integer atomics (no partial sums are left, `pending` stays empty).  A norm may
+ * then leave its work to the operation behind it: `x` is NULL though `x_live` is set, and
+ * `norm_weight` / `norm_eps` say what x would have been (rmsnorm(h_fixed) * weight).  Only
+ * programs whose every operation is of a kind flagged MK_OP_FIXED_STREAM are run this way.
  * x and pending live in the previous operation's arena, so they are alive for exactly one
  * operation: `x_live` / `pending_count` say whether the previous operation produced them.  An
  * operation that produces them for the next sets `out_*`.
@@ -81,6 +87,17 @@ typedef struct mk_op_context {
   void* (*alloc)(void* arena, size_t bytes);
   /* a message for a non-zero return */
   char error[512];
+  /* the residual stream in fixed point (then h is NULL), and the norm the operation before
+     left for this one to do (then x is NULL and x_live set); out_norm_*: the same for the
+     operation behind this one, with out_x NULL and out_x_live set */
+  int stream_fixed;        /* set in a dry walk too, where h_fixed is NULL like every pointer */
+  long long* h_fixed;
+  const void* norm_weight;
+  int norm_weight_dtype;
+  float norm_eps;
+  const void* out_norm_weight;
+  int out_norm_weight_dtype;
+  float out_norm_eps;
 } mk_op_context;
 
 /* What the shape of a step is before it is packed: enough to say which tile lists an
@@ -104,8 +121,10 @@ typedef int (*mk_op_tiles_fn)(const void* params, const mk_step_shape* shape, mk
 /* Flags of an operation kind: what it expects of the operation before it. */
 enum {
   MK_OP_READS_X = 1,        /* needs a live x */
-  MK_OP_FOLDS_PENDING = 2   /* adds live partial sums into h; without it, live partial sums
+  MK_OP_FOLDS_PENDING = 2,  /* adds live partial sums into h; without it, live partial sums
                                before this operation are an error (they would be lost) */
+  MK_OP_FIXED_STREAM = 4    /* also works on a residual stream in fixed point (h_fixed) and
+                               on an x left undone as a norm (norm_weight) */
 };
 
 #ifdef __cplusplus

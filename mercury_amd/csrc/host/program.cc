@@ -84,6 +84,16 @@ void Program::append_caller_step(int index, bool gives_x) {
 
 std::string Program::kind_of(size_t i) const { return entries_.at(i).kind.name; }
 
+bool Program::fixed_stream(int num_tokens) const {
+  const OpRegistry& registry = OpRegistry::instance();
+  if (num_tokens < 1 || entries_.empty()) return false;
+  for (const Entry& e : entries_) {
+    if (!e.kind.run || !(e.kind.flags & MK_OP_FIXED_STREAM)) return false;
+  }
+  if (registry.fixed_stream_limit >= 0) return num_tokens <= registry.fixed_stream_limit;
+  return registry.fixed_stream_tokens && num_tokens <= registry.fixed_stream_tokens(dtype_, hidden_);
+}
+
 std::vector<Program::TileNeed> Program::tile_needs(const std::vector<int>& counts, int max_q_len,
                                                    int max_kv_len) const {
   std::vector<TileNeed> out;
@@ -111,9 +121,11 @@ void* arena_alloc(void* arena, size_t bytes) { return static_cast<Arena*>(arena)
 void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes, void* stream,
                    RunState& state, bool dry, WorkspaceNeed* need) const {
   auto round = [](size_t b) { return (b + 255) & ~(size_t)255; };
-  const size_t h_bytes = round((size_t)step.num_tokens * hidden_ * 4);
+  const bool own = state.own_h != nullptr || state.own_stream;
+  const bool fixed = !own && state.begin == 0 && state.x == nullptr && state.x_rows == 0 &&
+                     fixed_stream(step.num_tokens);
+  const size_t h_bytes = round((size_t)step.num_tokens * hidden_ * (fixed ? 8 : 4));
   const size_t logit_bytes = round((size_t)step.num_rows * vocab_ * 4);
-  const bool own = state.own_h != nullptr;
   const size_t persistent = own ? 0 : h_bytes + logit_bytes;
   Arena arenas[2];
   if (dry) {
@@ -154,7 +166,9 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
   ctx.dtype = dtype_;
   ctx.hidden = hidden_;
   ctx.vocab = vocab_;
-  ctx.h = dry ? nullptr : (own ? state.own_h : (float*)workspace);
+  ctx.h = dry || fixed ? nullptr : (own ? state.own_h : (float*)workspace);
+  ctx.stream_fixed = fixed ? 1 : 0;
+  ctx.h_fixed = dry || !fixed ? nullptr : (long long*)workspace;
   ctx.logits = dry ? nullptr : (own ? state.own_logits : (float*)(workspace + h_bytes));
   ctx.alloc = &arena_alloc;
   state.h = ctx.h;
@@ -166,6 +180,9 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
   bool x_live = state.x != nullptr || (dry && state.x_rows > 0);
   const float* pending = state.pending;
   int pending_count = state.pending_count;
+  const void* norm_weight = nullptr;   // a norm left to the next operation (fixed point only)
+  int norm_weight_dtype = 0;
+  float norm_eps = 0.f;
 
   int i = state.begin;
   for (; i < (int)entries_.size(); ++i) {
@@ -188,6 +205,12 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
     ctx.x_live = x_live ? 1 : 0;
     ctx.pending = pending;
     ctx.pending_count = pending_count;
+    ctx.norm_weight = x_live ? norm_weight : nullptr;
+    ctx.norm_weight_dtype = norm_weight_dtype;
+    ctx.norm_eps = norm_eps;
+    ctx.out_norm_weight = nullptr;
+    ctx.out_norm_weight_dtype = 0;
+    ctx.out_norm_eps = 0.f;
     ctx.out_x = nullptr;
     ctx.out_x_rows = 0;
     ctx.out_x_live = 0;
@@ -206,6 +229,13 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
     x_live = ctx.out_x_live != 0;
     pending = ctx.out_pending;
     pending_count = ctx.out_pending_count;
+    norm_weight = ctx.out_norm_weight;
+    norm_weight_dtype = ctx.out_norm_weight_dtype;
+    norm_eps = ctx.out_norm_eps;
+    if (norm_weight && !fixed) {
+      throw KernelError("operation " + std::to_string(i) + " ('" + e.kind.name +
+                        "') left a norm undone outside a step in fixed point");
+    }
     if (ctx.out_logits_ready) state.logits = ctx.logits;
   }
   state.stopped_at = i;
@@ -219,9 +249,10 @@ void Program::walk(const StepView& step, char* workspace, size_t workspace_bytes
   }
 }
 
-WorkspaceNeed Program::measure(const StepView& step, int given_x_rows) const {
+WorkspaceNeed Program::measure(const StepView& step, int given_x_rows, bool own_stream) const {
   WorkspaceNeed need;
   RunState state;
+  state.own_stream = own_stream;
   int begin = 0;
   // every stretch between caller-run steps; behind such a step, x is there if it says so and
   // partial sums may or may not be (an operation that adds them up takes none as well)

@@ -43,6 +43,12 @@ class OpRegistry {
   const OpKind& get(const std::string& name) const;
   bool has(const std::string& name) const { return kinds_.count(name) != 0; }
   std::vector<std::string> names() const;
+  // Up to how many tokens a step of a model of this dtype and width keeps its residual
+  // stream in fixed point (op_abi.h), 0 for never: set by whoever registers operations that
+  // can (the rule depends on their kernels); null: never.
+  int (*fixed_stream_tokens)(int dtype, int hidden) = nullptr;
+  // >= 0: that many tokens whatever the rule says (0: never), for tests and for comparing.
+  int fixed_stream_limit = -1;
 
  private:
   std::map<std::string, OpKind> kinds_;
@@ -94,6 +100,7 @@ struct RunState {
   // operation run on tensors that exist already); the workspace is then all arena
   float* own_h = nullptr;
   float* own_logits = nullptr;
+  bool own_stream = false;      // a dry walk for such a run (own_h is null there like every pointer)
   // out: the entry the walk stopped before (size() when it ran to the end), and the
   // registers as they stand there
   int stopped_at = 0;
@@ -120,6 +127,9 @@ class Program {
   void append_caller_step(int index, bool gives_x);
 
   size_t size() const { return entries_.size(); }
+  // Whether a step of this many tokens runs on a residual stream in fixed point: every entry
+  // an operation of a kind that can, and few enough tokens for the registry's rule.
+  bool fixed_stream(int num_tokens) const;
   // The kind's name, or "host" for a caller-run step.
   std::string kind_of(size_t i) const;
   int caller_index(size_t i) const { return entries_.at(i).caller_index; }
@@ -134,7 +144,8 @@ class Program {
   // Walk without launching: what a step of this shape needs of its workspace.  Throws when
   // the operations do not fit together.  given_x_rows > 0: the caller brings an x of that
   // many rows for the first operation (a program that is one operation of a model).
-  WorkspaceNeed measure(const StepView& step, int given_x_rows = 0) const;
+  // own_stream: for a run on a residual stream of the caller's own.
+  WorkspaceNeed measure(const StepView& step, int given_x_rows = 0, bool own_stream = false) const;
   // Walk from state.begin until the end or a caller-run step.  `workspace` must hold
   // measure(step).total() bytes.
   void run(const StepView& step, char* workspace, size_t workspace_bytes, void* stream,

@@ -79,6 +79,16 @@ void bind_program(py::module_& m) {
   }, "Sizes and a few offsets of the structures of op_abi.h, for mirrors of them to check.");
   m.attr("OP_READS_X") = (int)MK_OP_READS_X;
   m.attr("OP_FOLDS_PENDING") = (int)MK_OP_FOLDS_PENDING;
+  m.attr("OP_FIXED_STREAM") = (int)MK_OP_FIXED_STREAM;
+  m.def("set_fixed_stream_limit", [](int limit) {
+    OpRegistry& r = OpRegistry::instance();
+    const int before = r.fixed_stream_limit;
+    r.fixed_stream_limit = limit;
+    return before;
+  }, py::arg("limit"),
+        "Steps of up to `limit` tokens keep their residual stream in fixed point where every "
+        "operation of the program can (0: none do; negative: the kernels' own rule).  Returns "
+        "the limit set before.");
 
   m.def("build_tiles", [](const std::vector<int>& counts, int group, int tile_rows) {
     std::vector<int> seq, row0;
@@ -113,15 +123,18 @@ void bind_program(py::module_& m) {
         }
         return out;
       })
+      .def("fixed_stream", [](const Program& p, int num_tokens) { return p.fixed_stream(num_tokens); },
+           py::arg("num_tokens"),
+           "Whether a step of this many tokens keeps its residual stream in fixed point.")
       .def("workspace_bytes", [](const Program& p, const PackedStep& step) {
         return p.measure(step.view(nullptr)).total();
       })
       .def("workspace_bytes_for", [](const Program& p, const std::vector<int>& counts, int num_rows,
-                                     int max_kv_len, int num_groups, int x_rows) {
-        return p.measure(StepView::shape_only(counts, num_rows, max_kv_len, num_groups), x_rows)
-            .total();
+                                     int max_kv_len, int num_groups, int x_rows, bool own_stream) {
+        return p.measure(StepView::shape_only(counts, num_rows, max_kv_len, num_groups), x_rows,
+                         own_stream).total();
       }, py::arg("counts"), py::arg("num_rows"), py::arg("max_kv_len"), py::arg("num_groups") = 1,
-           py::arg("x_rows") = 0,
+           py::arg("x_rows") = 0, py::arg("own_stream") = false,
            "What a step of this shape (tokens per sequence, wanted rows, longest sequence) needs "
            "of its workspace; also the check that the operations fit together.")
       .def("run", [](const Program& p, const PackedStep& step, uintptr_t ints, uintptr_t workspace,

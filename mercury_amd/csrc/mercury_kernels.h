@@ -10,7 +10,7 @@
 
 #include <hip/hip_runtime.h>
 
-#define MK_ABI_VERSION 20
+#define MK_ABI_VERSION 21
 
 #ifdef __cplusplus
 extern "C" {
@@ -231,8 +231,8 @@ int mk_attention_mfma(const void* q, int q_stride, void* out, int out_stride,
 // wavefronts may have added four parts up already).  mk_attention_out then merges them and
 // multiplies by the output matrix w_o [N, n_q d] in one kernel, for steps of one token per
 // sequence (tile = token, M of them): out[slice, M, N] are float32 partial sums over slices of
-// heads_per_slice query heads each (mk_attention_out_heads_per_slice: how many, 0 where the
-// sizes are not taken; mk_attention_out_max_parts: the most partial results per (tile, kv head)
+// heads_per_slice query heads each (mk_attention_out_heads_per_slice: how many, for slices
+// stored or, with `atomic`, added into the fixed-point stream; 0 where the sizes are not taken; mk_attention_out_max_parts: the most partial results per (tile, kv head)
 // it takes), to be added up by whoever consumes the projection; or, with `out` null, the
 // result is added into the fixed-point residual stream fixed_out [M, N] (see mk_embed_fixed).
 // wide: 128 rows of w_o per workgroup instead of 64.
@@ -243,7 +243,7 @@ int mk_attention_mfma_parts(const void* q, int q_stride, const void* k_cache, co
                             int table_stride, int page_size, int n_q, int n_kv, int d, float scale,
                             int window, int rows_per_tile, int num_splits, int split_blocks,
                             float* part_o, float* part_ml, hipStream_t stream);
-int mk_attention_out_heads_per_slice(int n_q, int n_kv, int d, int M, int N);
+int mk_attention_out_heads_per_slice(int n_q, int n_kv, int d, int M, int N, int atomic);
 int mk_attention_out_max_parts(int M, int heads_per_slice);
 int mk_attention_out(const float* part_o, const float* part_ml, int parts, const void* w_o,
                      float* out, long long* fixed_out, int M, int N, int n_q, int n_kv, int d,

@@ -41,9 +41,25 @@ int run_embed(const void* params, mk_op_context* ctx) {
   return guarded(ctx, [&] {
     const EmbedParams& p = *static_cast<const EmbedParams*>(params);
     Launch l(ctx);
+    if (ctx->stream_fixed) {
+      embed_fixed(l, ctx->step->token_ids, p.table, p.table_dtype, ctx->h_fixed,
+                  ctx->step->num_tokens, ctx->hidden, p.vocab, p.scale);
+      return;
+    }
     embed(l, ctx->step->token_ids, p.table, p.table_dtype, ctx->h, ctx->step->num_tokens,
           ctx->hidden, p.vocab, p.scale);
   });
+}
+
+// The x an operation reads in a step in fixed point: a norm left for it to fold in (x is
+// null then), or an x that exists.
+const NormFold* fold_of(const mk_op_context* ctx, NormFold& fold) {
+  if (!ctx->stream_fixed || ctx->x != nullptr || ctx->norm_weight == nullptr) return nullptr;
+  fold.h64 = ctx->h_fixed;
+  fold.weight = ctx->norm_weight;
+  fold.weight_dtype = ctx->norm_weight_dtype;
+  fold.eps = ctx->norm_eps;
+  return &fold;
 }
 
 int run_norm(const void* params, mk_op_context* ctx) {
@@ -52,6 +68,20 @@ int run_norm(const void* params, mk_op_context* ctx) {
     const mk_step_view& s = *ctx->step;
     Launch l(ctx);
     const int rows = p.select_rows ? s.num_rows : s.num_tokens;
+    if (ctx->stream_fixed) {
+      if (ctx->pending_count > 0) throw KernelError("partial sums beside a stream in fixed point");
+      ctx->out_x_rows = rows;
+      ctx->out_x_live = 1;
+      if (p.select_rows) {   // few rows for a head that reads an x that exists
+        ctx->out_x = rmsnorm_fixed(l, ctx->h_fixed, ctx->hidden, p.weight, p.weight_dtype, p.eps,
+                                   s.logit_rows, rows);
+      } else {               // left to the projection behind
+        ctx->out_norm_weight = p.weight;
+        ctx->out_norm_weight_dtype = p.weight_dtype;
+        ctx->out_norm_eps = p.eps;
+      }
+      return;
+    }
     ctx->out_x = rmsnorm(l, ctx->h, s.num_tokens, ctx->hidden, ctx->pending, ctx->pending_count,
                          p.weight, p.weight_dtype, p.eps, p.select_rows ? s.logit_rows : nullptr,
                          rows);
@@ -82,9 +112,11 @@ int run_attention(const void* params, mk_op_context* ctx) {
     if (ctx->x_rows != s.num_tokens) throw KernelError("attention reads an x of every token");
     Launch l(ctx);
     const StepArrays arrays = arrays_of(s, p.group);
-    const Queries q = qkv_project(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, arrays);
+    NormFold fold;
+    const Queries q = qkv_project(l, ctx->x, s.num_tokens, ctx->hidden, p.qkv, arrays, {},
+                                  fold_of(ctx, fold));
     attend_and_project(l, q, attend_args(p), arrays, s, p.w_o, p.b_o, p.b_o_dtype, ctx->hidden,
-                       ctx->h, ctx->out_pending, ctx->out_pending_count);
+                       ctx->h, ctx->out_pending, ctx->out_pending_count, {}, -1, ctx->h_fixed);
   });
 }
 
@@ -109,7 +141,12 @@ int run_gated_mlp(const void* params, mk_op_context* ctx) {
     const int m = ctx->step->num_tokens;
     if (ctx->x_rows != m) throw KernelError("the gated projection reads an x of every token");
     Launch l(ctx);
-    const void* act = gated(l, ctx->x, m, ctx->hidden, p.w_gate_up, p.inter);
+    NormFold fold;
+    const void* act = gated(l, ctx->x, m, ctx->hidden, p.w_gate_up, p.inter, -2, fold_of(ctx, fold));
+    if (ctx->stream_fixed) {
+      project_into_fixed(l, act, m, p.w_down, ctx->hidden, p.inter, nullptr, kF32, ctx->h_fixed);
+      return;
+    }
     project_into_stream(l, act, m, p.w_down, ctx->hidden, p.inter, nullptr, kF32, ctx->h,
                         ctx->out_pending, ctx->out_pending_count);
   });
@@ -133,11 +170,12 @@ int run_head(const void* params, mk_op_context* ctx) {
 
 void register_builtin_ops() {
   OpRegistry& r = OpRegistry::instance();
-  r.add(OpKind{"embed", &run_embed, nullptr, 0});
-  r.add(OpKind{"norm", &run_norm, nullptr, MK_OP_FOLDS_PENDING});
-  r.add(OpKind{"attention", &run_attention, &tiles_attention, MK_OP_READS_X});
-  r.add(OpKind{"gated_mlp", &run_gated_mlp, nullptr, MK_OP_READS_X});
-  r.add(OpKind{"head", &run_head, nullptr, MK_OP_READS_X});
+  r.add(OpKind{"embed", &run_embed, nullptr, MK_OP_FIXED_STREAM});
+  r.add(OpKind{"norm", &run_norm, nullptr, MK_OP_FOLDS_PENDING | MK_OP_FIXED_STREAM});
+  r.add(OpKind{"attention", &run_attention, &tiles_attention, MK_OP_READS_X | MK_OP_FIXED_STREAM});
+  r.add(OpKind{"gated_mlp", &run_gated_mlp, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
+  r.add(OpKind{"head", &run_head, nullptr, MK_OP_READS_X | MK_OP_FIXED_STREAM});
+  r.fixed_stream_tokens = &fixed_stream_tokens;
 }
 
 }  // namespace mercury

@@ -84,6 +84,22 @@ bool qkv_fusable(int x_dtype, int w_dtype, int m, int k, int head_dim, int rotar
          page_size > 0 && (page_size & (page_size - 1)) == 0;
 }
 
+// Measured on the 0.5B shapes (896 wide), a layer's kernels in replayed graphs: q/k/v with the
+// norm folded in 6.0 / 6.5 us at 1 / 8 tokens against 8.0 / 8.6 as norm and projection; gated
+// projection with the norm folded in plus a down projection adding with atomics 13.0 / 15.0
+// against 15.8 / 16.5; at 16 tokens every workgroup's copy of the rows (8 bytes a value)
+// costs more than the norm kernel did (20.6 against 16.8).
+constexpr int kFixedStreamMaxTokens = 8;
+
+bool folds_norm(int dtype, int m, int k) {
+  if (dtype != kBF16 || m < 1 || k % 8 != 0 || !kernels().has_mfma()) return false;
+  return k <= kernels().mk_skinny_normed_max_k(m);
+}
+
+int fixed_stream_tokens(int dtype, int hidden) {
+  return folds_norm(dtype, kFixedStreamMaxTokens, hidden) ? kFixedStreamMaxTokens : 0;
+}
+
 QkvKind choose_qkv(int x_dtype, int w_dtype, int m, int width, int k, int head_dim,
                    int rotary_dim, int page_size, bool half_layout) {
   const bool half = half_layout || rotary_dim == 0;

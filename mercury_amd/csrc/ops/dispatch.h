@@ -49,6 +49,13 @@ QkvKind choose_qkv(int x_dtype, int w_dtype, int m, int width, int k, int head_d
 bool qkv_fusable(int x_dtype, int w_dtype, int m, int k, int head_dim, int rotary_dim,
                  int page_size, bool half_layout);
 
+// Up to how many tokens a step keeps its residual stream in fixed point (64-bit integers that
+// projections add into with atomics, the norms folded into the projections behind them): a
+// model of bfloat16 whose width the norm-folding projections take; 0 for never.
+int fixed_stream_tokens(int dtype, int hidden);
+// Whether the norm-folding projections take m rows of width k.
+bool folds_norm(int dtype, int m, int k);
+
 // ---- attention
 
 struct AttentionPlan {

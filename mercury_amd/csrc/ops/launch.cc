@@ -24,6 +24,41 @@ void* rmsnorm(Launch& l, float* h, int tokens, int hidden, const float* pending,
   return out;
 }
 
+void embed_fixed(Launch& l, const int* ids, const void* table, int table_dtype, long long* out,
+                 int tokens, int hidden, int vocab, float scale) {
+  if (l.dry() || tokens == 0) return;
+  check_core(need_core().mk_embed_fixed(ids, table, table_dtype, out, tokens, hidden, vocab, scale,
+                                        l.stream()), "embed");
+}
+
+void* rmsnorm_fixed(Launch& l, const long long* h64, int hidden, const void* weight,
+                    int weight_dtype, float eps, const int* rows, int out_rows) {
+  void* out = l.alloc((size_t)out_rows * hidden * l.elem());
+  if (l.dry() || out_rows == 0) return out;
+  check_core(need_core().mk_rmsnorm_fixed(h64, weight, weight_dtype, eps, rows, out, l.dtype(),
+                                          out_rows, hidden, l.stream()), "rmsnorm");
+  return out;
+}
+
+void project_into_fixed(Launch& l, const void* x, int m, const void* w, int n, int k,
+                        const void* bias, int bias_dtype, long long* h64) {
+  if (m == 0) return;
+  const int bd = bias ? bias_dtype : kF32;
+  if (mfma_eligible(l.dtype(), l.dtype(), m, k) && m <= 16) {
+    if (l.dry()) return;
+    const KernelTable& t = need_mfma();
+    check_mfma(t.mk_linear_skinny_fixed(x, w, bias, bd, h64, m, n, k,
+                                        t.mk_linear_skinny_slices(m, n, k), l.stream()),
+               "project_into_fixed");
+    return;
+  }
+  // whatever kernel takes the product, into a buffer, and that into the stream
+  float* y = (float*)linear(l, x, m, w, n, k, bias, bias_dtype, nullptr, kF32, false);
+  if (l.dry()) return;
+  check_core(need_core().mk_fixed_add(h64, y, 1, (long long)m * n, (long long)m * n, l.stream()),
+             "project_into_fixed");
+}
+
 void* silu_mul(Launch& l, const void* gate_up, int tokens, int inter, void* out) {
   if (!out) out = l.alloc((size_t)tokens * inter * l.elem());
   if (l.dry() || tokens == 0) return out;
@@ -130,7 +165,7 @@ void* qkv_finish(Launch& l, const float* parts, int slices, int m, const QkvArgs
 }
 
 Queries qkv_project(Launch& l, const void* x, int m, int k, const QkvArgs& a, const StepArrays& s,
-                    QkvForce force) {
+                    QkvForce force, const NormFold* fold) {
   const int d = a.head_dim;
   const int width = qkv_width(a);
   const int page_size = a.writes ? a.page_size : 1;
@@ -144,13 +179,22 @@ Queries qkv_project(Launch& l, const void* x, int m, int k, const QkvArgs& a, co
       !qkv_fusable(l.dtype(), l.dtype(), m, k, d, p.rotary_dim, page_size, half)) {
     throw KernelError("qkv_project: these operands cannot take the fused kernel");
   }
+  const bool folded = fold && kind == QkvKind::SKINNY && m <= 16 && folds_norm(l.dtype(), m, k);
+  if (fold && !folded) {
+    x = rmsnorm_fixed(l, fold->h64, k, fold->weight, fold->weight_dtype, fold->eps, nullptr, m);
+  }
   if (kind == QkvKind::SKINNY || kind == QkvKind::TILED) {
     void* q = l.alloc((size_t)m * a.n_q * d * 2);
     if (!l.dry() && m > 0) {
       const KernelTable& t = need_mfma();
       void* kc = a.writes ? a.k_cache : nullptr;
       void* vc = a.writes ? a.v_cache : nullptr;
-      const int code = kind == QkvKind::SKINNY
+      const int code = folded
+          ? t.mk_qkv_skinny_normed(fold->h64, fold->weight, fold->weight_dtype, fold->eps, a.w,
+                                   a.bias, bd, q, p.cos, p.sin, p.table_positions, s.positions,
+                                   s.token_seq, s.table, s.table_stride, kc, vc, page_size, a.n_q,
+                                   kv_heads(a), d, p.rotary_dim > 0, m, k, l.stream())
+          : kind == QkvKind::SKINNY
           ? t.mk_qkv_skinny(x, a.w, a.bias, bd, q, p.cos, p.sin, p.table_positions, s.positions,
                             s.token_seq, s.table, s.table_stride, kc, vc, page_size, a.n_q,
                             kv_heads(a), d, p.rotary_dim > 0, m, k, l.stream())
@@ -239,18 +283,19 @@ constexpr int kFoldWideFromHidden = 2048;
 void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
                         const mk_step_view& step, const void* w_o, const void* b_o, int b_o_dtype,
                         int hidden, float* h, const float*& pending, int& pending_count,
-                        AttendForce force, int fold) {
+                        AttendForce force, int fold, long long* h_fixed) {
   const int m = step.num_tokens, d = a.head_dim;
   pending = nullptr;
   pending_count = 0;
   const AttentionPlan plan = plan_for(l.dtype(), a, step, force);
   int heads_per_slice = 0, written = 0;
   bool wide = false;
+  const bool fixed = h_fixed != nullptr || (l.dry() && l.ctx->stream_fixed);
   if (fold != 0 && plan.mfma && plan.splits > 1 && !plan.staged && plan.rows == 16 &&
       step.max_q_len == 1 && plan.num_tiles == m && !b_o && a.n_q / a.n_kv <= 16) {
     const KernelTable& t = need_mfma();
     written = t.mk_attention_mfma_parts_written(plan.rows, plan.splits, d);
-    heads_per_slice = t.mk_attention_out_heads_per_slice(a.n_q, a.n_kv, d, m, hidden);
+    heads_per_slice = t.mk_attention_out_heads_per_slice(a.n_q, a.n_kv, d, m, hidden, fixed ? 1 : 0);
     wide = hidden >= kFoldWideFromHidden;
     if (heads_per_slice &&
         (written < 2 || written > t.mk_attention_out_max_parts(m, heads_per_slice))) {
@@ -265,17 +310,24 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
   if (!heads_per_slice) {
     if (fold > 0) throw KernelError("attention: these sizes do not take the folded merge");
     const void* attended = attend(l, q, a, s, step, force);
-    project_into_stream(l, attended, m, w_o, hidden, a.n_q * d, b_o, b_o_dtype, h, pending,
-                        pending_count);
+    if (fixed) {
+      project_into_fixed(l, attended, m, w_o, hidden, a.n_q * d, b_o, b_o_dtype, h_fixed);
+    } else {
+      project_into_stream(l, attended, m, w_o, hidden, a.n_q * d, b_o, b_o_dtype, h, pending,
+                          pending_count);
+    }
     return;
   }
   const size_t rows = (size_t)plan.num_tiles * a.n_kv * plan.splits * plan.rows;
   float* part_o = (float*)l.alloc(rows * d * 4);
   float* part_ml = (float*)l.alloc(rows * 2 * 4);
   const int slices = a.n_q / heads_per_slice;
-  float* out = (float*)l.alloc((size_t)slices * m * hidden * 4);
-  pending = out;
-  pending_count = slices;
+  float* out = nullptr;
+  if (!fixed) {
+    out = (float*)l.alloc((size_t)slices * m * hidden * 4);
+    pending = out;
+    pending_count = slices;
+  }
   if (l.dry() || m == 0) return;
   const KernelTable& t = need_mfma();
   const mk_tile_list& tiles = tiles_for(step, a.n_q / a.n_kv, plan.tile_rows);
@@ -285,16 +337,27 @@ void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const 
                                        a.page_size, a.n_q, a.n_kv, d, a.scale, a.window, plan.rows,
                                        plan.splits, plan.split_blocks, part_o, part_ml, l.stream()),
              "attention");
-  check_mfma(t.mk_attention_out(part_o, part_ml, written, w_o, out, nullptr, m, hidden, a.n_q, a.n_kv, d,
+  check_mfma(t.mk_attention_out(part_o, part_ml, written, w_o, out, h_fixed, m, hidden, a.n_q, a.n_kv, d,
                                 heads_per_slice, wide ? 1 : 0, l.stream()), "attention_out");
 }
 
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
-            int tile_config) {
-  if (fuses_gating(l.dtype(), l.dtype(), m, k, 2 * inter)) {
+            int tile_config, const NormFold* fold) {
+  const bool fuses = fuses_gating(l.dtype(), l.dtype(), m, k, 2 * inter);
+  const bool folded = fold && fuses && tile_config == -2 && m <= 16 && folds_norm(l.dtype(), m, k);
+  if (fold && !folded) {
+    x = rmsnorm_fixed(l, fold->h64, k, fold->weight, fold->weight_dtype, fold->eps, nullptr, m);
+  }
+  if (fuses) {
     void* act = l.alloc((size_t)m * inter * 2);
     if (l.dry() || m == 0) return act;
     const KernelTable& t = need_mfma();
+    if (folded) {
+      check_mfma(t.mk_gated_skinny_normed(fold->h64, fold->weight, fold->weight_dtype, fold->eps,
+                                          w_gate_up, act, m, inter, k, l.stream()),
+                 "gated_projection");
+      return act;
+    }
     const bool skinny = gated_is_skinny(m) && tile_config == -2;
     check_mfma(skinny ? t.mk_gated_skinny(x, w_gate_up, act, m, inter, k, l.stream())
                       : t.mk_gated_tiled(x, w_gate_up, act, m, inter, k,

@@ -34,6 +34,22 @@ void* rmsnorm(Launch& l, float* h, int tokens, int hidden, const float* pending,
               const void* weight, int weight_dtype, float eps, const int* rows, int out_rows,
               void* out = nullptr);
 
+// The residual stream of a step of few tokens in fixed point (op_abi.h): its start, the norm
+// of rows of it, and a norm left for the projection behind it to fold in.
+void embed_fixed(Launch& l, const int* ids, const void* table, int table_dtype, long long* out,
+                 int tokens, int hidden, int vocab, float scale);
+void* rmsnorm_fixed(Launch& l, const long long* h64, int hidden, const void* weight,
+                    int weight_dtype, float eps, const int* rows, int out_rows);
+struct NormFold {
+  const long long* h64 = nullptr;
+  const void* weight = nullptr;
+  int weight_dtype = 0;
+  float eps = 0.f;
+};
+// h64 += x W^T (+ bias).
+void project_into_fixed(Launch& l, const void* x, int m, const void* w, int n, int k,
+                        const void* bias, int bias_dtype, long long* h64);
+
 void* silu_mul(Launch& l, const void* gate_up, int tokens, int inter, void* out = nullptr);
 
 // logits <- cap * tanh(logits / cap), in place.
@@ -101,8 +117,10 @@ struct QkvForce {
 
 // q, k, v = x W^T + bias, q and k rotated, k and v written to the paged cache; the rotated
 // queries come back (rows of `stride` elements).
+// With `fold`, x is rmsnorm(fold->h64) * fold->weight and `x` is ignored: the projection makes
+// it itself where its kernel can, else the norm runs first.
 Queries qkv_project(Launch& l, const void* x, int m, int k, const QkvArgs& a, const StepArrays& s,
-                    QkvForce force = {});
+                    QkvForce force = {}, const NormFold* fold = nullptr);
 
 // Rotation and cache write of an already projected qkv [m, row_stride] (q rotated in place).
 void rope_kv_write(Launch& l, void* qkv, int row_stride, int m, const QkvArgs& a,
@@ -142,15 +160,17 @@ void* attend(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays&
 // project_into_stream does it (pending / pending_count: partial sums left for the next norm).
 // Decoding with the keys split over workgroups takes two kernels instead of three: the
 // attention leaves its partial results, and one kernel merges them and multiplies by w_o
-// (`fold`: -1 where the sizes allow and it pays, 0 never, 1 wherever the sizes allow).
+// (`fold`: -1 where the sizes allow and it pays, 0 never, 1 wherever the sizes allow).  With
+// h_fixed the residual stream is that one (h is ignored) and nothing is left pending.
 void attend_and_project(Launch& l, const Queries& q, const AttendArgs& a, const StepArrays& s,
                         const mk_step_view& step, const void* w_o, const void* b_o, int b_o_dtype,
                         int hidden, float* h, const float*& pending, int& pending_count,
-                        AttendForce force = {}, int fold = -1);
+                        AttendForce force = {}, int fold = -1, long long* h_fixed = nullptr);
 
 // act = silu(x Wg^T) * (x Wu^T) for w = [Wg | Wu] stacked [2 inter, k].  tile_config: -2 by the
 // sizes, else the tiled kernel with that configuration (-1: its own choice).
+// `fold` as for qkv_project.
 void* gated(Launch& l, const void* x, int m, int k, const void* w_gate_up, int inter,
-            int tile_config = -2);
+            int tile_config = -2, const NormFold* fold = nullptr);
 
 }  // namespace mercury

@@ -58,7 +58,7 @@ class OneOp:
         rows = step.num_logit_rows
         x_rows = 0 if x is None else x.shape[0]
         need = program.workspace_bytes_for(counts, rows, step.max_kv_len,
-                                           max(1, len(step.block_tables)), x_rows)
+                                           max(1, len(step.block_tables)), x_rows, own_stream=True)
         scratch = torch.empty(max(need, 256), dtype=torch.uint8, device=h.device)
         logits = None
         if want_logits:

@@ -45,7 +45,13 @@ class OpContext(ctypes.Structure):
                 ("out_x", c_void_p), ("out_x_rows", c_int), ("out_x_live", c_int),
                 ("out_pending", c_void_p), ("out_pending_count", c_int),
                 ("out_logits_ready", c_int),
-                ("arena", c_void_p), ("alloc", ALLOC), ("error", c_char * 512)]
+                ("arena", c_void_p), ("alloc", ALLOC), ("error", c_char * 512),
+                # a step of few tokens with its residual stream in fixed point (h is then
+                # null), which only kinds flagged FIXED_STREAM ever see
+                ("stream_fixed", c_int), ("h_fixed", c_void_p),
+                ("norm_weight", c_void_p), ("norm_weight_dtype", c_int), ("norm_eps", c_float),
+                ("out_norm_weight", c_void_p), ("out_norm_weight_dtype", c_int),
+                ("out_norm_eps", c_float)]
 
     def allocate(self, nbytes: int) -> int:
         """Device memory from the operation's arena (0 in a dry walk)."""
@@ -56,6 +62,7 @@ RUN = ctypes.CFUNCTYPE(c_int, c_void_p, POINTER(OpContext))
 
 READS_X = core.OP_READS_X
 FOLDS_PENDING = core.OP_FOLDS_PENDING
+FIXED_STREAM = core.OP_FIXED_STREAM
 
 _kept: dict = {}      # name -> the C function object; the registry holds its bare address
 
@@ -80,5 +87,5 @@ def register_python_op(name: str, run, flags: int = 0) -> None:
     core.register_op(name, ctypes.cast(function, c_void_p).value, 0, flags)
 
 
-__all__ = ["ALLOC", "FOLDS_PENDING", "OpContext", "READS_X", "RUN", "StepView", "TileList",
+__all__ = ["ALLOC", "FIXED_STREAM", "FOLDS_PENDING", "OpContext", "READS_X", "RUN", "StepView", "TileList",
            "c_float", "register_python_op"]

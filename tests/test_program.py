@@ -149,3 +149,80 @@ def test_an_error_inside_an_operation_names_it():
     program.append("test_failing", b"")
     with pytest.raises(RuntimeError, match=r"operation 1 \('test_failing'\): ValueError: made to fail"):
         program.workspace_bytes_for([3], 1, 3)
+
+
+# ---- steps of few tokens with the residual stream in fixed point
+
+SEEN: list = []
+
+
+def watching(params, ctx):
+    """A kind that records what the walk tells it about the stream, and may leave a norm to
+    the operation behind it."""
+    p = Sizes.from_address(params)
+    SEEN.append((ctx.stream_fixed, bool(ctx.x_live), ctx.norm_weight or 0, round(ctx.norm_eps, 6)))
+    at = ctx.allocate(p.bytes_out)
+    if p.gives_x:
+        ctx.out_x_rows, ctx.out_x_live = ctx.step.contents.num_tokens, 1
+        if ctx.stream_fixed or p.gives_x == 2:   # a norm left undone: no x, but its weight and eps
+            ctx.out_norm_weight, ctx.out_norm_weight_dtype, ctx.out_norm_eps = 4096, 1, 0.125
+        else:
+            ctx.out_x = at
+
+
+op_abi.register_python_op("test_fixed_any", watching, op_abi.FIXED_STREAM)
+op_abi.register_python_op("test_fixed_reader", watching, op_abi.READS_X | op_abi.FIXED_STREAM)
+
+
+@pytest.fixture
+def fixed_up_to_four():
+    before = core.set_fixed_stream_limit(4)
+    yield
+    core.set_fixed_stream_limit(before)
+
+
+def test_few_tokens_walk_in_fixed_point_when_every_operation_can(fixed_up_to_four):
+    program = core.Program(F32, 64, 100)
+    program.append("test_fixed_any", op(256, gives_x=1))
+    program.append("test_fixed_reader", op(256))
+    assert program.fixed_stream(4) and not program.fixed_stream(5) and not program.fixed_stream(0)
+    rows = 1
+    logits = (rows * 100 * 4 + 255) // 256 * 256
+    # 8 bytes a value of the stream instead of 4
+    assert program.workspace_bytes_for([3], rows, 9) == 3 * 64 * 8 + logits + 2 * 256
+    assert program.workspace_bytes_for([5], rows, 9) == 5 * 64 * 4 + logits + 2 * 256
+    # a run on a stream of the caller's own is never in fixed point
+    assert program.workspace_bytes_for([3], rows, 9, own_stream=True) == 2 * 256
+    SEEN.clear()
+    program.workspace_bytes_for([3], rows, 9)
+    assert SEEN == [(1, False, 0, 0.0), (1, True, 4096, 0.125)]     # the norm reaches the reader
+    mixed = core.Program(F32, 64, 100)
+    mixed.append("test_fixed_any", op(256))
+    mixed.append("test_producer", op(256))
+    assert not mixed.fixed_stream(2)              # one operation that cannot: the float stream
+    SEEN.clear()
+    mixed.workspace_bytes_for([2], rows, 9)
+    assert SEEN == [(0, False, 0, 0.0)]
+
+
+def test_a_norm_left_undone_outside_fixed_point_is_refused(fixed_up_to_four):
+    program = core.Program(F32, 64, 100)
+    program.append("test_fixed_any", op(256, gives_x=2))      # leaves it whatever the stream is
+    program.append("test_fixed_reader", op(256))
+    assert program.workspace_bytes_for([3], 1, 9) > 0
+    with pytest.raises(RuntimeError, match="left a norm undone outside a step in fixed point"):
+        program.workspace_bytes_for([7], 1, 9)
+
+
+def test_the_limit_switches_fixed_point_off():
+    before = core.set_fixed_stream_limit(0)
+    try:
+        program = core.Program(1, 64, 100)
+        program.append("test_fixed_any", op(256))
+        assert not program.fixed_stream(1)
+    finally:
+        core.set_fixed_stream_limit(before)
+    # the kernels' own rule again: float32 models never
+    program = core.Program(F32, 64, 100)
+    program.append("test_fixed_any", op(256))
+    assert not program.fixed_stream(1)
