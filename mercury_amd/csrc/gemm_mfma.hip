@@ -200,10 +200,11 @@ __device__ __forceinline__ void qkv_store(const QkvTarget& p, const QkvPlace& pl
 // current step's products; the wavefronts' results are added through LDS in wave order.
 // Product j of a step takes k = step*128 + j*32 + g4*8 .. + 8 from a lane, so that one load
 // instruction reads 64 contiguous bytes of each of its 16 rows.
-template <int MT, int NT, int EPI, int WAVES, bool NORMED = false>
+template <int MT, int NT, int EPI, int WAVES, int NORMED = 0>
 __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   static_assert((EPI != SK_GATED && EPI != SK_QKV) || NT == 2, "paired tiles");
-  static_assert(!NORMED || MT == 1, "rows made in LDS: at most 16");
+  static_assert(NORMED == 0 || MT == 1, "rows made in LDS: at most 16");
+  static_assert(NORMED == 0 || NORMED == 8 || NORMED == 16, "a lane's pairs of a row: 8 or 16");
   __shared__ float red[WAVES - 1][NT * MT * 4][64];
   const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 15, g4 = lane >> 4;
   const int M = p.M, N = p.N, K = p.K;
@@ -265,9 +266,9 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   // and worked on while the first weights of W are still on their way from HBM.  (Loads at
   // clamped places and values chosen afterwards: a load under a condition is a branch, and
   // the compiler waits for it before the next.)
-  constexpr int HOLD = 8;
-  float g[NORMED ? HOLD : 1][2];
-  longlong2 v[NORMED ? HOLD : 1];
+  constexpr int HOLD = NORMED ? NORMED : 1;   // rows of up to 128 * HOLD values
+  float g[HOLD][2];
+  longlong2 v[HOLD];
   if constexpr (NORMED) {
     if (wave < M) {
       if (p.norm_bf16) {
@@ -350,7 +351,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   }
 
   // NORMED: wavefront w makes rows w, w + WAVES, ...: a lane holds its two values of every
-  // 128 of the row (at most 1,024 wide: eight loads, all in flight at once; the norm's
+  // 128 of the row (at most 2,048 wide: eight or sixteen loads, all in flight at once; the norm's
   // weights at the same places are shared by every row of the wavefront), adds up their
   // squares, and leaves the normalised, weighted, rounded values in LDS.  The lane layout is
   // the same whichever wavefront takes the row, so a row's x does not depend on the batch.
@@ -585,7 +586,7 @@ extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
   return whole < 0.9 * split;
 }
 
-template <int NT, int EPI, bool NORMED = false, int WAVES = 0>
+template <int NT, int EPI, int NORMED = 0, int WAVES = 0>
 static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream, size_t lds = 0) {
   // 8 wavefronts where the grid is small; with 3 or 4 tiles of x rows they would not fit
   // the register file.  More than 16 rows of x only for the q/k/v projection: the others
@@ -688,7 +689,7 @@ extern "C" int mk_gated_skinny(const void* x, const void* w, void* act, int M, i
 extern "C" int mk_skinny_normed_max_k(int M) {
   if (M < 1 || M > 16) return 0;
   const int fits = ((48 * 1024) / (2 * M) - 8) / 8 * 8;
-  return fits < 1024 ? fits : 1024;   // a lane holds its share of a row in registers
+  return fits < 2048 ? fits : 2048;   // a lane holds its share of a row in registers
 }
 
 static int set_normed(SkinnyArgs& a, const long long* h64, const void* norm_w, int norm_dtype,
@@ -719,8 +720,14 @@ extern "C" int mk_gated_skinny_normed(const long long* h64, const void* norm_w, 
   MK_REQUIRE(w && act, "gated projection: null argument");
   SkinnyArgs a = skinny_args(nullptr, w, act, M, inter, K, (K + 127) / 128);
   if (set_normed(a, h64, norm_w, norm_dtype, eps)) return 1;
-  if (M <= 4) launch_skinny<2, SK_GATED, true, 4>(a, dim3((inter + 15) / 16, 1), stream, normed_lds(a));
-  else launch_skinny<2, SK_GATED, true, 8>(a, dim3((inter + 15) / 16, 1), stream, normed_lds(a));
+  const dim3 grid((inter + 15) / 16, 1);
+  if (K <= 1024) {
+    if (M <= 4) launch_skinny<2, SK_GATED, 8, 4>(a, grid, stream, normed_lds(a));
+    else launch_skinny<2, SK_GATED, 8, 8>(a, grid, stream, normed_lds(a));
+  } else {
+    if (M <= 4) launch_skinny<2, SK_GATED, 16, 4>(a, grid, stream, normed_lds(a));
+    else launch_skinny<2, SK_GATED, 16, 8>(a, grid, stream, normed_lds(a));
+  }
   MK_LAUNCH_CHECK("gated_skinny_normed");
   return 0;
 }
@@ -767,7 +774,8 @@ static int qkv_skinny_any(const void* x, const long long* h64, const void* norm_
   const dim3 grid((n_q + 2 * n_kv) * (d / 32), 1);
   if (h64) {
     if (set_normed(a, h64, norm_w, norm_dtype, eps)) return 1;
-    launch_skinny<2, SK_QKV, true>(a, grid, stream, normed_lds(a));
+    if (K <= 1024) launch_skinny<2, SK_QKV, 8>(a, grid, stream, normed_lds(a));
+    else launch_skinny<2, SK_QKV, 16>(a, grid, stream, normed_lds(a));
   } else {
     MK_REQUIRE(x, "qkv projection: null argument");
     launch_skinny<2, SK_QKV>(a, grid, stream);
