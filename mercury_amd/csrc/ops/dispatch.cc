@@ -88,8 +88,13 @@ bool qkv_fusable(int x_dtype, int w_dtype, int m, int k, int head_dim, int rotar
 // norm folded in 6.0 / 6.5 us at 1 / 8 tokens against 8.0 / 8.6 as norm and projection; gated
 // projection with the norm folded in plus a down projection adding with atomics 13.0 / 15.0
 // against 15.8 / 16.5; at 16 tokens every workgroup's copy of the rows (8 bytes a value)
-// costs more than the norm kernel did (20.6 against 16.8).
+// costs more than the norm kernel did (20.6 against 16.8).  Wider rows cost every workgroup
+// more: at 1,536 and 2,048 (the 1.5B and 3B shapes) q/k/v still saves 1.6-1.9 us a layer up
+// to 8 tokens, but the gated projection and its down projection only break even up to 4
+// (27.8 against 27.8, 36.6 against 38.1 us) and lose at 8 (31.0 against 28.4, 39.6 against
+// 38.7).
 constexpr int kFixedStreamMaxTokens = 8;
+constexpr int kFixedStreamNarrow = 1024, kFixedStreamMaxTokensWide = 4;
 
 bool folds_norm(int dtype, int m, int k) {
   if (dtype != kBF16 || m < 1 || k % 8 != 0 || !kernels().has_mfma()) return false;
@@ -97,7 +102,8 @@ bool folds_norm(int dtype, int m, int k) {
 }
 
 int fixed_stream_tokens(int dtype, int hidden) {
-  return folds_norm(dtype, kFixedStreamMaxTokens, hidden) ? kFixedStreamMaxTokens : 0;
+  const int most = hidden <= kFixedStreamNarrow ? kFixedStreamMaxTokens : kFixedStreamMaxTokensWide;
+  return folds_norm(dtype, most, hidden) ? most : 0;
 }
 
 QkvKind choose_qkv(int x_dtype, int w_dtype, int m, int width, int k, int head_dim,

@@ -118,7 +118,8 @@ def test_a_projection_adds_into_the_fixed_stream(m, n, k, bias_dtype):
 
 
 @pytest.mark.parametrize("m,k,inter", [(1, 896, 4864), (8, 896, 4864), (3, 168, 410), (16, 64, 176),
-                                       (4, 1024, 96), (13, 1000, 24)])
+                                       (4, 1024, 96), (13, 1000, 24), (2, 1536, 200), (4, 2048, 48),
+                                       (7, 1032, 64), (11, 2000, 32)])
 def test_the_gated_projection_makes_its_own_normalised_rows(m, k, inter):
     lib, core, mfma = libs()
     h = rnd(m, k, seed=21) * torch.logspace(-3, 2, k)
@@ -151,7 +152,8 @@ def test_the_gated_projection_makes_its_own_normalised_rows(m, k, inter):
 
 @pytest.mark.parametrize("n_q,n_kv,d,page,k,m", [(14, 2, 64, 16, 896, 8), (6, 1, 32, 8, 168, 1),
                                                  (4, 4, 128, 32, 264, 16), (3, 1, 96, 16, 72, 5),
-                                                 (2, 2, 64, 16, 1024, 3)])
+                                                 (2, 2, 64, 16, 1024, 3), (2, 1, 128, 16, 1536, 4),
+                                                 (1, 1, 64, 16, 2048, 9), (3, 1, 32, 8, 1096, 2)])
 def test_the_qkv_projection_makes_its_own_normalised_rows(n_q, n_kv, d, page, k, m):
     """Against the same kernel on rows the norm kernel made: the same wavefronts take the same
     k-steps, so wherever the rows agree the results are the same bits; rotation, bias and the
@@ -193,14 +195,17 @@ def test_the_qkv_projection_makes_its_own_normalised_rows(n_q, n_kv, d, page, k,
 
 def test_rows_too_wide_or_too_many_are_refused():
     lib, core, mfma = libs()
-    assert mfma.mk_skinny_normed_max_k(8) == 1024 and mfma.mk_skinny_normed_max_k(17) == 0
-    h64 = torch.zeros(16, 2048, dtype=torch.long, device=DEV)
-    g = torch.ones(2048, dtype=BF, device=DEV)
-    w = torch.zeros(64, 2048, dtype=BF, device=DEV)
+    # a lane holds at most 16 pairs of a row; 16 rows of LDS leave room for 1,528 values each
+    assert mfma.mk_skinny_normed_max_k(8) == 2048 and mfma.mk_skinny_normed_max_k(16) == 1528
+    assert mfma.mk_skinny_normed_max_k(17) == 0
+    h64 = torch.zeros(16, 2056, dtype=torch.long, device=DEV)
+    g = torch.ones(2056, dtype=BF, device=DEV)
+    w = torch.zeros(64, 2056, dtype=BF, device=DEV)
     act = torch.zeros(16, 32, dtype=BF, device=DEV)
-    with pytest.raises(lib.KernelLibraryError, match="more than its workgroups hold"):
-        lib.check(mfma, mfma.mk_gated_skinny_normed(h64.data_ptr(), g.data_ptr(), 1, 1e-6, w.data_ptr(),
-                                                    act.data_ptr(), 16, 32, 2048, stream()), "too wide")
+    for rows, width in ((16, 2048), (2, 2056)):
+        with pytest.raises(lib.KernelLibraryError, match="more than its workgroups hold"):
+            lib.check(mfma, mfma.mk_gated_skinny_normed(h64.data_ptr(), g.data_ptr(), 1, 1e-6, w.data_ptr(),
+                                                        act.data_ptr(), rows, 32, width, stream()), "too wide")
     with pytest.raises(lib.KernelLibraryError, match="more than its workgroups hold"):
         lib.check(mfma, mfma.mk_gated_skinny_normed(h64.data_ptr(), g.data_ptr(), 1, 1e-6, w.data_ptr(),
                                                     act.data_ptr(), 17, 32, 64, stream()), "too many")
@@ -255,6 +260,32 @@ def test_decoding_with_the_stream_in_fixed_point_and_without(name, page, limit):
     for k in keys:
         apart = float((got["fixed"][k] - got["float"][k]).abs().max())
         assert apart <= case.cost[k], (k, apart, case.cost[k])
+
+
+def test_a_model_1536_wide_decodes_in_fixed_point_up_to_four_tokens(limit):
+    """Rows of more than 1,024 values take the projections' instantiation of sixteen pairs a
+    lane, and the rule stops at four tokens there."""
+    from tests.test_gpu_replay_bench_sizes import folder_for, session
+
+    limit(-1)
+    folder = folder_for("S128", hidden_size=1536, num_attention_heads=12, intermediate_size=1288,
+                        vocab_size=1003)
+    weights, cfg = helpers.plain_model(folder)
+    tokens = helpers.random_tokens(cfg["vocab_size"], 90, seed=5)
+    want = plain.forward_logits(weights, cfg, tokens)
+    from tests.test_gpu_replay import bf16_cost
+
+    cost = bf16_cost(folder, cfg, tokens, want)
+    s = session(folder, "bfloat16", 256, 32)
+    assert s.runner.program.fixed_stream(4) and not s.runner.program.fixed_stream(5)
+    rows, done = [], 0
+    for size in (50, 1, 1, 4, 3, 1, 2, 5, 1, 4, 1, 8, 1, 1, 4, 3):
+        rows.append(s.step([entry("x", tokens[done:done + size])], []))
+        done += size
+    assert done == len(tokens)
+    check(torch.cat(rows), want, "bfloat16", "1536 wide", cost)
+    s.step([], ["x"])
+    assert s.manager.leaked_pages() == 0
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
