@@ -200,7 +200,7 @@ __device__ __forceinline__ void qkv_store(const QkvTarget& p, const QkvPlace& pl
 // current step's products; the wavefronts' results are added through LDS in wave order.
 // Product j of a step takes k = step*128 + j*32 + g4*8 .. + 8 from a lane, so that one load
 // instruction reads 64 contiguous bytes of each of its 16 rows.
-template <int MT, int NT, int EPI, int WAVES, int NORMED = 0>
+template <int MT, int NT, int EPI, int WAVES, int NORMED = 0, bool ONE_ROW = false>
 __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   static_assert((EPI != SK_GATED && EPI != SK_QKV) || NT == 2, "paired tiles");
   static_assert(NORMED == 0 || MT == 1, "rows made in LDS: at most 16");
@@ -233,7 +233,13 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
   const bf16_t* made = (const bf16_t*)skinny_rows;   // NORMED
   const int made_stride = K + 8, made_row = min(r, M - 1) * made_stride;
 
-  constexpr int DEPTH = MT == 1 ? 3 : (MT == 2 ? 2 : 1);
+  // Eight wavefronts over rows of at most 1,024 (NORMED 8) take one k-step each: no buffers
+  // for steps ahead, and with the registers they would take, two workgroups fit a compute
+  // unit, so that the gated projection's 304 workgroups run in one round instead of two.
+  // (ONE_ROW: at most one row a wavefront, M <= WAVES; the instantiation for more rows keeps
+  // the buffers.)
+  static_assert(!ONE_ROW || NORMED != 0, "rows made by the workgroup");
+  constexpr int DEPTH = (NORMED == 8 && WAVES == 8 && ONE_ROW) ? 1 : (MT == 1 ? 3 : (MT == 2 ? 2 : 1));
   Frag a[DEPTH][NT][4], b[DEPTH][MT][4];
   auto load_w = [&](int buf, int step) {
     const int kk = step * 128 + g4 * 8;
@@ -361,7 +367,7 @@ __global__ __launch_bounds__(64 * WAVES) void gemm_skinny_kernel(SkinnyArgs p) {
     for (int d = 1; d < DEPTH - 1; ++d)
       if (step + d * WAVES < step_end) load_w(d, step + d * WAVES);
     bf16_t* rows_out = (bf16_t*)skinny_rows;
-    for (int m = wave; m < M; m += WAVES) {
+    for (int m = wave; m < M; m += ONE_ROW ? M : WAVES) {
       if (m != wave) {
 #pragma unroll
         for (int i = 0; i < HOLD; ++i)
@@ -586,7 +592,7 @@ extern "C" int mk_linear_skinny_unsplit(int M, int N, int K) {
   return whole < 0.9 * split;
 }
 
-template <int NT, int EPI, int NORMED = 0, int WAVES = 0>
+template <int NT, int EPI, int NORMED = 0, int WAVES = 0, bool ONE_ROW = false>
 static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream, size_t lds = 0) {
   // 8 wavefronts where the grid is small; with 3 or 4 tiles of x rows they would not fit
   // the register file.  More than 16 rows of x only for the q/k/v projection: the others
@@ -594,7 +600,7 @@ static void launch_skinny(const SkinnyArgs& a, dim3 grid, hipStream_t stream, si
   constexpr int W = WAVES ? WAVES : ((EPI == SK_ACC || EPI == SK_QKV || NORMED) ? 8 : SK_WAVES);
   const int tiles = (a.M + 15) / 16;
   if (tiles == 1) {
-    gemm_skinny_kernel<1, NT, EPI, W, NORMED><<<grid, 64 * W, lds, stream>>>(a);
+    gemm_skinny_kernel<1, NT, EPI, W, NORMED, ONE_ROW><<<grid, 64 * W, lds, stream>>>(a);
   } else if constexpr (EPI == SK_QKV && !NORMED) {
     if (tiles == 2) gemm_skinny_kernel<2, NT, EPI, W><<<grid, 64 * W, 0, stream>>>(a);
     else if (tiles == 3) gemm_skinny_kernel<3, NT, EPI, SK_WAVES><<<grid, 64 * SK_WAVES, 0, stream>>>(a);
@@ -723,6 +729,7 @@ extern "C" int mk_gated_skinny_normed(const long long* h64, const void* norm_w, 
   const dim3 grid((inter + 15) / 16, 1);
   if (K <= 1024) {
     if (M <= 4) launch_skinny<2, SK_GATED, 8, 4>(a, grid, stream, normed_lds(a));
+    else if (M <= 8) launch_skinny<2, SK_GATED, 8, 8, true>(a, grid, stream, normed_lds(a));
     else launch_skinny<2, SK_GATED, 8, 8>(a, grid, stream, normed_lds(a));
   } else {
     if (M <= 4) launch_skinny<2, SK_GATED, 16, 4>(a, grid, stream, normed_lds(a));
@@ -774,7 +781,8 @@ static int qkv_skinny_any(const void* x, const long long* h64, const void* norm_
   const dim3 grid((n_q + 2 * n_kv) * (d / 32), 1);
   if (h64) {
     if (set_normed(a, h64, norm_w, norm_dtype, eps)) return 1;
-    if (K <= 1024) launch_skinny<2, SK_QKV, 8>(a, grid, stream, normed_lds(a));
+    if (K <= 1024 && M <= 8) launch_skinny<2, SK_QKV, 8, 8, true>(a, grid, stream, normed_lds(a));
+    else if (K <= 1024) launch_skinny<2, SK_QKV, 8>(a, grid, stream, normed_lds(a));
     else launch_skinny<2, SK_QKV, 16>(a, grid, stream, normed_lds(a));
   } else {
     MK_REQUIRE(x, "qkv projection: null argument");

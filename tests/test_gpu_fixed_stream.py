@@ -119,7 +119,7 @@ def test_a_projection_adds_into_the_fixed_stream(m, n, k, bias_dtype):
 
 @pytest.mark.parametrize("m,k,inter", [(1, 896, 4864), (8, 896, 4864), (3, 168, 410), (16, 64, 176),
                                        (4, 1024, 96), (13, 1000, 24), (2, 1536, 200), (4, 2048, 48),
-                                       (7, 1032, 64), (11, 2000, 32)])
+                                       (7, 1032, 64), (11, 2000, 32), (16, 256, 704), (12, 896, 64)])
 def test_the_gated_projection_makes_its_own_normalised_rows(m, k, inter):
     lib, core, mfma = libs()
     h = rnd(m, k, seed=21) * torch.logspace(-3, 2, k)
@@ -153,7 +153,8 @@ def test_the_gated_projection_makes_its_own_normalised_rows(m, k, inter):
 @pytest.mark.parametrize("n_q,n_kv,d,page,k,m", [(14, 2, 64, 16, 896, 8), (6, 1, 32, 8, 168, 1),
                                                  (4, 4, 128, 32, 264, 16), (3, 1, 96, 16, 72, 5),
                                                  (2, 2, 64, 16, 1024, 3), (2, 1, 128, 16, 1536, 4),
-                                                 (1, 1, 64, 16, 2048, 9), (3, 1, 32, 8, 1096, 2)])
+                                                 (1, 1, 64, 16, 2048, 9), (3, 1, 32, 8, 1096, 2), (8, 1, 32, 8, 256, 16),
+                                                 (14, 2, 64, 16, 896, 13)])
 def test_the_qkv_projection_makes_its_own_normalised_rows(n_q, n_kv, d, page, k, m):
     """Against the same kernel on rows the norm kernel made: the same wavefronts take the same
     k-steps, so wherever the rows agree the results are the same bits; rotation, bias and the
