@@ -454,7 +454,7 @@ def main(argv=None) -> int:
             "prefill_tokens": PREFILL_TOKENS, "parallelism": "single GPU",
         },
         "prefill": {"value": round(pre["tok_s"], 1), "tokens": PREFILL_TOKENS,
-                    "ms": round(pre["ms"], 3),
+                    "ms": round(pre["ms"], 4),
                     "frac": round(prefill_rate / PEAK_FLOPS[short], 5),
                     "measured_peak": peaks.get("gemm_flops"),
                     "frac_of_measured": (round(prefill_rate / peaks["gemm_flops"], 5)
